@@ -1,0 +1,249 @@
+// C ABI of libdsdpa.so (declared in include/dsdpa.h): argument checks, kernel
+// selection and launches. No allocation, no synchronisation, no torch types.
+#include "../../include/dsdpa.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+
+#include "dsdpa_common.h"
+#include "dsdpa_gather.h"
+
+using namespace dsdpa;
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+std::atomic<int> g_path{DSDPA_PATH_AUTO};
+
+// ------------------------------------------------------------------ small kernels
+__global__ void fill_zero_kernel(float4 *__restrict__ p, size_t n4)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += stride) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+// fp32 accumulators -> 16-bit storage, 8 elements per thread
+template <typename S>
+__global__ void cast_kernel(const float *__restrict__ src, void *__restrict__ dst, size_t n8)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n8; i += stride) {
+        float v[8];
+        const float4 *s4 = reinterpret_cast<const float4 *>(src) + 2 * i;
+        float4 a = s4[0], b = s4[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        store_chunk<S, 8>((char *)dst + i * 16, v);
+    }
+}
+
+int check_launch()
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return DSDPA_ERR_HIP;
+    }
+    return DSDPA_OK;
+}
+
+int make_dims(int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, Dims *dm)
+{
+    if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || P < 1) return DSDPA_ERR_BAD_SHAPE;
+    if (!(D == 16 || D == 32 || D == 64 || D == 128 || D == 256)) return DSDPA_ERR_HEAD_DIM;
+    const long long L = (long long)Himg * Wimg;
+    const long long slab = (long long)V * H * L * D;           // one batch item of k/v
+    const long long rows = (long long)B * V * H * L;
+    const long long N = (long long)V * P;
+    if (L > (1ll << 24) || slab > (1ll << 30) || rows > 0x7fffffffll - 1024 || N > (1ll << 24))
+        return DSDPA_ERR_TOO_LARGE;
+    dm->B = B; dm->V = V; dm->H = H; dm->Himg = Himg; dm->Wimg = Wimg;
+    dm->L = (int)L; dm->P = P; dm->N = (int)N; dm->rows = (int)rows; dm->sm_scale = sm_scale;
+    return DSDPA_OK;
+}
+
+// lanes per sample are D/DC; DC is chosen so that a lane moves 16 bytes per tap
+// (32 or 64 for the widest heads) and a sample never spans more than 16 lanes.
+template <typename S, int D> struct Chunk {
+    static constexpr int kMin = 16 / S::kBytes;
+    static constexpr int value = (D / kMin > 16) ? D / 16 : kMin;
+};
+
+template <typename S, int D>
+int launch_fwd_gather(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+                      const Dims &dm, hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
+    hipLaunchKernelGGL((fwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                       q, k, v, coords, out, lse, dm);
+    return check_launch();
+}
+
+template <typename S, int D>
+int launch_bwd_gather(const void *q, const void *k, const void *v, const float *coords, const void *out,
+                      const float *lse, const void *dout, void *dq, float *dk_acc, float *dv_acc,
+                      const Dims &dm, hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
+    hipLaunchKernelGGL((bwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                       q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm);
+    return check_launch();
+}
+
+template <typename S>
+int fwd_impl(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    if (!q || !k || !v || !coords || !out || !lse) return DSDPA_ERR_NULL_POINTER;
+    Dims dm;
+    int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
+    if (rc != DSDPA_OK) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    switch (D) {
+    case 16: return launch_fwd_gather<S, 16>(q, k, v, coords, out, lse, dm, st);
+    case 32: return launch_fwd_gather<S, 32>(q, k, v, coords, out, lse, dm, st);
+    case 64: return launch_fwd_gather<S, 64>(q, k, v, coords, out, lse, dm, st);
+    case 128: return launch_fwd_gather<S, 128>(q, k, v, coords, out, lse, dm, st);
+    case 256: return launch_fwd_gather<S, 256>(q, k, v, coords, out, lse, dm, st);
+    }
+    return DSDPA_ERR_HEAD_DIM;
+}
+
+int zero_fill(float *p, size_t n, hipStream_t st)   // n is a multiple of 4 (D >= 16)
+{
+    const size_t n4 = n / 4;
+    const int threads = 256;
+    size_t blocks = (n4 + threads - 1) / threads;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(threads), 0, st, (float4 *)p, n4);
+    return check_launch();
+}
+
+template <typename S>
+int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
+             const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,
+             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    if (!q || !k || !v || !coords || !out || !lse || !dout || !dq || !dk || !dv) return DSDPA_ERR_NULL_POINTER;
+    if (S::kBytes != 4 && !workspace) return DSDPA_ERR_NULL_POINTER;
+    Dims dm;
+    int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
+    if (rc != DSDPA_OK) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const size_t n = (size_t)dm.rows * D;
+    float *dk_acc, *dv_acc;
+    if (S::kBytes == 4) {
+        dk_acc = (float *)dk;
+        dv_acc = (float *)dv;
+        if ((rc = zero_fill(dk_acc, n, st)) != DSDPA_OK) return rc;
+        if ((rc = zero_fill(dv_acc, n, st)) != DSDPA_OK) return rc;
+    } else {
+        dk_acc = (float *)workspace;
+        dv_acc = dk_acc + n;
+        if ((rc = zero_fill(dk_acc, 2 * n, st)) != DSDPA_OK) return rc;
+    }
+    switch (D) {
+    case 16: rc = launch_bwd_gather<S, 16>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st); break;
+    case 32: rc = launch_bwd_gather<S, 32>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st); break;
+    case 64: rc = launch_bwd_gather<S, 64>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st); break;
+    case 128: rc = launch_bwd_gather<S, 128>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st); break;
+    case 256: rc = launch_bwd_gather<S, 256>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st); break;
+    default: return DSDPA_ERR_HEAD_DIM;
+    }
+    if (rc != DSDPA_OK) return rc;
+    if (S::kBytes != 4) {
+        const size_t n8 = n / 8;
+        const int threads = 256;
+        size_t blocks = (n8 + threads - 1) / threads;
+        if (blocks > 256 * 16) blocks = 256 * 16;
+        hipLaunchKernelGGL((cast_kernel<S>), dim3((unsigned)blocks), dim3(threads), 0, st, dk_acc, dk, n8);
+        hipLaunchKernelGGL((cast_kernel<S>), dim3((unsigned)blocks), dim3(threads), 0, st, dv_acc, dv, n8);
+        rc = check_launch();
+    }
+    return rc;
+}
+
+}  // namespace
+
+extern "C" {
+
+int dsdpa_fwd_f32(const float *q, const float *k, const float *v, const float *coords, float *out, float *lse,
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    return fwd_impl<F32>(q, k, v, coords, out, lse, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+}
+
+int dsdpa_fwd_bf16(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    return fwd_impl<BF16>(q, k, v, coords, out, lse, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+}
+
+int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    return fwd_impl<F16>(q, k, v, coords, out, lse, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+}
+
+int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords, const float *out,
+                  const float *lse, const float *dout, float *dq, float *dk, float *dv, void *workspace,
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    return bwd_impl<F32>(q, k, v, coords, out, lse, dout, dq, dk, dv, workspace, B, V, H, Himg, Wimg, D, P,
+                         sm_scale, stream);
+}
+
+int dsdpa_bwd_bf16(const void *q, const void *k, const void *v, const float *coords, const void *out,
+                   const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,
+                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    return bwd_impl<BF16>(q, k, v, coords, out, lse, dout, dq, dk, dv, workspace, B, V, H, Himg, Wimg, D, P,
+                          sm_scale, stream);
+}
+
+int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coords, const void *out,
+                  const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    return bwd_impl<F16>(q, k, v, coords, out, lse, dout, dq, dk, dv, workspace, B, V, H, Himg, Wimg, D, P,
+                         sm_scale, stream);
+}
+
+size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D)
+{
+    if (dtype == DSDPA_F32) return 0;
+    if (dtype != DSDPA_BF16 && dtype != DSDPA_F16) return 0;
+    if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || D < 1) return 0;
+    return (size_t)2 * sizeof(float) * (size_t)B * V * H * (size_t)Himg * Wimg * D;
+}
+
+const char *dsdpa_error_string(int code)
+{
+    switch (code) {
+    case DSDPA_OK: return "ok";
+    case DSDPA_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case DSDPA_ERR_BAD_SHAPE: return "a dimension is smaller than 1";
+    case DSDPA_ERR_HEAD_DIM: return "head dim must be one of 16, 32, 64, 128, 256";
+    case DSDPA_ERR_TOO_LARGE: return "shape exceeds the 32-bit indexing limits of the kernels";
+    case DSDPA_ERR_HIP: return "a HIP launch failed (see dsdpa_last_hip_error)";
+    case DSDPA_ERR_DTYPE: return "unknown dtype code";
+    }
+    return "unknown error code";
+}
+
+int dsdpa_last_hip_error(void) { return g_last_hip_error; }
+
+int dsdpa_version(void) { return 100; }
+
+int dsdpa_set_path(int path)
+{
+    if (path != DSDPA_PATH_AUTO && path != DSDPA_PATH_GATHER && path != DSDPA_PATH_LDS) return -1;
+    return g_path.exchange(path);
+}
+
+}  // extern "C"

@@ -1,0 +1,198 @@
+// Device-side building blocks shared by every kernel of the deformable
+// multi-view SDPA library: storage-type conversion, bilinear tap computation,
+// wave-level (64-lane) reductions, XCD-aware work mapping.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dsdpa {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kNegBig = -1.0e30f;   // finite stand-in for -inf in running maxima
+constexpr int kWave = 64;
+constexpr int kXcds = 8;              // MI355X: 8 XCDs, workgroups dealt round-robin
+
+struct Dims {
+    int B, V, H, Himg, Wimg, L, P, N;   // N = V*P samples per query row
+    int rows;                           // B*V*H*L query rows
+    float sm_scale;
+};
+
+// ------------------------------------------------------------------ storage types
+struct F32 {
+    using type = float;
+    static constexpr int kBytes = 4;
+    static constexpr bool kBf16 = false;
+};
+struct BF16 {
+    using type = uint16_t;
+    static constexpr int kBytes = 2;
+    static constexpr bool kBf16 = true;
+};
+struct F16 {
+    using type = _Float16;
+    static constexpr int kBytes = 2;
+    static constexpr bool kBf16 = false;
+};
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t x) { return __uint_as_float(((uint32_t)x) << 16); }
+
+// round-to-nearest-even; NaN stays NaN (quiet)
+__device__ __forceinline__ uint16_t f32_to_bf16(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// Load DC consecutive elements starting at a 16-byte aligned address, widened to fp32.
+template <typename S, int DC>
+__device__ __forceinline__ void load_chunk(const void *p, float (&dst)[DC])
+{
+    if constexpr (S::kBytes == 4) {
+        static_assert(DC % 4 == 0, "fp32 chunks are multiples of 4 elements");
+        const float4 *src = reinterpret_cast<const float4 *>(p);
+#pragma unroll
+        for (int i = 0; i < DC / 4; ++i) {
+            float4 t = src[i];
+            dst[4 * i + 0] = t.x; dst[4 * i + 1] = t.y; dst[4 * i + 2] = t.z; dst[4 * i + 3] = t.w;
+        }
+    } else {
+        static_assert(DC % 8 == 0, "16-bit chunks are multiples of 8 elements");
+        const uint4 *src = reinterpret_cast<const uint4 *>(p);
+#pragma unroll
+        for (int i = 0; i < DC / 8; ++i) {
+            uint4 t = src[i];
+            uint32_t w[4] = { t.x, t.y, t.z, t.w };
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (S::kBf16) {
+                    dst[8 * i + 2 * j + 0] = __uint_as_float(w[j] << 16);
+                    dst[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+                } else {
+                    union { uint32_t u; _Float16 h[2]; } cv;
+                    cv.u = w[j];
+                    dst[8 * i + 2 * j + 0] = (float)cv.h[0];
+                    dst[8 * i + 2 * j + 1] = (float)cv.h[1];
+                }
+            }
+        }
+    }
+}
+
+// Store DC consecutive fp32 values, narrowed (RNE) to the storage type.
+template <typename S, int DC>
+__device__ __forceinline__ void store_chunk(void *p, const float (&src)[DC])
+{
+    if constexpr (S::kBytes == 4) {
+        float4 *dst = reinterpret_cast<float4 *>(p);
+#pragma unroll
+        for (int i = 0; i < DC / 4; ++i)
+            dst[i] = make_float4(src[4 * i], src[4 * i + 1], src[4 * i + 2], src[4 * i + 3]);
+    } else {
+        uint4 *dst = reinterpret_cast<uint4 *>(p);
+#pragma unroll
+        for (int i = 0; i < DC / 8; ++i) {
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float a = src[8 * i + 2 * j], b = src[8 * i + 2 * j + 1];
+                if constexpr (S::kBf16) {
+                    w[j] = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+                } else {
+                    union { uint32_t u; _Float16 h[2]; } cv;
+                    cv.h[0] = (_Float16)a;
+                    cv.h[1] = (_Float16)b;
+                    w[j] = cv.u;
+                }
+            }
+            dst[i] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ bilinear taps
+// The four taps of one normalised coordinate. x_pix = x*(W-1), y_pix = y*(Himg-1)
+// (align_corners=True), written as the two-step un-normalisation the library
+// routine uses so that both sides see the same fp32 roundings. Zero padding is
+// per tap: a tap outside the image gets weight 0 (its pixel index is clamped
+// into the image so that the gather stays in bounds), the other taps keep
+// theirs. NaN/inf coordinates drop all four taps.
+struct Taps {
+    float w[4];     // 00 (row0,col0), 01 (row0,col1), 10, 11
+    int pix[4];     // row*W + col, always inside [0, L)
+};
+
+__device__ __forceinline__ Taps make_taps(float cx, float cy, int Wimg, int Himg)
+{
+    float gx = cx * 2.0f - 1.0f;
+    float gy = cy * 2.0f - 1.0f;
+    float x = (gx + 1.0f) * ((float)(Wimg - 1) * 0.5f);
+    float y = (gy + 1.0f) * ((float)(Himg - 1) * 0.5f);
+    float x0f = floorf(x), y0f = floorf(y);
+    float fx = x - x0f, fy = y - y0f;
+    x0f = fminf(fmaxf(x0f, -2.0f), (float)Wimg + 1.0f);   // NaN -> -2 (outside)
+    y0f = fminf(fmaxf(y0f, -2.0f), (float)Himg + 1.0f);
+    int x0 = (int)x0f, y0 = (int)y0f;
+    int x1 = x0 + 1, y1 = y0 + 1;
+    bool vx0 = (x0 >= 0) & (x0 < Wimg), vx1 = (x1 >= 0) & (x1 < Wimg);
+    bool vy0 = (y0 >= 0) & (y0 < Himg), vy1 = (y1 >= 0) & (y1 < Himg);
+    int cx0 = min(max(x0, 0), Wimg - 1), cx1 = min(max(x1, 0), Wimg - 1);
+    int cy0 = min(max(y0, 0), Himg - 1), cy1 = min(max(y1, 0), Himg - 1);
+    float wx0 = 1.0f - fx, wy0 = 1.0f - fy;
+    Taps t;
+    t.w[0] = (vx0 & vy0) ? wx0 * wy0 : 0.0f;
+    t.w[1] = (vx1 & vy0) ? fx * wy0 : 0.0f;
+    t.w[2] = (vx0 & vy1) ? wx0 * fy : 0.0f;
+    t.w[3] = (vx1 & vy1) ? fx * fy : 0.0f;
+    t.pix[0] = cy0 * Wimg + cx0;
+    t.pix[1] = cy0 * Wimg + cx1;
+    t.pix[2] = cy1 * Wimg + cx0;
+    t.pix[3] = cy1 * Wimg + cx1;
+    return t;
+}
+
+// ------------------------------------------------------------------ wave-level helpers
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float x)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
+
+// Sum over aligned groups of G consecutive lanes (G a power of two <= 64); every
+// lane of the group ends up with the group's sum.
+template <int G>
+__device__ __forceinline__ float group_sum(float x)
+{
+    if constexpr (G >= 2) x += dpp_f32<0xB1>(x);    // quad_perm [1,0,3,2]
+    if constexpr (G >= 4) x += dpp_f32<0x4E>(x);    // quad_perm [2,3,0,1]
+    if constexpr (G >= 8) x += dpp_f32<0x141>(x);   // row_half_mirror
+    if constexpr (G >= 16) x += dpp_f32<0x140>(x);  // row_mirror
+    if constexpr (G >= 32) x += __shfl_xor(x, 16, kWave);
+    if constexpr (G >= 64) x += __shfl_xor(x, 32, kWave);
+    return x;
+}
+
+// Orders this wave's LDS writes before its later LDS reads (and the reverse):
+// waits for the wave's outstanding LDS traffic and stops the compiler from
+// moving LDS accesses across. No workgroup barrier is involved.
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// Workgroups are dealt to the 8 XCDs round-robin by their linear id, and each
+// XCD has its own L2. This maps the hardware block id to a logical one so that
+// every XCD walks one contiguous range of logical ids (hence of (batch, head)
+// pairs, whose K/V planes then stay in that XCD's L2). A bijection on [0, nb).
+__device__ __forceinline__ int xcd_logical_block(int bid, int nb)
+{
+    int x = bid % kXcds, i = bid / kXcds;
+    int qn = nb / kXcds, rn = nb % kXcds;
+    return x * qn + min(x, rn) + i;
+}
+
+}  // namespace dsdpa

@@ -1,0 +1,76 @@
+"""ctypes binding of libdsdpa.so (the C ABI declared in ``include/dsdpa.h``).
+
+The library is loaded from ``lib/libdsdpa.so`` next to this package. There is
+no fallback: if the library is missing, or a call returns an error code, an
+exception is raised.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libdsdpa.so")
+
+# every symbol include/dsdpa.h declares
+SYMBOLS = (
+    "dsdpa_fwd_f32", "dsdpa_fwd_bf16", "dsdpa_fwd_f16",
+    "dsdpa_bwd_f32", "dsdpa_bwd_bf16", "dsdpa_bwd_f16",
+    "dsdpa_bwd_workspace_bytes", "dsdpa_error_string", "dsdpa_last_hip_error",
+    "dsdpa_version", "dsdpa_set_path",
+)
+
+DSDPA_F32, DSDPA_BF16, DSDPA_F16 = 0, 1, 2
+PATH_AUTO, PATH_GATHER, PATH_LDS = 0, 1, 2
+
+_lib = None
+
+
+class DsdpaError(RuntimeError):
+    """A libdsdpa entry point returned a non-zero code."""
+
+
+def load():
+    """Load libdsdpa.so once and declare the signatures. Raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python build.py` (hipcc, gfx950). "
+            "There is no fallback path for the fused operator.")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, i, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    dims = [i, i, i, i, i, i, i, f, vp]            # B V H Himg Wimg D P sm_scale stream
+    for sfx in ("f32", "bf16", "f16"):
+        fwd = getattr(lib, "dsdpa_fwd_" + sfx)
+        fwd.argtypes = [vp] * 6 + dims
+        fwd.restype = i
+        bwd = getattr(lib, "dsdpa_bwd_" + sfx)
+        bwd.argtypes = [vp] * 11 + dims
+        bwd.restype = i
+    lib.dsdpa_bwd_workspace_bytes.argtypes = [i] * 7
+    lib.dsdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.dsdpa_error_string.argtypes = [i]
+    lib.dsdpa_error_string.restype = ctypes.c_char_p
+    lib.dsdpa_last_hip_error.argtypes = []
+    lib.dsdpa_last_hip_error.restype = i
+    lib.dsdpa_version.argtypes = []
+    lib.dsdpa_version.restype = i
+    lib.dsdpa_set_path.argtypes = [i]
+    lib.dsdpa_set_path.restype = i
+    _lib = lib
+    return lib
+
+
+def check(code):
+    if code != 0:
+        lib = load()
+        msg = lib.dsdpa_error_string(code).decode()
+        raise DsdpaError(f"libdsdpa error {code}: {msg} (hip error {lib.dsdpa_last_hip_error()})")
+
+
+def set_path(path):
+    """Force a kernel path (PATH_AUTO / PATH_GATHER / PATH_LDS); returns the previous one."""
+    prev = load().dsdpa_set_path(int(path))
+    if prev < 0:
+        raise ValueError(f"unknown kernel path {path}")
+    return prev

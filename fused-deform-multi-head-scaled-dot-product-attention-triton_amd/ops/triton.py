@@ -1,0 +1,112 @@
+"""Fused deformable multi-view SDPA: the autograd front-end over libdsdpa.so.
+
+Drop-in for the reference operator ``deform_sdpa_triton`` (``ops/triton.py:466``;
+the module and function names are kept so ``from ops.triton import
+deform_sdpa_triton`` keeps working -- there is no Triton here, the kernels are
+hand-written HIP for gfx950 reached through a C ABI).
+
+Contract mirrored from ``_fused_deform_sdpa`` (``ops/triton.py:377-466``):
+
+* ``deform_sdpa_triton(q, k, v, coords, WIDTH, HEIGHT, sm_scale) -> out``,
+  positional; q/k/v ``(B, N_VIEWS, N_HEADS, H*W, D)``, coords
+  ``(B, N_VIEWS, H*W, N_VIEWS, N_SAMPLES, 2)`` normalised ``(x, y)``;
+* gradients for q, k, v only; coords/WIDTH/HEIGHT/sm_scale get ``None``;
+* ``AssertionError`` for unequal head dims, ``D`` outside {16,32,64,128,256},
+  ``q.shape[3] != WIDTH*HEIGHT``, non-contiguous coords;
+  ``NotImplementedError`` for an unsupported dtype;
+* fp32 storage, or bf16/fp16 storage with fp32 accumulation.
+
+Differences, all on purpose: coords are not cloned or pre-scaled (the kernels
+un-normalise), ``out``/``dq`` are not zero-filled first, no scaled copy of K is
+made, out-of-image taps follow the eager operator's per-tap zero padding
+(``ops/torch.py:14-15``) rather than ``ops/triton.py:129,135-136``, q/k/v/dout
+are made contiguous instead of asserted, and only the log-sum-exp is saved on
+top of the inputs and output.
+"""
+import torch
+
+from . import _native
+
+_SUFFIX = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}
+_DTYPE_CODE = {torch.float32: _native.DSDPA_F32, torch.bfloat16: _native.DSDPA_BF16,
+               torch.float16: _native.DSDPA_F16}
+
+
+def _suffix_from(t):
+    """Storage mode of a tensor (the reference's ``_dtype_mode_from``, ops/triton.py:367-375)."""
+    try:
+        return _SUFFIX[t.dtype]
+    except KeyError:
+        raise NotImplementedError(f"unsupported dtype {t.dtype}") from None
+
+
+def _stream_ptr(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _check_inputs(q, k, v, coords, WIDTH, HEIGHT):
+    sfx = _suffix_from(q)
+    assert q.dim() == 5 and k.shape == q.shape and v.shape == q.shape, "q, k, v must share (B, V, H, L, D)"
+    assert q.shape[-1] == k.shape[-1] == v.shape[-1]
+    assert q.shape[-1] in {16, 32, 64, 128, 256}
+    assert q.shape[3] == WIDTH * HEIGHT
+    assert coords.is_contiguous()
+    B, V, H, L, D = q.shape
+    if coords.dim() != 6 or coords.shape[:4] != (B, V, L, V) or coords.shape[-1] != 2:
+        raise RuntimeError(f"coords must be (B, V, L, V, P, 2) = ({B}, {V}, {L}, {V}, P, 2), got {tuple(coords.shape)}")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError("q, k, v must share one dtype")
+    if not q.is_cuda:
+        raise RuntimeError("deform_sdpa_triton runs on the GPU only (HIP kernels); "
+                           "use ops.torch.deform_sdpa_torch for an eager operator")
+    if not (k.device == q.device and v.device == q.device and coords.device == q.device):
+        raise RuntimeError("q, k, v, coords must be on one device")
+    return sfx
+
+
+class _fused_deform_sdpa(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, coords, WIDTH, HEIGHT, sm_scale):
+        sfx = _check_inputs(q, k, v, coords, WIDTH, HEIGHT)
+        lib = _native.load()
+        B, V, H, L, D = q.shape
+        P = coords.shape[-2]
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        if coords.dtype != torch.float32:
+            coords = coords.float()
+        out = torch.empty_like(q)
+        lse = torch.empty((B, V, H, L), device=q.device, dtype=torch.float32)
+        with torch.cuda.device(q.device):
+            rc = getattr(lib, "dsdpa_fwd_" + sfx)(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), coords.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                B, V, H, HEIGHT, WIDTH, D, P, float(sm_scale), _stream_ptr(q.device))
+        _native.check(rc)
+        ctx.save_for_backward(q, k, v, coords, out, lse)
+        ctx.sm_scale = float(sm_scale)
+        ctx.WIDTH, ctx.HEIGHT = WIDTH, HEIGHT
+        return out
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, coords, out, lse = ctx.saved_tensors
+        lib = _native.load()
+        sfx = _SUFFIX[q.dtype]
+        B, V, H, L, D = q.shape
+        P = coords.shape[-2]
+        do = do.contiguous()
+        if do.dtype != q.dtype:
+            do = do.to(q.dtype)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        ws_bytes = lib.dsdpa_bwd_workspace_bytes(_DTYPE_CODE[q.dtype], B, V, H, ctx.HEIGHT, ctx.WIDTH, D)
+        ws = torch.empty(ws_bytes // 4, device=q.device, dtype=torch.float32) if ws_bytes else None
+        with torch.cuda.device(q.device):
+            rc = getattr(lib, "dsdpa_bwd_" + sfx)(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), coords.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                do.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                ws.data_ptr() if ws is not None else None,
+                B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P, ctx.sm_scale, _stream_ptr(q.device))
+        _native.check(rc)
+        return dq, dk, dv, None, None, None, None
+
+
+deform_sdpa_triton = _fused_deform_sdpa.apply

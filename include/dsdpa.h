@@ -1,0 +1,129 @@
+/*
+ * dsdpa.h -- C ABI of the MI355X (gfx950) fused deformable multi-view
+ * scaled-dot-product attention library (libdsdpa.so).
+ *
+ * The reference is pure Python: its operator boundary is the autograd
+ * function `_fused_deform_sdpa` (ops/triton.py:377-466), which launches the
+ * Triton kernels `_fwd_kernel` (ops/triton.py:27-194), `_bwd_preprocess`
+ * (ops/triton.py:197-215) and `_bwd_kernel` (ops/triton.py:219-365). It has no
+ * FFI of its own; the entry points below are what a binding for that path
+ * would call instead of those three launches.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every pointer is DEVICE memory owned by
+ *     the caller; nothing is allocated or freed by the library;
+ *   - tensors are contiguous, row-major:
+ *         q, k, v, out, dout, dq, dk, dv : [B][V][H][L][D],  L = Himg*Wimg
+ *         coords : [B][V][L][V][P][2] float32, (x, y) normalised to [0, 1],
+ *                  x along WIDTH (columns), y along HEIGHT (rows); shared by
+ *                  all heads (ops/torch.py:10, ops/triton.py:51)
+ *         lse    : [B][V][H][L] float32, base-2 log-sum-exp of
+ *                  sm_scale*log2(e)*(q.k~) per query row (the reference's
+ *                  `M`, ops/triton.py:187-190)
+ *   - coordinates are passed NORMALISED; the un-normalisation
+ *     x_pix = x*(W-1), y_pix = y*(Himg-1) (ops/triton.py:381-383) is done
+ *     inside the kernels, and out-of-image taps follow the eager reference's
+ *     per-tap zero padding (ops/torch.py:14-15), not ops/triton.py:129;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     all work is enqueued on it and the call returns without synchronising;
+ *   - D (head dim) must be one of 16, 32, 64, 128, 256 (ops/triton.py:386);
+ *   - every entry point returns 0 on success or a DSDPA_ERR_* code, never
+ *     throws, and is re-entrant (no global mutable state).
+ */
+#ifndef DSDPA_H
+#define DSDPA_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    DSDPA_OK = 0,
+    DSDPA_ERR_NULL_POINTER = 1,   /* a required pointer is NULL                           */
+    DSDPA_ERR_BAD_SHAPE = 2,      /* a dimension is < 1                                   */
+    DSDPA_ERR_HEAD_DIM = 3,       /* D not in {16,32,64,128,256} (ops/triton.py:386)      */
+    DSDPA_ERR_TOO_LARGE = 4,      /* a per-batch slab V*H*L*D exceeds 2^30 elements or
+                                     rows exceed 2^31-1                                   */
+    DSDPA_ERR_HIP = 5,            /* a HIP launch failed; see dsdpa_last_hip_error()      */
+    DSDPA_ERR_DTYPE = 6           /* unknown dtype code                                   */
+};
+
+/* Storage types (accumulation is always fp32). Mirrors the reference's dtype
+ * modes, ops/triton.py:367-375: fp32 = mode 0, fp16/bf16 = mode 1. */
+enum { DSDPA_F32 = 0, DSDPA_BF16 = 1, DSDPA_F16 = 2 };
+
+/*
+ * Forward: replaces the `_fwd_kernel[grid](...)` launch, ops/triton.py:396-411,
+ * including the coords clone/scale (:381-383) and the zero-fill of `o` (:389).
+ * Writes out (storage dtype) and lse (fp32).
+ */
+int dsdpa_fwd_f32(const float *q, const float *k, const float *v, const float *coords,
+                  float *out, float *lse,
+                  int B, int V, int H, int Himg, int Wimg, int D, int P,
+                  float sm_scale, void *stream);
+int dsdpa_fwd_bf16(const void *q, const void *k, const void *v, const float *coords,
+                   void *out, float *lse,
+                   int B, int V, int H, int Himg, int Wimg, int D, int P,
+                   float sm_scale, void *stream);
+int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coords,
+                  void *out, float *lse,
+                  int B, int V, int H, int Himg, int Wimg, int D, int P,
+                  float sm_scale, void *stream);
+
+/*
+ * Backward: replaces everything `_fused_deform_sdpa.backward` enqueues,
+ * ops/triton.py:427-462: the zero-fills (:427-430), the scaled copy of K
+ * (:431-432), `_bwd_preprocess` (:436-441), `_bwd_kernel` (:443-459) and the
+ * fp32 -> storage casts of dk/dv (:461-462).
+ *
+ * dq, dk, dv are fully overwritten (no pre-zeroing by the caller needed).
+ * fp32: dk and dv are themselves the accumulators; `workspace` may be NULL.
+ * bf16/fp16: `workspace` must hold dsdpa_bwd_workspace_bytes(...) bytes; it
+ * carries the fp32 dk/dv accumulators that are rounded to the storage type at
+ * the end. Accumulation order into dk/dv is not deterministic (float atomics,
+ * as in the reference, ops/triton.py:345-360).
+ */
+int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords,
+                  const float *out, const float *lse, const float *dout,
+                  float *dq, float *dk, float *dv, void *workspace,
+                  int B, int V, int H, int Himg, int Wimg, int D, int P,
+                  float sm_scale, void *stream);
+int dsdpa_bwd_bf16(const void *q, const void *k, const void *v, const float *coords,
+                   const void *out, const float *lse, const void *dout,
+                   void *dq, void *dk, void *dv, void *workspace,
+                   int B, int V, int H, int Himg, int Wimg, int D, int P,
+                   float sm_scale, void *stream);
+int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coords,
+                  const void *out, const float *lse, const void *dout,
+                  void *dq, void *dk, void *dv, void *workspace,
+                  int B, int V, int H, int Himg, int Wimg, int D, int P,
+                  float sm_scale, void *stream);
+
+/* Bytes of device workspace dsdpa_bwd_* needs for a storage dtype (0 for fp32).
+ * Counterpart of the reference's dk32/dv32 temporaries, ops/triton.py:428-429. */
+size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D);
+
+/* Human-readable text for a DSDPA_ERR_* code. */
+const char *dsdpa_error_string(int code);
+
+/* hipError_t (as int) of the most recent failed launch on the calling thread, 0 if none. */
+int dsdpa_last_hip_error(void);
+
+/* Library version: major*10000 + minor*100 + patch. */
+int dsdpa_version(void);
+
+/*
+ * Kernel-path selection, for measurement and tests. `path` is one of
+ * DSDPA_PATH_*; AUTO picks per shape. Returns the previous value, or -1 if
+ * `path` is unknown. Process-wide; the reference's analogue is the autotune
+ * table, ops/triton.py:10-25.
+ */
+enum { DSDPA_PATH_AUTO = 0, DSDPA_PATH_GATHER = 1, DSDPA_PATH_LDS = 2 };
+int dsdpa_set_path(int path);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DSDPA_H */

@@ -1,0 +1,88 @@
+"""CPU-side checks of the C ABI: the library loads without a GPU and exports
+every symbol include/dsdpa.h declares; argument validation happens before any
+launch, so the error paths run here too."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from ops import _native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "dsdpa.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dsdpa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_all_exported():
+    lib = _native.load()
+    declared = _declared_symbols()
+    assert len(declared) >= 11
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/dsdpa.h but not exported"
+    assert sorted(_native.SYMBOLS) == declared
+
+
+def test_version_and_error_strings():
+    lib = _native.load()
+    assert lib.dsdpa_version() >= 100
+    assert lib.dsdpa_error_string(0) == b"ok"
+    for code in range(1, 7):
+        assert len(lib.dsdpa_error_string(code)) > 3
+    assert b"unknown" in lib.dsdpa_error_string(99)
+
+
+def test_workspace_bytes():
+    lib = _native.load()
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32) == 0
+    n = 2 * 6 * 8 * 48 * 48 * 64
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64) == 8 * n
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F16, 2, 6, 8, 48, 48, 64) == 8 * n
+
+
+def test_argument_validation_before_launch():
+    """Bad arguments are rejected with an error code before anything touches the GPU."""
+    lib = _native.load()
+    fake = ctypes.c_void_p(0x1000)   # never dereferenced: validation fails first
+    ok_dims = (1, 2, 2, 3, 4, 32, 2, 0.5, None)
+    assert lib.dsdpa_fwd_f32(None, fake, fake, fake, fake, fake, *ok_dims) == 1
+    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, 0, 2, 2, 3, 4, 32, 2, 0.5, None) == 2
+    assert lib.dsdpa_fwd_bf16(fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 48, 2, 0.5, None) == 3
+    assert lib.dsdpa_fwd_f16(fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 8, 2, 0.5, None) == 3
+    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, 1, 64, 64, 1024, 1024, 256, 2, 0.5, None) == 4
+    # backward: 16-bit storage needs a workspace
+    args = [fake] * 10
+    assert lib.dsdpa_bwd_bf16(*args, None, *ok_dims) == 1
+    assert lib.dsdpa_bwd_f32(*args[:9], None, None, *ok_dims) == 1
+    assert lib.dsdpa_bwd_f32(*args, None, 1, 2, 2, 3, 4, 33, 2, 0.5, None) == 3
+
+
+def test_path_selector():
+    assert _native.set_path(_native.PATH_AUTO) in (0, 1, 2)
+    prev = _native.set_path(_native.PATH_GATHER)
+    assert prev == _native.PATH_AUTO
+    assert _native.set_path(_native.PATH_AUTO) == _native.PATH_GATHER
+    with pytest.raises(ValueError):
+        _native.set_path(77)
+
+
+def test_operator_contract_errors_on_cpu():
+    """The Python front-end raises the reference's exception classes (ops/triton.py:375,385-388)."""
+    import torch
+    from ops.triton import deform_sdpa_triton
+    q = torch.randn(1, 2, 2, 12, 32)
+    c = torch.rand(1, 2, 12, 2, 3, 2)
+    with pytest.raises(NotImplementedError):
+        deform_sdpa_triton(q.double(), q.double(), q.double(), c, 4, 3, 0.5)
+    with pytest.raises(AssertionError):
+        deform_sdpa_triton(q, q, q, c, 4, 4, 0.5)                      # L != W*H
+    with pytest.raises(AssertionError):
+        deform_sdpa_triton(q[..., :24], q[..., :24], q[..., :24], c, 4, 3, 0.5)   # head dim 24
+    with pytest.raises(AssertionError):
+        deform_sdpa_triton(q, q, q, c.transpose(3, 4).contiguous().transpose(3, 4), 4, 3, 0.5)
+    with pytest.raises(RuntimeError):
+        deform_sdpa_triton(q, q, q, c, 4, 3, 0.5)                      # CPU tensors: no fallback

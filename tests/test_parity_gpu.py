@@ -1,0 +1,230 @@
+"""GPU parity: the HIP kernels (through the operator and the C ABI) against the CPU oracle.
+
+Error measure, everywhere: rel = max|x - ref| / max|ref| per tensor.
+Bars: fp32 forward 1e-4, fp32 gradients 1e-3 (atomic ordering is not
+deterministic), 16-bit storage 2e-2 (bf16 and fp16; the oracle is fed the
+rounded inputs up-cast to fp32, which is what ops/torch.py:8,9,20 does).
+"""
+import glob
+import math
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle_bwd, oracle_fwd
+from ops import _native
+from ops.triton import deform_sdpa_triton
+from workloads import WORKLOADS, gen_inputs
+
+pytestmark = pytest.mark.gpu
+
+TOL_FWD = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+TOL_BWD = {torch.float32: 1e-3, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+PATHS = {"gather": _native.PATH_GATHER, "auto": _native.PATH_AUTO}
+
+
+def rel(a, b):
+    a = a.detach().double().cpu().numpy() if torch.is_tensor(a) else np.asarray(a, dtype=np.float64)
+    b = b.detach().double().cpu().numpy() if torch.is_tensor(b) else np.asarray(b, dtype=np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def run_op(q, k, v, coords, dout, W, Himg, scale):
+    dev = "cuda:0"
+    qg, kg, vg = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    out = deform_sdpa_triton(qg, kg, vg, coords.to(dev), W, Himg, scale)
+    out.backward(dout.to(dev))
+    torch.cuda.synchronize()
+    return out.detach(), qg.grad, kg.grad, vg.grad
+
+
+def oracle_all(q, k, v, coords, dout, W, Himg, scale):
+    f = lambda t: t.float().numpy()
+    out, lse = oracle_fwd(f(q), f(k), f(v), f(coords), W, Himg, scale)
+    dq, dk, dv = oracle_bwd(f(q), f(k), f(v), f(coords), f(dout), W, Himg, scale)
+    return out, lse, dq, dk, dv
+
+
+def make_case(seed, B, V, H, Himg, Wimg, D, P, lo, hi, dtype):
+    g = torch.Generator().manual_seed(seed)
+    L = Himg * Wimg
+    q, k, v = (torch.randn(B, V, H, L, D, generator=g).to(dtype) for _ in range(3))
+    coords = torch.rand(B, V, L, V, P, 2, generator=g) * (hi - lo) + lo
+    dout = torch.randn(B, V, H, L, D, generator=g).to(dtype)
+    return q, k, v, coords, dout
+
+
+SMALL = [
+    # seed B  V  H  Himg Wimg D    P   lo    hi
+    (1, 1, 2, 2, 3, 5, 16, 3, -0.25, 1.25),     # tiny, non-square, N=6 < one chunk
+    (2, 2, 3, 2, 6, 4, 32, 23, -0.1, 1.1),      # N=69: one full chunk + ragged tail
+    (3, 1, 4, 3, 7, 9, 32, 32, 0.0, 1.0),       # N=128, L=63 not a multiple of the row tile
+    (4, 1, 2, 2, 5, 6, 64, 17, -0.5, 1.5),      # heavy out-of-image
+    (5, 2, 2, 1, 4, 7, 128, 40, 0.0, 1.0),
+    (6, 1, 2, 1, 3, 3, 256, 9, -0.1, 1.1),
+    (7, 1, 1, 1, 1, 1, 16, 1, 0.0, 1.0),        # degenerate 1x1 image, one sample
+    (8, 1, 3, 2, 1, 11, 32, 5, -0.2, 1.2),      # single-row image
+    (9, 1, 3, 2, 11, 1, 32, 5, -0.2, 1.2),      # single-column image
+]
+
+
+@pytest.mark.parametrize("path", sorted(PATHS))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("case", SMALL, ids=[f"s{c[0]}" for c in SMALL])
+def test_small_cases_vs_oracle(case, dtype, path):
+    seed, B, V, H, Himg, Wimg, D, P, lo, hi = case
+    say(f"[case] small seed={seed} B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} {dtype} path={path}")
+    q, k, v, c, do = make_case(seed, B, V, H, Himg, Wimg, D, P, lo, hi, dtype)
+    scale = 1.0 / math.sqrt(D)
+    prev = _native.set_path(PATHS[path])
+    try:
+        out, dq, dk, dv = run_op(q, k, v, c, do, Wimg, Himg, scale)
+    finally:
+        _native.set_path(prev)
+    ro, _, rdq, rdk, rdv = oracle_all(q, k, v, c, do, Wimg, Himg, scale)
+    assert out.dtype == dtype and dq.dtype == dtype and dk.dtype == dtype and dv.dtype == dtype
+    assert rel(out, ro) < TOL_FWD[dtype]
+    assert rel(dq, rdq) < TOL_BWD[dtype]
+    assert rel(dk, rdk) < TOL_BWD[dtype]
+    assert rel(dv, rdv) < TOL_BWD[dtype]
+
+
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-4] for p in GOLDEN])
+def test_golden_fixtures(path):
+    z = np.load(path)
+    say(f"[case] golden {os.path.basename(path)}")
+    W, Himg, scale = int(z["WIDTH"]), int(z["HEIGHT"]), float(z["sm_scale"])
+    t = lambda n: torch.from_numpy(z[n])
+    out, dq, dk, dv = run_op(t("q"), t("k"), t("v"), t("coords"), t("dout"), W, Himg, scale)
+    assert rel(out, z["out"]) < 1e-4
+    assert rel(dq, z["dq"]) < 1e-3
+    assert rel(dk, z["dk"]) < 1e-3
+    assert rel(dv, z["dv"]) < 1e-3
+
+
+def test_lse_through_c_abi():
+    """Direct C-ABI forward call: out and the base-2 log-sum-exp side buffer."""
+    say("[case] c-abi forward lse")
+    q, k, v, c, _ = make_case(21, 2, 3, 2, 6, 4, 32, 23, -0.1, 1.1, torch.float32)
+    lib = _native.load()
+    dev = "cuda:0"
+    qg, kg, vg, cg = (t.to(dev).contiguous() for t in (q, k, v, c))
+    out = torch.empty_like(qg)
+    lse = torch.empty(q.shape[:4], device=dev, dtype=torch.float32)
+    rc = lib.dsdpa_fwd_f32(qg.data_ptr(), kg.data_ptr(), vg.data_ptr(), cg.data_ptr(), out.data_ptr(),
+                           lse.data_ptr(), 2, 3, 2, 6, 4, 32, 23, 0.2, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ro, rl = oracle_fwd(q.numpy(), k.numpy(), v.numpy(), c.numpy(), 4, 6, 0.2)
+    assert rel(out, ro) < 1e-4
+    assert np.abs(lse.cpu().numpy() - rl).max() < 1e-4
+
+
+def test_closed_forms_on_gpu():
+    say("[case] closed forms")
+    q, k, v, c, do = make_case(22, 1, 2, 2, 4, 3, 32, 5, 0.0, 1.0, torch.float32)
+    dev = "cuda:0"
+    # constant V -> out is that constant
+    out = deform_sdpa_triton(q.to(dev), k.to(dev), torch.full_like(v, 2.5).to(dev), c.to(dev), 3, 4, 0.9)
+    assert (out - 2.5).abs().max().item() < 1e-5
+    # everything far outside: out = 0, all gradients 0
+    out, dq, dk, dv = run_op(q, k, v, c + 7.0, do, 3, 4, 0.9)
+    assert out.abs().max().item() == 0.0
+    assert dq.abs().max().item() == 0.0 and dk.abs().max().item() == 0.0 and dv.abs().max().item() == 0.0
+    # NaN coordinates drop their samples instead of poisoning the row
+    cn = c.clone()
+    cn[0, 0, 0, 0, 0, 0] = float("nan")
+    out = deform_sdpa_triton(q.to(dev), k.to(dev), v.to(dev), cn.to(dev), 3, 4, 0.9)
+    ro, _ = oracle_fwd(q.numpy(), k.numpy(), v.numpy(), cn.numpy(), 3, 4, 0.9)
+    assert torch.isfinite(out).all()
+    assert rel(out, ro) < 1e-4
+
+
+def test_reentrant_backward_and_noncontiguous_inputs():
+    """retain_graph re-entry (benchmark.py:79) and strided q/k/v/dout."""
+    say("[case] re-entrant backward")
+    q, k, v, c, do = make_case(23, 1, 2, 2, 4, 5, 32, 6, 0.0, 1.0, torch.float32)
+    dev = "cuda:0"
+    base = torch.randn(1, 2, 2, 20, 64, generator=torch.Generator().manual_seed(1)).to(dev)
+    qg = base[..., ::2].detach().requires_grad_(True)          # non-contiguous view
+    kg, vg = k.to(dev).requires_grad_(True), v.to(dev).requires_grad_(True)
+    out = deform_sdpa_triton(qg, kg, vg, c.to(dev), 5, 4, 0.3)
+    dog = do.to(dev)
+    out.backward(dog, retain_graph=True)
+    g1 = (qg.grad.clone(), kg.grad.clone(), vg.grad.clone())
+    qg.grad = kg.grad = vg.grad = None
+    out.backward(dog.transpose(-1, -2).contiguous().transpose(-1, -2), retain_graph=True)
+    ro, _, rdq, rdk, rdv = oracle_all(qg.detach().cpu(), k, v, c, do, 5, 4, 0.3)
+    assert rel(out, ro) < 1e-4
+    for got, again, ref in zip((qg.grad, kg.grad, vg.grad), g1, (rdq, rdk, rdv)):
+        assert rel(got, ref) < 1e-3 and rel(again, ref) < 1e-3
+
+
+# ------------------------------------------------------------------ the five named workloads
+def _slice_bh(t, b, h):
+    return t[b:b + 1, :, h:h + 1].contiguous()
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
+def test_named_workloads_full_size(name):
+    """Full-size run of each workload. The oracle checks (batch, head) slices (batches
+    and heads are independent and coords are shared by heads, so a slice of the full
+    result must equal the oracle run on the slice); size-independent identities cover
+    the whole tensors: <q,dq> = <K,dK> (logits bilinear in q,K) and <V,dV> = <dout,out>."""
+    wl = WORKLOADS[name]
+    say(f"[case] workload {name} {wl}")
+    q, k, v, c, do = gen_inputs(wl)
+    dt = wl.torch_dtype()
+    out, dq, dk, dv = run_op(q, k, v, c, do, wl.W_IMG, wl.H_IMG, wl.sm_scale)
+    assert torch.isfinite(out).all() and torch.isfinite(dq).all()
+    assert torch.isfinite(dk).all() and torch.isfinite(dv).all()
+    # identities over the full tensors (fp64 sums on the GPU)
+    a = (q.to("cuda").double() * dq.double()).sum().item()
+    b = (k.to("cuda").double() * dk.double()).sum().item()
+    e = (v.to("cuda").double() * dv.double()).sum().item()
+    f = (do.to("cuda").double() * out.double()).sum().item()
+    tol_id = 1e-3 if dt == torch.float32 else 3e-2
+    norm_qk = (q.double().norm() * dq.double().norm().cpu()).item()
+    norm_v = (do.double().norm() * out.double().norm().cpu()).item()
+    assert abs(a - b) < tol_id * norm_qk, (a, b)
+    assert abs(e - f) < tol_id * norm_v, (e, f)
+    # oracle on slices
+    slices = [(0, 0), (wl.B - 1, wl.H - 1)] if wl.query_samples <= 2e7 else [(wl.B - 1, wl.H // 2)]
+    for (bb, hh) in slices:
+        say(f"        oracle slice b={bb} h={hh}")
+        ro, _, rdq, rdk, rdv = oracle_all(_slice_bh(q, bb, hh), _slice_bh(k, bb, hh), _slice_bh(v, bb, hh),
+                                          c[bb:bb + 1].contiguous(), _slice_bh(do, bb, hh),
+                                          wl.W_IMG, wl.H_IMG, wl.sm_scale)
+        assert rel(_slice_bh(out, bb, hh), ro) < TOL_FWD[dt]
+        assert rel(_slice_bh(dq, bb, hh), rdq) < TOL_BWD[dt]
+        assert rel(_slice_bh(dk, bb, hh), rdk) < TOL_BWD[dt]
+        assert rel(_slice_bh(dv, bb, hh), rdv) < TOL_BWD[dt]
+
+
+def test_peak_memory_is_linear_in_tensor_size():
+    """No sampled-tensor materialisation: fwd+bwd peak stays within a small multiple of
+    the q/k/v/out/grad tensors (the eager path needs 2*QS*D*4 bytes = 1.5 GB here)."""
+    wl = WORKLOADS["C2"]
+    say("[case] peak memory C2")
+    q, k, v, c, do = gen_inputs(wl, device="cuda")
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    out = deform_sdpa_triton(q, k, v, c, wl.W_IMG, wl.H_IMG, wl.sm_scale)
+    out.backward(do)
+    torch.cuda.synchronize()
+    extra = torch.cuda.max_memory_allocated() - base
+    tensor_bytes = q.numel() * q.element_size()
+    assert extra <= 8 * tensor_bytes, (extra, tensor_bytes)
