@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused deformable multi-view SDPA operator on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--all] [--no-cpu]
+
+A "step" is one forward + backward pass of the public operator
+(`deform_sdpa_triton`, autograd) over one batch of the workload, inputs already
+resident in HBM. Prints ONE JSON line on stdout:
+
+  metric/value   M query.samples/s of fwd+bwd (query.samples = B*V*H*L * V*P)
+  roofline       the dominant kernel against the 8 TB/s HBM roofline on its
+                 algorithmic (compulsory) bytes; its average duration is measured
+                 here with HIP events recorded by the library around that kernel
+                 on the launch stream, during the timed steps
+  cpu_baseline   the same workload through the host-CPU PyTorch path
+                 (grid_sample + softmax, oracle/torch_eager.py), same run
+
+Per-workload details (forward alone, backward alone, all five shapes with --all)
+go to stderr and, as JSON, to gpurun_out/bench_details.json when that folder exists.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "fused-deform-multi-head-scaled-dot-product-attention-triton_amd")
+for _p in (ROOT, PKG):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0     # MI355X published HBM3E bandwidth
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def load_traffic(workload, which):
+    """Measured HBM bytes per launch from profiles/hbm_traffic.json (rocprofv3 --pmc runs), or None."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(workload, {}).get(which)
+    except (OSError, ValueError):
+        return None
+
+
+def measure_gpu(wl, steps, warmup):
+    import torch
+    from ops import _native
+    from ops.triton import deform_sdpa_triton
+    from workloads import gen_inputs
+
+    dev = torch.device("cuda:0")
+    q, k, v, coords, dout = gen_inputs(wl, device=dev)
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    W, Hh, scale = wl.W_IMG, wl.H_IMG, wl.sm_scale
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        out = deform_sdpa_triton(q, k, v, coords, W, Hh, scale)
+        out.backward(dout)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _native.timer_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    _native.timer_enable(False)
+    fwd_ms, fwd_n = _native.timer_collect(0)
+    bwd_ms, bwd_n = _native.timer_collect(1)
+    ms_step = (t1 - t0) * 1e3 / steps
+
+    # forward alone (no autograd graph), timed separately
+    with torch.no_grad():
+        for _ in range(max(2, warmup // 2)):
+            deform_sdpa_triton(q, k, v, coords, W, Hh, scale)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            deform_sdpa_triton(q, k, v, coords, W, Hh, scale)
+        torch.cuda.synchronize()
+        fwd_only_ms = (time.perf_counter() - t0) * 1e3 / steps
+
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    step()
+    torch.cuda.synchronize()
+    peak_extra = torch.cuda.max_memory_allocated() - base
+    return {
+        "ms_per_step": ms_step,
+        "fwd_only_ms": fwd_only_ms,
+        "fwd_kernel_ms": fwd_ms / max(fwd_n, 1),
+        "bwd_kernel_ms": bwd_ms / max(bwd_n, 1),
+        "kernel_launches": [fwd_n, bwd_n],
+        "peak_extra_bytes": int(peak_extra),
+    }
+
+
+def measure_cpu(wl, budget_s=25.0):
+    """Host-CPU PyTorch path on the same workload; bounded to about budget_s seconds."""
+    import torch
+    from oracle.torch_eager import eager_fwd_bwd
+    from workloads import gen_inputs
+
+    q, k, v, coords, dout = gen_inputs(wl)
+    threads = torch.get_num_threads()
+    chunked = wl.query_samples * wl.D * 8 > 8e9       # sampled K~+V~ above 8 GB: one (b, h) at a time
+    f = lambda: eager_fwd_bwd(q.float(), k.float(), v.float(), coords, dout.float(),
+                              wl.W_IMG, wl.H_IMG, wl.sm_scale, chunked=chunked)
+    t0 = time.perf_counter()
+    f()                                                # warm-up
+    warm = time.perf_counter() - t0
+    reps = int(max(1, min(5, (budget_s - warm) // max(warm, 1e-3))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        f()
+    dt = (time.perf_counter() - t0) / reps
+    return {
+        "value": wl.query_samples / dt / 1e6,
+        "unit": "M query*samples/s (fwd+bwd)",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{wl.name} full workload, fwd+bwd, 1 warm-up + {reps} timed reps, "
+                  f"{dt * 1e3:.0f} ms/step, os.cpu_count()={os.cpu_count()}"
+                  + (", chunked over (batch, head)" if chunked else ""),
+        "ms_per_step": dt * 1e3,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="C2")
+    ap.add_argument("--all", action="store_true", help="also report the other workloads on stderr")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build targets one GPU; run with --gpus 1 "
+                 "(the operator shards over (batch, head) with no exchange, see DESIGN.md)")
+
+    from workloads import WORKLOADS
+    wl = WORKLOADS[args.workload]
+    g = measure_gpu(wl, args.steps, args.warmup)
+    qs = wl.query_samples
+    value = qs / (g["ms_per_step"] * 1e-3) / 1e6
+
+    dominant = "bwd" if g["bwd_kernel_ms"] >= g["fwd_kernel_ms"] else "fwd"
+    dom_ms = g[dominant + "_kernel_ms"]
+    dom_bytes = wl.algorithmic_bytes(dominant)
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBS, "traffic": load_traffic(wl.name, dominant),
+        "algorithmic_bytes": dom_bytes, "kernel_ms": dom_ms,
+    }
+    other = "fwd" if dominant == "bwd" else "bwd"
+    oth_bytes = wl.algorithmic_bytes(other)
+    oth_ach = oth_bytes / (g[other + "_kernel_ms"] * 1e-3) / 1e9
+    details = {
+        "workload": wl.name, "query_samples": qs, **g,
+        "fwd_only_MQS_per_s": qs / (g["fwd_only_ms"] * 1e-3) / 1e6,
+        "roofline_" + other: {"achieved": oth_ach, "frac": oth_ach / HBM_PEAK_GBS,
+                              "algorithmic_bytes": oth_bytes, "kernel_ms": g[other + "_kernel_ms"]},
+        "fwd_bwd_kernels_frac_of_roofline":
+            wl.algorithmic_bytes("fwd+bwd") / ((g["fwd_kernel_ms"] + g["bwd_kernel_ms"]) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+    }
+    log("[bench]", json.dumps(details))
+
+    all_details = {wl.name: details}
+    if args.all:
+        for name, w in WORKLOADS.items():
+            if name == wl.name:
+                continue
+            gg = measure_gpu(w, max(5, args.steps // 5), max(2, args.warmup // 2))
+            d = {"workload": name, "query_samples": w.query_samples, **gg,
+                 "MQS_per_s": w.query_samples / (gg["ms_per_step"] * 1e-3) / 1e6,
+                 "fwd_frac": w.algorithmic_bytes("fwd") / (gg["fwd_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                 "bwd_frac": w.algorithmic_bytes("bwd") / (gg["bwd_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            log("[bench]", json.dumps(d))
+            all_details[name] = d
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = measure_cpu(wl)
+        log("[bench] cpu baseline", json.dumps(cpu))
+
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, "bench_details.json"), "w") as f:
+            json.dump({"gpu": all_details, "cpu": cpu}, f, indent=1)
+
+    line = {
+        "metric": "fused fwd+bwd M query*samples/s (and % of HBM roofline), 1xMI355X vs host-CPU torch",
+        "value": value, "unit": "M query*samples/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": g["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32" if wl.dtype == "fp32" else wl.dtype, "data": "synthetic",
+        "config": {"workload": f"{wl.name}: B{wl.B} V{wl.V} H{wl.H} D{wl.D} {wl.H_IMG}x{wl.W_IMG} P{wl.P} "
+                               f"{wl.dtype} coords={wl.coords}, fwd+bwd through the autograd operator",
+                   "query_samples_per_step": qs,
+                   "fwd_only_ms": g["fwd_only_ms"], "fwd_kernel_ms": g["fwd_kernel_ms"],
+                   "bwd_kernel_ms": g["bwd_kernel_ms"], "peak_extra_bytes": g["peak_extra_bytes"]},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -5,9 +5,12 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <mutex>
+#include <vector>
 
 #include "dsdpa_common.h"
 #include "dsdpa_gather.h"
+#include "dsdpa_tile.h"
 
 using namespace dsdpa;
 
@@ -15,6 +18,38 @@ namespace {
 
 thread_local int g_last_hip_error = 0;
 std::atomic<int> g_path{DSDPA_PATH_AUTO};
+
+// Optional kernel timer: while enabled, every main forward/backward kernel
+// launch is bracketed by a pair of HIP events on the launch stream. Process-wide
+// (a framework may run the backward pass on another thread than the forward).
+struct EventPair { hipEvent_t start, stop; };
+struct KernelTimer {
+    std::atomic<bool> on{false};
+    std::mutex mu;
+    std::vector<EventPair> pairs[2];   // [0] forward kernels, [1] backward kernels
+};
+KernelTimer g_timer;
+
+struct ScopedKernelTimer {
+    hipStream_t st;
+    EventPair ev{nullptr, nullptr};
+    int which;
+    bool armed = false;
+    ScopedKernelTimer(int which_, hipStream_t st_) : st(st_), which(which_)
+    {
+        if (!g_timer.on.load(std::memory_order_relaxed)) return;
+        if (hipEventCreate(&ev.start) != hipSuccess) return;
+        if (hipEventCreate(&ev.stop) != hipSuccess) { (void)hipEventDestroy(ev.start); return; }
+        armed = hipEventRecord(ev.start, st) == hipSuccess;
+    }
+    ~ScopedKernelTimer()
+    {
+        if (!armed) return;
+        (void)hipEventRecord(ev.stop, st);
+        std::lock_guard<std::mutex> lock(g_timer.mu);
+        g_timer.pairs[which].push_back(ev);
+    }
+};
 
 // ------------------------------------------------------------------ small kernels
 __global__ void fill_zero_kernel(float4 *__restrict__ p, size_t n4)
@@ -78,6 +113,7 @@ int launch_fwd_gather(const void *q, const void *k, const void *v, const float *
 {
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
+    ScopedKernelTimer timer(0, st);
     hipLaunchKernelGGL((fwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                        q, k, v, coords, out, lse, dm);
     return check_launch();
@@ -90,8 +126,82 @@ int launch_bwd_gather(const void *q, const void *k, const void *v, const float *
 {
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
+    ScopedKernelTimer timer(1, st);
     hipLaunchKernelGGL((bwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                        q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm);
+    return check_launch();
+}
+
+template <typename S, int D>
+int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const float *coords, const void *out,
+                         const float *lse, const void *dout, void *dq, float *delta, const Dims &dm,
+                         hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
+    hipLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                       q, k, v, coords, out, lse, dout, dq, delta, dm);
+    return check_launch();
+}
+
+constexpr int kLdsBytes = 160 * 1024;                                   // LDS per workgroup on gfx950
+constexpr int kTileDescBytes = kTileWaves * kWave * (16 + 16 + 4);      // per-wave tap descriptors
+
+// Tile geometry for the dk/dv kernel: as few tiles per plane as the LDS budget allows
+// (every tile costs one more pass over the plane's coordinates and one halo ring).
+TileGeom make_tile_geom(const Dims &dm, int D)
+{
+    const int maxpx = (kLdsBytes - kTileDescBytes) / (2 * (int)sizeof(double) * D);   // dK + dV, fp64
+    const int Hh = dm.Himg, Ww = dm.Wimg;
+    auto ceil_div = [](int a, int b) { return (a + b - 1) / b; };
+    // option A: full-width row bands
+    int a_nty = 1 << 30, a_th = 0;
+    if (Ww * 2 <= maxpx || Hh * Ww <= maxpx) {
+        const int rows = maxpx / Ww;                       // rows of pixels that fit
+        const int th_max = rows >= Hh ? Hh : rows - 1;     // one halo row unless the whole image fits
+        a_nty = ceil_div(Hh, th_max);
+        a_th = ceil_div(Hh, a_nty);
+    }
+    // option B: square-ish 2-D tiles
+    int side = 2;
+    while ((side + 1) * (side + 1) <= maxpx) ++side;
+    const int cells = side - 1 > 0 ? side - 1 : 1;
+    const int b_nty = ceil_div(Hh, cells), b_ntx = ceil_div(Ww, cells);
+    TileGeom tg;
+    if (a_nty <= b_nty * b_ntx) {
+        tg.th = a_th; tg.tw = Ww; tg.nty = a_nty; tg.ntx = 1;
+    } else {
+        tg.th = ceil_div(Hh, b_nty); tg.tw = ceil_div(Ww, b_ntx); tg.nty = b_nty; tg.ntx = b_ntx;
+    }
+    tg.lh = tg.nty == 1 ? Hh : tg.th + 1;
+    tg.lw = tg.ntx == 1 ? Ww : tg.tw + 1;
+    const long long groups = (long long)dm.B * dm.H * dm.V * tg.nty * tg.ntx;
+    long long qsplit = (1024 + groups - 1) / groups;
+    const long long max_split = ((long long)dm.V * dm.L + 63) / 64;    // keep >= 64 query rows per workgroup
+    if (qsplit > max_split) qsplit = max_split;
+    if (qsplit < 1) qsplit = 1;
+    tg.qsplit = (int)qsplit;
+    return tg;
+}
+
+template <typename S, int D>
+int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const float *coords, const float *lse,
+                         const float *delta, const void *dout, float *dk_acc, float *dv_acc, const Dims &dm,
+                         hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const TileGeom tg = make_tile_geom(dm, D);
+    const size_t smem = (size_t)2 * sizeof(double) * tg.lh * tg.lw * D + kTileDescBytes;
+    if (smem > (size_t)kLdsBytes) return DSDPA_ERR_TOO_LARGE;
+    const long long blocks = (long long)dm.B * dm.H * dm.V * tg.nty * tg.ntx * tg.qsplit;
+    if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+    auto kern = bwd_dkdv_tile_kernel<S, D, DC>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    ScopedKernelTimer timer(1, st);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kTileWaves * kWave), smem, st,
+                       q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, tg);
     return check_launch();
 }
 
@@ -124,18 +234,22 @@ int zero_fill(float *p, size_t n, hipStream_t st)   // n is a multiple of 4 (D >
     return check_launch();
 }
 
+// workspace: [delta: rows floats, rounded up to 256 bytes][dk_acc, dv_acc: 2*n floats, 16-bit storage only]
+size_t delta_bytes(size_t rows) { return (rows * sizeof(float) + 255) / 256 * 256; }
+
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
              const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,
              int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
 {
-    if (!q || !k || !v || !coords || !out || !lse || !dout || !dq || !dk || !dv) return DSDPA_ERR_NULL_POINTER;
-    if (S::kBytes != 4 && !workspace) return DSDPA_ERR_NULL_POINTER;
+    if (!q || !k || !v || !coords || !out || !lse || !dout || !dq || !dk || !dv || !workspace)
+        return DSDPA_ERR_NULL_POINTER;
     Dims dm;
     int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
     if (rc != DSDPA_OK) return rc;
     hipStream_t st = (hipStream_t)stream;
     const size_t n = (size_t)dm.rows * D;
+    float *delta = (float *)workspace;
     float *dk_acc, *dv_acc;
     if (S::kBytes == 4) {
         dk_acc = (float *)dk;
@@ -143,18 +257,30 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
         if ((rc = zero_fill(dk_acc, n, st)) != DSDPA_OK) return rc;
         if ((rc = zero_fill(dv_acc, n, st)) != DSDPA_OK) return rc;
     } else {
-        dk_acc = (float *)workspace;
+        dk_acc = (float *)((char *)workspace + delta_bytes(dm.rows));
         dv_acc = dk_acc + n;
         if ((rc = zero_fill(dk_acc, 2 * n, st)) != DSDPA_OK) return rc;
     }
+    const bool fused_atomics = g_path.load() == DSDPA_PATH_GATHER;
+#define DSDPA_BWD_CASE(DD)                                                                                      \
+    case DD:                                                                                                    \
+        if (fused_atomics) {                                                                                    \
+            rc = launch_bwd_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st);         \
+        } else {                                                                                                \
+            rc = launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dm, st);               \
+            if (rc == DSDPA_OK)                                                                                 \
+                rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, st);    \
+        }                                                                                                       \
+        break;
     switch (D) {
-    case 16: rc = launch_bwd_gather<S, 16>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st); break;
-    case 32: rc = launch_bwd_gather<S, 32>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st); break;
-    case 64: rc = launch_bwd_gather<S, 64>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st); break;
-    case 128: rc = launch_bwd_gather<S, 128>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st); break;
-    case 256: rc = launch_bwd_gather<S, 256>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st); break;
+        DSDPA_BWD_CASE(16)
+        DSDPA_BWD_CASE(32)
+        DSDPA_BWD_CASE(64)
+        DSDPA_BWD_CASE(128)
+        DSDPA_BWD_CASE(256)
     default: return DSDPA_ERR_HEAD_DIM;
     }
+#undef DSDPA_BWD_CASE
     if (rc != DSDPA_OK) return rc;
     if (S::kBytes != 4) {
         const size_t n8 = n / 8;
@@ -216,10 +342,12 @@ int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coor
 
 size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D)
 {
-    if (dtype == DSDPA_F32) return 0;
-    if (dtype != DSDPA_BF16 && dtype != DSDPA_F16) return 0;
+    if (dtype != DSDPA_F32 && dtype != DSDPA_BF16 && dtype != DSDPA_F16) return 0;
     if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || D < 1) return 0;
-    return (size_t)2 * sizeof(float) * (size_t)B * V * H * (size_t)Himg * Wimg * D;
+    const size_t rows = (size_t)B * V * H * (size_t)Himg * Wimg;
+    size_t bytes = delta_bytes(rows);
+    if (dtype != DSDPA_F32) bytes += (size_t)2 * sizeof(float) * rows * D;
+    return bytes;
 }
 
 const char *dsdpa_error_string(int code)
@@ -239,6 +367,34 @@ const char *dsdpa_error_string(int code)
 int dsdpa_last_hip_error(void) { return g_last_hip_error; }
 
 int dsdpa_version(void) { return 100; }
+
+int dsdpa_timer_enable(int on)
+{
+    return g_timer.on.exchange(on != 0) ? 1 : 0;
+}
+
+int dsdpa_timer_collect(int which, double *total_ms, int *launches)
+{
+    if (which < 0 || which > 1 || !total_ms || !launches) return DSDPA_ERR_NULL_POINTER;
+    double sum = 0.0;
+    int n = 0, rc = DSDPA_OK;
+    std::vector<EventPair> taken;
+    {
+        std::lock_guard<std::mutex> lock(g_timer.mu);
+        taken.swap(g_timer.pairs[which]);
+    }
+    for (EventPair &ev : taken) {
+        float ms = 0.f;
+        hipError_t e = hipEventSynchronize(ev.stop);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, ev.start, ev.stop);
+        if (e == hipSuccess) { sum += ms; ++n; } else { g_last_hip_error = (int)e; rc = DSDPA_ERR_HIP; }
+        (void)hipEventDestroy(ev.start);
+        (void)hipEventDestroy(ev.stop);
+    }
+    *total_ms = sum;
+    *launches = n;
+    return rc;
+}
 
 int dsdpa_set_path(int path)
 {

@@ -122,6 +122,7 @@ __device__ __forceinline__ void store_chunk(void *p, const float (&src)[DC])
 struct Taps {
     float w[4];     // 00 (row0,col0), 01 (row0,col1), 10, 11
     int pix[4];     // row*W + col, always inside [0, L)
+    int x0, y0;     // floor of the pixel coordinate, limited to [-2, size+1] (not clamped into the image)
 };
 
 __device__ __forceinline__ Taps make_taps(float cx, float cy, int Wimg, int Himg)
@@ -150,6 +151,8 @@ __device__ __forceinline__ Taps make_taps(float cx, float cy, int Wimg, int Himg
     t.pix[1] = cy0 * Wimg + cx1;
     t.pix[2] = cy1 * Wimg + cx0;
     t.pix[3] = cy1 * Wimg + cx1;
+    t.x0 = x0;
+    t.y0 = y0;
     return t;
 }
 

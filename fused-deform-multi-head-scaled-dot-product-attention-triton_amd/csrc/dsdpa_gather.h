@@ -289,4 +289,85 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_gather_kernel(
     }
 }
 
+// ------------------------------------------------------------------ backward, dq only
+// Same walk as bwd_gather_kernel without the dk/dv scatter: writes dq and the
+// per-row delta = dout.out (consumed by the tile kernel that produces dk/dv).
+template <typename S, int D, int DC>
+__global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
+    const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
+    const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
+    const void *__restrict__ dout_, void *__restrict__ dq_, float *__restrict__ delta_, Dims dm)
+{
+    constexpr int G = D / DC;
+    constexpr int NS = kWave / G;
+    constexpr int ITS = G;
+    static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
+    __shared__ float4 s_w[kGatherWaves][kWave];
+    __shared__ int4 s_e[kGatherWaves][kWave];
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
+    if (work >= dm.rows) return;
+    const RowCtx rc = decode_row(work, dm, D);
+    const int g = lane % G, slot = lane / G, lane_elem = g * DC;
+    const char *kb = (const char *)k_ + rc.kv_base * S::kBytes;
+    const char *vb = (const char *)v_ + rc.kv_base * S::kBytes;
+    const float2 *coords = (const float2 *)coords_;
+
+    float qf[DC], dof[DC], of[DC];
+    const size_t roff = (rc.row * D + lane_elem) * S::kBytes;
+    load_chunk<S, DC>((const char *)q_ + roff, qf);
+    load_chunk<S, DC>((const char *)dout_ + roff, dof);
+    load_chunk<S, DC>((const char *)out_ + roff, of);
+    float delta = 0.f;
+#pragma unroll
+    for (int d = 0; d < DC; ++d) delta = fmaf(dof[d], of[d], delta);
+    delta = group_sum<G>(delta);
+    if (lane == 0) delta_[rc.row] = delta;
+    const float qscale = dm.sm_scale * kLog2e;
+    const float lse = lse_[rc.row];
+
+    float dqa[DC];
+#pragma unroll
+    for (int d = 0; d < DC; ++d) dqa[d] = 0.f;
+
+    for (int c0 = 0; c0 < dm.N; c0 += kWave) {
+        stage_descriptors<D>(coords, rc, dm, c0, lane, s_w[wave], s_e[wave]);
+        const int cnt = min(kWave, dm.N - c0);
+#pragma unroll
+        for (int it = 0; it < ITS; ++it) {
+            if (it * NS < cnt) {
+                int j = it * NS + slot;
+                float4 w = s_w[wave][j];
+                int4 e = s_e[wave][j];
+                float kk[DC], vv[DC];
+                blend_taps<S, DC>(kb, e, w, lane_elem, kk);
+                blend_taps<S, DC>(vb, e, w, lane_elem, vv);
+                float dot = 0.f, dp = 0.f;
+#pragma unroll
+                for (int d = 0; d < DC; ++d) {
+                    dot = fmaf(qf[d], kk[d], dot);
+                    dp = fmaf(dof[d], vv[d], dp);
+                }
+                dot = group_sum<G>(dot);
+                dp = group_sum<G>(dp);
+                float p = (j < cnt) ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
+                float ds = p * (dp - delta);
+#pragma unroll
+                for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
+            }
+        }
+    }
+#pragma unroll
+    for (int off = G; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int d = 0; d < DC; ++d) dqa[d] += __shfl_xor(dqa[d], off, kWave);
+    }
+    if (slot == 0) {
+#pragma unroll
+        for (int d = 0; d < DC; ++d) dqa[d] *= dm.sm_scale;
+        store_chunk<S, DC>((char *)dq_ + roff, dqa);
+    }
+}
+
 }  // namespace dsdpa

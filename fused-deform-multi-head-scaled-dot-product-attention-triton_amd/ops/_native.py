@@ -15,7 +15,7 @@ SYMBOLS = (
     "dsdpa_fwd_f32", "dsdpa_fwd_bf16", "dsdpa_fwd_f16",
     "dsdpa_bwd_f32", "dsdpa_bwd_bf16", "dsdpa_bwd_f16",
     "dsdpa_bwd_workspace_bytes", "dsdpa_error_string", "dsdpa_last_hip_error",
-    "dsdpa_version", "dsdpa_set_path",
+    "dsdpa_version", "dsdpa_set_path", "dsdpa_timer_enable", "dsdpa_timer_collect",
 )
 
 DSDPA_F32, DSDPA_BF16, DSDPA_F16 = 0, 1, 2
@@ -57,6 +57,10 @@ def load():
     lib.dsdpa_version.restype = i
     lib.dsdpa_set_path.argtypes = [i]
     lib.dsdpa_set_path.restype = i
+    lib.dsdpa_timer_enable.argtypes = [i]
+    lib.dsdpa_timer_enable.restype = i
+    lib.dsdpa_timer_collect.argtypes = [i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(i)]
+    lib.dsdpa_timer_collect.restype = i
     _lib = lib
     return lib
 
@@ -74,3 +78,15 @@ def set_path(path):
     if prev < 0:
         raise ValueError(f"unknown kernel path {path}")
     return prev
+
+
+def timer_enable(on):
+    """Bracket every main fwd/bwd kernel launch (process-wide) with HIP events; returns the previous state."""
+    return load().dsdpa_timer_enable(1 if on else 0)
+
+
+def timer_collect(which):
+    """(total kernel ms, launches) of the events recorded since the last collect; which: 0 fwd, 1 bwd."""
+    ms, n = ctypes.c_double(0.0), ctypes.c_int(0)
+    check(load().dsdpa_timer_collect(int(which), ctypes.byref(ms), ctypes.byref(n)))
+    return ms.value, n.value

@@ -28,7 +28,8 @@
  *     all work is enqueued on it and the call returns without synchronising;
  *   - D (head dim) must be one of 16, 32, 64, 128, 256 (ops/triton.py:386);
  *   - every entry point returns 0 on success or a DSDPA_ERR_* code, never
- *     throws, and is re-entrant (no global mutable state).
+ *     throws, and is re-entrant; the only process-wide state is the kernel-path
+ *     selector (dsdpa_set_path) and the optional kernel timer.
  */
 #ifndef DSDPA_H
 #define DSDPA_H
@@ -79,10 +80,11 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
  * fp32 -> storage casts of dk/dv (:461-462).
  *
  * dq, dk, dv are fully overwritten (no pre-zeroing by the caller needed).
- * fp32: dk and dv are themselves the accumulators; `workspace` may be NULL.
- * bf16/fp16: `workspace` must hold dsdpa_bwd_workspace_bytes(...) bytes; it
- * carries the fp32 dk/dv accumulators that are rounded to the storage type at
- * the end. Accumulation order into dk/dv is not deterministic (float atomics,
+ * `workspace` must hold dsdpa_bwd_workspace_bytes(...) bytes (256-byte aligned):
+ * the per-row delta = dout.out (one float per query row, the reference's `delta`,
+ * ops/triton.py:430) and, for bf16/fp16, the fp32 dk/dv accumulators that are
+ * rounded to the storage type at the end (fp32: dk and dv are themselves the
+ * accumulators). Accumulation order into dk/dv is not deterministic (float atomics,
  * as in the reference, ops/triton.py:345-360).
  */
 int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords,
@@ -101,8 +103,8 @@ int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coor
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
                   float sm_scale, void *stream);
 
-/* Bytes of device workspace dsdpa_bwd_* needs for a storage dtype (0 for fp32).
- * Counterpart of the reference's dk32/dv32 temporaries, ops/triton.py:428-429. */
+/* Bytes of device workspace dsdpa_bwd_* needs for a storage dtype (0 if an argument is invalid).
+ * Counterpart of the reference's delta and dk32/dv32 temporaries, ops/triton.py:428-430. */
 size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D);
 
 /* Human-readable text for a DSDPA_ERR_* code. */
@@ -122,6 +124,18 @@ int dsdpa_version(void);
  */
 enum { DSDPA_PATH_AUTO = 0, DSDPA_PATH_GATHER = 1, DSDPA_PATH_LDS = 2 };
 int dsdpa_set_path(int path);
+
+/*
+ * Kernel timer, for measurement (the reference times whole calls with
+ * triton.testing.do_bench, benchmark.py:90). While enabled (process-wide),
+ * every main forward / backward kernel launch is bracketed by a pair of
+ * HIP events recorded on the launch stream. dsdpa_timer_collect waits for the
+ * recorded events, returns the summed kernel time and the number of launches
+ * for `which` (0 = forward kernels, 1 = backward kernels) and releases them.
+ * dsdpa_timer_enable returns the previous state.
+ */
+int dsdpa_timer_enable(int on);
+int dsdpa_timer_collect(int which, double *total_ms, int *launches);
 
 #ifdef __cplusplus
 }

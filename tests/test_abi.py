@@ -38,10 +38,16 @@ def test_version_and_error_strings():
 
 def test_workspace_bytes():
     lib = _native.load()
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32) == 0
-    n = 2 * 6 * 8 * 48 * 48 * 64
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64) == 8 * n
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F16, 2, 6, 8, 48, 48, 64) == 8 * n
+    def delta_bytes(rows):
+        return (rows * 4 + 255) // 256 * 256
+    rows = 2 * 6 * 8 * 18 * 18
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32) == delta_bytes(rows)
+    rows = 2 * 6 * 8 * 48 * 48
+    n = rows * 64
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64) == 8 * n + delta_bytes(rows)
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F16, 2, 6, 8, 48, 48, 64) == 8 * n + delta_bytes(rows)
+    assert lib.dsdpa_bwd_workspace_bytes(7, 2, 6, 8, 48, 48, 64) == 0
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 0, 6, 8, 48, 48, 64) == 0
 
 
 def test_argument_validation_before_launch():
@@ -54,11 +60,12 @@ def test_argument_validation_before_launch():
     assert lib.dsdpa_fwd_bf16(fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 48, 2, 0.5, None) == 3
     assert lib.dsdpa_fwd_f16(fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 8, 2, 0.5, None) == 3
     assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, 1, 64, 64, 1024, 1024, 256, 2, 0.5, None) == 4
-    # backward: 16-bit storage needs a workspace
+    # backward: the workspace is required
     args = [fake] * 10
     assert lib.dsdpa_bwd_bf16(*args, None, *ok_dims) == 1
-    assert lib.dsdpa_bwd_f32(*args[:9], None, None, *ok_dims) == 1
-    assert lib.dsdpa_bwd_f32(*args, None, 1, 2, 2, 3, 4, 33, 2, 0.5, None) == 3
+    assert lib.dsdpa_bwd_f32(*args, None, *ok_dims) == 1
+    assert lib.dsdpa_bwd_f32(*args[:9], None, fake, *ok_dims) == 1
+    assert lib.dsdpa_bwd_f32(*args, fake, 1, 2, 2, 3, 4, 33, 2, 0.5, None) == 3
 
 
 def test_path_selector():
