@@ -11,6 +11,7 @@
 #include "dsdpa_common.h"
 #include "dsdpa_gather.h"
 #include "dsdpa_tile.h"
+#include "dsdpa_cell.h"
 
 using namespace dsdpa;
 
@@ -234,8 +235,69 @@ int zero_fill(float *p, size_t n, hipStream_t st)   // n is a multiple of 4 (D >
     return check_launch();
 }
 
-// workspace: [delta: rows floats, rounded up to 256 bytes][dk_acc, dv_acc: 2*n floats, 16-bit storage only]
-size_t delta_bytes(size_t rows) { return (rows * sizeof(float) + 255) / 256 * 256; }
+// Backward workspace, every segment rounded up to 256 bytes:
+//   delta    rows floats                     dout.out per query row
+//   counters B*V*NC u32                      per (batch, key view) cell counts, then fill cursors
+//   start    B*V*(NC+1) u32                  exclusive scan of the counts
+//   sorted   B*V*(V*L*P) u32                 sample ids ordered by cell
+//   acc      2*n floats                      fp32 dk/dv accumulators (16-bit storage only)
+// with NC = (Himg+1)*(Wimg+1) cells.
+size_t round256(size_t b) { return (b + 255) / 256 * 256; }
+struct WorkspaceLayout {
+    size_t delta, counters, start, sorted, acc, total;
+    size_t counters_bytes;
+    int NC;
+};
+WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Himg, size_t Wimg, size_t D, size_t P,
+                                 bool storage16)
+{
+    WorkspaceLayout w;
+    const size_t rows = B * V * H * Himg * Wimg;
+    w.NC = (int)((Himg + 1) * (Wimg + 1));
+    size_t off = 0;
+    w.delta = off; off += round256(rows * 4);
+    w.counters = off; w.counters_bytes = round256(B * V * (size_t)w.NC * 4); off += w.counters_bytes;
+    w.start = off; off += round256(B * V * ((size_t)w.NC + 1) * 4);
+    w.sorted = off; off += round256(B * V * (V * Himg * Wimg * P) * 4);
+    w.acc = off; if (storage16) off += round256(2 * rows * D * 4);
+    w.total = off;
+    return w;
+}
+
+template <typename S, int D> struct CellChunk {
+    static constexpr int value = Chunk<S, D>::value > 8 ? 8 : Chunk<S, D>::value;
+};
+
+int launch_binning(const float *coords, const Dims &dm, const WorkspaceLayout &wl, char *ws, hipStream_t st)
+{
+    unsigned *counters = (unsigned *)(ws + wl.counters);
+    unsigned *start = (unsigned *)(ws + wl.start);
+    unsigned *sorted = (unsigned *)(ws + wl.sorted);
+    const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
+    const long long blocks = (total + kBinThreads - 1) / kBinThreads;
+    if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(bin_samples_kernel<0>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
+                       coords, dm, wl.NC, counters, sorted);
+    hipLaunchKernelGGL(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st, counters, start, wl.NC);
+    hipLaunchKernelGGL(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
+                       coords, dm, wl.NC, counters, sorted);
+    return check_launch();
+}
+
+template <typename S, int D>
+int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const float *coords, const float *lse,
+                         const float *delta, const void *dout, const unsigned *start, const unsigned *sorted,
+                         float *dk_acc, float *dv_acc, const Dims &dm, int NC, hipStream_t st)
+{
+    constexpr int DC = CellChunk<S, D>::value;
+    const long long nwork = (long long)dm.B * dm.H * dm.V * NC;
+    const long long blocks = (nwork + kCellWaves - 1) / kCellWaves;
+    if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+    ScopedKernelTimer timer(1, st);
+    hipLaunchKernelGGL((bwd_dkdv_cell_kernel<S, D, DC>), dim3((unsigned)blocks), dim3(kCellWaves * kWave), 0, st,
+                       q, k, v, coords, lse, delta, dout, start, sorted, dk_acc, dv_acc, dm, NC);
+    return check_launch();
+}
 
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
@@ -247,9 +309,12 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     Dims dm;
     int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
     if (rc != DSDPA_OK) return rc;
+    if ((long long)dm.L * dm.N > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;   // sample ids are 32-bit
     hipStream_t st = (hipStream_t)stream;
     const size_t n = (size_t)dm.rows * D;
-    float *delta = (float *)workspace;
+    const WorkspaceLayout wl = workspace_layout(B, V, H, Himg, Wimg, D, P, S::kBytes != 4);
+    char *ws = (char *)workspace;
+    float *delta = (float *)(ws + wl.delta);
     float *dk_acc, *dv_acc;
     if (S::kBytes == 4) {
         dk_acc = (float *)dk;
@@ -257,18 +322,29 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
         if ((rc = zero_fill(dk_acc, n, st)) != DSDPA_OK) return rc;
         if ((rc = zero_fill(dv_acc, n, st)) != DSDPA_OK) return rc;
     } else {
-        dk_acc = (float *)((char *)workspace + delta_bytes(dm.rows));
+        dk_acc = (float *)(ws + wl.acc);
         dv_acc = dk_acc + n;
         if ((rc = zero_fill(dk_acc, 2 * n, st)) != DSDPA_OK) return rc;
     }
-    const bool fused_atomics = g_path.load() == DSDPA_PATH_GATHER;
+    const int path = g_path.load();
+    const bool fused_atomics = path == DSDPA_PATH_GATHER;
+    const bool cell_binned = path == DSDPA_PATH_AUTO;
+    const unsigned *start = (const unsigned *)(ws + wl.start);
+    const unsigned *sorted = (const unsigned *)(ws + wl.sorted);
+    if (cell_binned) {
+        if ((rc = zero_fill((float *)(ws + wl.counters), wl.counters_bytes / 4, st)) != DSDPA_OK) return rc;
+        if ((rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
+    }
 #define DSDPA_BWD_CASE(DD)                                                                                      \
     case DD:                                                                                                    \
         if (fused_atomics) {                                                                                    \
             rc = launch_bwd_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st);         \
         } else {                                                                                                \
             rc = launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dm, st);               \
-            if (rc == DSDPA_OK)                                                                                 \
+            if (rc == DSDPA_OK && cell_binned)                                                                  \
+                rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, lse, delta, dout, start, sorted, dk_acc,      \
+                                                 dv_acc, dm, wl.NC, st);                                        \
+            else if (rc == DSDPA_OK)                                                                            \
                 rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, st);    \
         }                                                                                                       \
         break;
@@ -340,14 +416,11 @@ int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coor
                          sm_scale, stream);
 }
 
-size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D)
+size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P)
 {
     if (dtype != DSDPA_F32 && dtype != DSDPA_BF16 && dtype != DSDPA_F16) return 0;
-    if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || D < 1) return 0;
-    const size_t rows = (size_t)B * V * H * (size_t)Himg * Wimg;
-    size_t bytes = delta_bytes(rows);
-    if (dtype != DSDPA_F32) bytes += (size_t)2 * sizeof(float) * rows * D;
-    return bytes;
+    if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || D < 1 || P < 1) return 0;
+    return workspace_layout(B, V, H, Himg, Wimg, D, P, dtype != DSDPA_F32).total;
 }
 
 const char *dsdpa_error_string(int code)

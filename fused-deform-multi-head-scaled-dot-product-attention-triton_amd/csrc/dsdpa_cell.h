@@ -1,0 +1,242 @@
+// Cell-binned dk/dv: scatter turned into register accumulation.
+//
+// A sample's four bilinear taps are the 2x2 pixel block whose top-left pixel is
+// (y0, x0) = floor of its pixel coordinate -- its "cell". Which cell a sample
+// falls in depends on the coordinates only, not on the head, so one counting
+// sort per (batch, key view) -- bin_count / bin_scan / bin_fill below -- orders
+// the samples (s1, l, p) of every key view by cell, and all H heads reuse it.
+//
+// The dk/dv kernel then gives one wave to one (plane (b, h, s2), cell): the
+// cell's four K and four V tap rows are loaded ONCE into registers; for every
+// sample in the cell's list the wave gathers the sample's query row (q, dout,
+// log-sum-exp, delta), recomputes p and ds, and adds w_t*ds*scale*q and
+// w_t*p*dout into register accumulators for the four pixels. Only the cell's
+// final sums go to memory: 8*D float atomics per non-empty cell instead of 8*D
+// per sample (each pixel is shared by four cells, hence atomics for that last
+// step). Heavy cells (clustered coordinates) are the best case, not the worst.
+//
+// Cells are indexed on a (Himg+1) x (Wimg+1) grid, y0 in [-1, Himg-1] and x0 in
+// [-1, Wimg-1]: border cells hold the samples with some taps outside the image
+// (weight 0 there, zero padding per tap). Samples with all four taps outside
+// contribute nothing to dk/dv and are left out of the lists.
+#pragma once
+#include "dsdpa_common.h"
+
+namespace dsdpa {
+
+constexpr int kBinThreads = 256;
+constexpr int kCellWaves = 4;
+
+__device__ __forceinline__ int cell_of(const Taps &tp, int Wimg) { return (tp.y0 + 1) * (Wimg + 1) + (tp.x0 + 1); }
+
+__device__ __forceinline__ bool taps_any(const Taps &tp)
+{
+    return (tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f);
+}
+
+// One thread per coordinate pair, in memory order (b, s1, l, s2, p).
+// mode 0: count[(b*V+s2)*NC + cell] += 1
+// mode 1: sorted[(b*V+s2)*M + cursor[(b*V+s2)*NC + cell]++] = (s1*L + l)*P + p
+template <int MODE>
+__global__ __launch_bounds__(kBinThreads) void bin_samples_kernel(const float *__restrict__ coords_, Dims dm,
+                                                                  int NC, unsigned *__restrict__ counters,
+                                                                  unsigned *__restrict__ sorted)
+{
+    const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
+    const long long i = (long long)blockIdx.x * kBinThreads + threadIdx.x;
+    if (i >= total) return;
+    const float2 xy = reinterpret_cast<const float2 *>(coords_)[i];
+    const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
+    if (!taps_any(tp)) return;
+    const int p = (int)(i % dm.P);
+    long long t = i / dm.P;
+    const int s2 = (int)(t % dm.V);
+    t /= dm.V;                                   // t = (b*V + s1)*L + l
+    const int ql = (int)(t % ((long long)dm.V * dm.L));   // s1*L + l
+    const int b = (int)(t / ((long long)dm.V * dm.L));
+    const size_t grp = (size_t)b * dm.V + s2;
+    unsigned *ctr = counters + grp * NC + cell_of(tp, dm.Wimg);
+    if (MODE == 0) {
+        atomicAdd(ctr, 1u);
+    } else {
+        const unsigned pos = atomicAdd(ctr, 1u);
+        const size_t M = (size_t)dm.V * dm.L * dm.P;
+        sorted[grp * M + pos] = (unsigned)ql * (unsigned)dm.P + (unsigned)p;
+    }
+}
+
+// One workgroup per (b, s2): exclusive scan of the NC cell counts. Writes
+// start[grp*(NC+1) + c] (with the total at c = NC) and resets counters to the
+// same starts, so that the fill pass can use them as cursors.
+__global__ __launch_bounds__(1024) void bin_scan_kernel(unsigned *__restrict__ counters,
+                                                        unsigned *__restrict__ start, int NC)
+{
+    __shared__ unsigned s_part[1024];
+    __shared__ unsigned s_carry;
+    unsigned *cnt = counters + (size_t)blockIdx.x * NC;
+    unsigned *st = start + (size_t)blockIdx.x * (NC + 1);
+    if (threadIdx.x == 0) s_carry = 0;
+    __syncthreads();
+    for (int base = 0; base < NC; base += 1024) {
+        const int c = base + threadIdx.x;
+        const unsigned v = c < NC ? cnt[c] : 0u;
+        s_part[threadIdx.x] = v;
+        __syncthreads();
+        for (int off = 1; off < 1024; off <<= 1) {             // Hillis-Steele inclusive scan
+            unsigned add = threadIdx.x >= (unsigned)off ? s_part[threadIdx.x - off] : 0u;
+            __syncthreads();
+            s_part[threadIdx.x] += add;
+            __syncthreads();
+        }
+        const unsigned excl = s_carry + s_part[threadIdx.x] - v;
+        if (c < NC) {
+            st[c] = excl;
+            cnt[c] = excl;
+        }
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry += s_part[1023];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) st[NC] = s_carry;
+}
+
+template <typename S, int DC>
+__device__ __forceinline__ void load_tap_or_zero(const char *base, int pix, int D, int lane_elem, bool valid,
+                                                 float (&dst)[DC])
+{
+    if (valid) {
+        load_chunk<S, DC>(base + ((size_t)pix * D + lane_elem) * S::kBytes, dst);
+    } else {
+#pragma unroll
+        for (int d = 0; d < DC; ++d) dst[d] = 0.f;
+    }
+}
+
+template <typename S, int D, int DC>
+__global__ __launch_bounds__(kCellWaves *kWave) void bwd_dkdv_cell_kernel(
+    const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
+    const float *__restrict__ coords_, const float *__restrict__ lse_, const float *__restrict__ delta_,
+    const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
+    float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC)
+{
+    constexpr int G = D / DC;
+    constexpr int NS = kWave / G;
+    static_assert(G >= 1 && G <= 64 && G * DC == D, "lane split");
+    __shared__ float4 s_w[kCellWaves][kWave];
+    __shared__ unsigned s_row[kCellWaves][kWave];
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const long long work = (long long)xcd_logical_block(blockIdx.x, gridDim.x) * kCellWaves + wave;
+    const long long nwork = (long long)dm.B * dm.H * dm.V * NC;
+    if (work >= nwork) return;
+    // plane-major: (b, h, s2, cell)
+    const int cell = (int)(work % NC);
+    long long t = work / NC;
+    const int s2 = (int)(t % dm.V);
+    t /= dm.V;
+    const int h = (int)(t % dm.H);
+    const int b = (int)(t / dm.H);
+    const size_t grp = (size_t)b * dm.V + s2;
+    const unsigned lo = start[grp * (NC + 1) + cell], hi = start[grp * (NC + 1) + cell + 1];
+    if (lo == hi) return;
+
+    const int g = lane % G, slot = lane / G, lane_elem = g * DC;
+    const int y0 = cell / (dm.Wimg + 1) - 1, x0 = cell % (dm.Wimg + 1) - 1;
+    const bool vy0 = y0 >= 0, vy1 = y0 + 1 < dm.Himg, vx0 = x0 >= 0, vx1 = x0 + 1 < dm.Wimg;
+    const bool tv[4] = { vy0 && vx0, vy0 && vx1, vy1 && vx0, vy1 && vx1 };
+    const int tpix[4] = { y0 * dm.Wimg + x0, y0 * dm.Wimg + x0 + 1, (y0 + 1) * dm.Wimg + x0,
+                          (y0 + 1) * dm.Wimg + x0 + 1 };
+    const size_t plane_base = ((grp * dm.H) + h) * (size_t)dm.L * D;          // elements; grp = b*V + s2
+    const char *kb = (const char *)k_ + plane_base * S::kBytes;
+    const char *vb = (const char *)v_ + plane_base * S::kBytes;
+    float kt[4][DC], vt[4][DC], aK[4][DC], aV[4][DC];
+#pragma unroll
+    for (int tpi = 0; tpi < 4; ++tpi) {
+        load_tap_or_zero<S, DC>(kb, tpix[tpi], D, lane_elem, tv[tpi], kt[tpi]);
+        load_tap_or_zero<S, DC>(vb, tpix[tpi], D, lane_elem, tv[tpi], vt[tpi]);
+#pragma unroll
+        for (int d = 0; d < DC; ++d) { aK[tpi][d] = 0.f; aV[tpi][d] = 0.f; }
+    }
+    const float qscale = dm.sm_scale * kLog2e;
+    const size_t M = (size_t)dm.V * dm.L * dm.P;
+    const unsigned *list = sorted + grp * M;
+    const float2 *coords = reinterpret_cast<const float2 *>(coords_);
+
+    for (unsigned c0 = lo; c0 < hi; c0 += kWave) {
+        // one list entry per lane: weights and query row
+        const unsigned idx = c0 + lane;
+        const bool in_range = idx < hi;
+        const unsigned id = list[in_range ? idx : hi - 1];
+        const unsigned p = id % (unsigned)dm.P, ql = id / (unsigned)dm.P;      // ql = s1*L + l
+        const unsigned s1 = ql / (unsigned)dm.L, l = ql % (unsigned)dm.L;
+        const size_t ci = ((((size_t)b * dm.V + s1) * dm.L + l) * dm.V + s2) * (size_t)dm.P + p;
+        const float2 xy = coords[ci];
+        const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
+        const unsigned row = (unsigned)((((size_t)b * dm.V + s1) * dm.H + h) * dm.L + l);
+        wave_lds_sync();
+        s_w[wave][lane] = make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]);
+        s_row[wave][lane] = row;
+        wave_lds_sync();
+        const int cnt = (int)min((unsigned)kWave, hi - c0);
+        for (int j0 = 0; j0 < cnt; j0 += NS) {
+            const int j = j0 + slot;
+            const bool live = j < cnt;
+            const int jj = live ? j : cnt - 1;
+            const float4 w = s_w[wave][jj];
+            const size_t r = s_row[wave][jj];
+            float qf[DC], dof[DC];
+            load_chunk<S, DC>((const char *)q_ + (r * D + lane_elem) * S::kBytes, qf);
+            load_chunk<S, DC>((const char *)dout_ + (r * D + lane_elem) * S::kBytes, dof);
+            const float lse = lse_[r], delta = delta_[r];
+            float dot = 0.f, dp = 0.f;
+#pragma unroll
+            for (int d = 0; d < DC; ++d) {
+                const float kk = fmaf(w.x, kt[0][d], fmaf(w.y, kt[1][d], fmaf(w.z, kt[2][d], w.w * kt[3][d])));
+                const float vv = fmaf(w.x, vt[0][d], fmaf(w.y, vt[1][d], fmaf(w.z, vt[2][d], w.w * vt[3][d])));
+                dot = fmaf(qf[d], kk, dot);
+                dp = fmaf(dof[d], vv, dp);
+            }
+            dot = group_sum<G>(dot);
+            dp = group_sum<G>(dp);
+            const float p_n = live ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
+            const float dss = p_n * (dp - delta) * dm.sm_scale;
+            const float ck[4] = { w.x * dss, w.y * dss, w.z * dss, w.w * dss };
+            const float cv[4] = { w.x * p_n, w.y * p_n, w.z * p_n, w.w * p_n };
+#pragma unroll
+            for (int tpi = 0; tpi < 4; ++tpi) {
+#pragma unroll
+                for (int d = 0; d < DC; ++d) {
+                    aK[tpi][d] = fmaf(ck[tpi], qf[d], aK[tpi][d]);
+                    aV[tpi][d] = fmaf(cv[tpi], dof[d], aV[tpi][d]);
+                }
+            }
+        }
+    }
+    // sum the NS slots, then one flush per pixel of the cell
+#pragma unroll
+    for (int off = G; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int tpi = 0; tpi < 4; ++tpi) {
+#pragma unroll
+            for (int d = 0; d < DC; ++d) {
+                aK[tpi][d] += __shfl_xor(aK[tpi][d], off, kWave);
+                aV[tpi][d] += __shfl_xor(aV[tpi][d], off, kWave);
+            }
+        }
+    }
+    if (slot == 0) {
+        float *dkb = dk_acc + plane_base + lane_elem, *dvb = dv_acc + plane_base + lane_elem;
+#pragma unroll
+        for (int tpi = 0; tpi < 4; ++tpi) {
+            if (tv[tpi]) {
+#pragma unroll
+                for (int d = 0; d < DC; ++d) {
+                    atomicAdd(dkb + (size_t)tpix[tpi] * D + d, aK[tpi][d]);
+                    atomicAdd(dvb + (size_t)tpix[tpi] * D + d, aV[tpi][d]);
+                }
+            }
+        }
+    }
+}
+
+}  // namespace dsdpa

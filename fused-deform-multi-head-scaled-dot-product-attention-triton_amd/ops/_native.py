@@ -47,7 +47,7 @@ def load():
         bwd = getattr(lib, "dsdpa_bwd_" + sfx)
         bwd.argtypes = [vp] * 11 + dims
         bwd.restype = i
-    lib.dsdpa_bwd_workspace_bytes.argtypes = [i] * 7
+    lib.dsdpa_bwd_workspace_bytes.argtypes = [i] * 8
     lib.dsdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.dsdpa_error_string.argtypes = [i]
     lib.dsdpa_error_string.restype = ctypes.c_char_p

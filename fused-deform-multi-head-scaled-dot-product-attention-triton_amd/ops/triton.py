@@ -97,13 +97,13 @@ class _fused_deform_sdpa(torch.autograd.Function):
         if do.dtype != q.dtype:
             do = do.to(q.dtype)
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-        ws_bytes = lib.dsdpa_bwd_workspace_bytes(_DTYPE_CODE[q.dtype], B, V, H, ctx.HEIGHT, ctx.WIDTH, D)
-        ws = torch.empty(ws_bytes // 4, device=q.device, dtype=torch.float32) if ws_bytes else None
+        ws_bytes = lib.dsdpa_bwd_workspace_bytes(_DTYPE_CODE[q.dtype], B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P)
+        ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
         with torch.cuda.device(q.device):
             rc = getattr(lib, "dsdpa_bwd_" + sfx)(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), coords.data_ptr(), out.data_ptr(), lse.data_ptr(),
                 do.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-                ws.data_ptr() if ws is not None else None,
+                ws.data_ptr(),
                 B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P, ctx.sm_scale, _stream_ptr(q.device))
         _native.check(rc)
         return dq, dk, dv, None, None, None, None

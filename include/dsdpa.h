@@ -82,9 +82,11 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
  * dq, dk, dv are fully overwritten (no pre-zeroing by the caller needed).
  * `workspace` must hold dsdpa_bwd_workspace_bytes(...) bytes (256-byte aligned):
  * the per-row delta = dout.out (one float per query row, the reference's `delta`,
- * ops/triton.py:430) and, for bf16/fp16, the fp32 dk/dv accumulators that are
- * rounded to the storage type at the end (fp32: dk and dv are themselves the
- * accumulators). Accumulation order into dk/dv is not deterministic (float atomics,
+ * ops/triton.py:430), the per-(batch, key view) ordering of the samples by
+ * bilinear cell (one u32 per coordinate pair plus the cell offsets; it depends on
+ * coords only and is shared by all heads) and, for bf16/fp16, the fp32 dk/dv
+ * accumulators that are rounded to the storage type at the end (fp32: dk and dv
+ * are themselves the accumulators). Accumulation order into dk/dv is not deterministic (float atomics,
  * as in the reference, ops/triton.py:345-360).
  */
 int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords,
@@ -105,7 +107,7 @@ int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coor
 
 /* Bytes of device workspace dsdpa_bwd_* needs for a storage dtype (0 if an argument is invalid).
  * Counterpart of the reference's delta and dk32/dv32 temporaries, ops/triton.py:428-430. */
-size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D);
+size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P);
 
 /* Human-readable text for a DSDPA_ERR_* code. */
 const char *dsdpa_error_string(int code);
@@ -122,6 +124,9 @@ int dsdpa_version(void);
  * `path` is unknown. Process-wide; the reference's analogue is the autotune
  * table, ops/triton.py:10-25.
  */
+/* Backward dk/dv: AUTO = cell-binned register accumulation, LDS = tiles of the
+ * plane accumulated in LDS with fp64 atomics, GATHER = global float atomics per
+ * tap as in the reference (ops/triton.py:345-360). Forward: one path so far. */
 enum { DSDPA_PATH_AUTO = 0, DSDPA_PATH_GATHER = 1, DSDPA_PATH_LDS = 2 };
 int dsdpa_set_path(int path);
 

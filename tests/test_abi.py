@@ -38,16 +38,18 @@ def test_version_and_error_strings():
 
 def test_workspace_bytes():
     lib = _native.load()
-    def delta_bytes(rows):
-        return (rows * 4 + 255) // 256 * 256
-    rows = 2 * 6 * 8 * 18 * 18
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32) == delta_bytes(rows)
-    rows = 2 * 6 * 8 * 48 * 48
-    n = rows * 64
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64) == 8 * n + delta_bytes(rows)
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F16, 2, 6, 8, 48, 48, 64) == 8 * n + delta_bytes(rows)
-    assert lib.dsdpa_bwd_workspace_bytes(7, 2, 6, 8, 48, 48, 64) == 0
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 0, 6, 8, 48, 48, 64) == 0
+    r256 = lambda b: (b + 255) // 256 * 256
+
+    def expect(B, V, H, Himg, Wimg, D, P, storage16):
+        rows, NC = B * V * H * Himg * Wimg, (Himg + 1) * (Wimg + 1)
+        total = r256(rows * 4) + r256(B * V * NC * 4) + r256(B * V * (NC + 1) * 4) + r256(B * V * V * Himg * Wimg * P * 4)
+        return total + (r256(2 * rows * D * 4) if storage16 else 0)
+
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32) == expect(2, 6, 8, 18, 18, 32, 32, False)
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64, 32) == expect(2, 6, 8, 48, 48, 64, 32, True)
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F16, 1, 2, 1, 3, 5, 16, 7) == expect(1, 2, 1, 3, 5, 16, 7, True)
+    assert lib.dsdpa_bwd_workspace_bytes(7, 2, 6, 8, 48, 48, 64, 32) == 0
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 0, 6, 8, 48, 48, 64, 32) == 0
 
 
 def test_argument_validation_before_launch():

@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 
 TOL_FWD = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 2e-2}
 TOL_BWD = {torch.float32: 1e-3, torch.bfloat16: 2e-2, torch.float16: 2e-2}
-PATHS = {"gather": _native.PATH_GATHER, "auto": _native.PATH_AUTO}
+PATHS = {"gather": _native.PATH_GATHER, "lds": _native.PATH_LDS, "auto": _native.PATH_AUTO}
 
 
 def rel(a, b):
