@@ -12,6 +12,7 @@
 #include "dsdpa_gather.h"
 #include "dsdpa_tile.h"
 #include "dsdpa_cell.h"
+#include "dsdpa_plane.h"
 
 using namespace dsdpa;
 
@@ -51,6 +52,10 @@ struct ScopedKernelTimer {
         g_timer.pairs[which].push_back(ev);
     }
 };
+
+constexpr int kLdsBytes = 160 * 1024;                                   // LDS per workgroup on gfx950
+// query rows per wave in the plane kernels: rows * elements-per-lane = 16 keeps them at 128 VGPRs
+template <int DC> struct PlaneRows { static constexpr int value = 16 / DC >= 1 ? 16 / DC : 1; };
 
 // ------------------------------------------------------------------ small kernels
 __global__ void fill_zero_kernel(float4 *__restrict__ p, size_t n4)
@@ -145,7 +150,6 @@ int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const floa
     return check_launch();
 }
 
-constexpr int kLdsBytes = 160 * 1024;                                   // LDS per workgroup on gfx950
 constexpr int kTileDescBytes = kTileWaves * kWave * (16 + 16 + 4);      // per-wave tap descriptors
 
 // Tile geometry for the dk/dv kernel: as few tiles per plane as the LDS budget allows
@@ -206,6 +210,51 @@ int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const floa
     return check_launch();
 }
 
+// The plane kernels need one K and one V plane of a (b, s2, h) in LDS next to the descriptors.
+template <typename S>
+bool plane_fits(const Dims &dm, int D)
+{
+    return (size_t)2 * dm.L * D * S::kBytes + kPlaneDescBytes <= (size_t)kLdsBytes;
+}
+
+template <typename S, int D>
+int launch_fwd_plane(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+                     const Dims &dm, hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const size_t smem = (size_t)2 * dm.L * D * S::kBytes + kPlaneDescBytes;
+    constexpr int QW = PlaneRows<DC>::value;
+    const int rows_per_block = kPlaneWaves * QW;
+    const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
+    auto kern = fwd_plane_kernel<S, D, DC, QW>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    ScopedKernelTimer timer(0, st);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
+                       q, k, v, coords, out, lse, dm);
+    return check_launch();
+}
+
+template <typename S, int D>
+int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float *coords, const void *out,
+                        const float *lse, const void *dout, void *dq, float *delta, const Dims &dm,
+                        hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const size_t smem = (size_t)2 * dm.L * D * S::kBytes + kPlaneDescBytes;
+    constexpr int QW = PlaneRows<DC>::value;
+    const int rows_per_block = kPlaneWaves * QW;
+    const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
+    auto kern = bwd_dq_plane_kernel<S, D, DC, QW>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
+                       q, k, v, coords, out, lse, dout, dq, delta, dm);
+    return check_launch();
+}
+
 template <typename S>
 int fwd_impl(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
              int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
@@ -215,13 +264,19 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
     int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
     if (rc != DSDPA_OK) return rc;
     hipStream_t st = (hipStream_t)stream;
+    const bool staged = g_path.load() != DSDPA_PATH_GATHER && plane_fits<S>(dm, D);
+#define DSDPA_FWD_CASE(DD)                                                                        \
+    case DD:                                                                                      \
+        return staged ? launch_fwd_plane<S, DD>(q, k, v, coords, out, lse, dm, st)                \
+                      : launch_fwd_gather<S, DD>(q, k, v, coords, out, lse, dm, st);
     switch (D) {
-    case 16: return launch_fwd_gather<S, 16>(q, k, v, coords, out, lse, dm, st);
-    case 32: return launch_fwd_gather<S, 32>(q, k, v, coords, out, lse, dm, st);
-    case 64: return launch_fwd_gather<S, 64>(q, k, v, coords, out, lse, dm, st);
-    case 128: return launch_fwd_gather<S, 128>(q, k, v, coords, out, lse, dm, st);
-    case 256: return launch_fwd_gather<S, 256>(q, k, v, coords, out, lse, dm, st);
+        DSDPA_FWD_CASE(16)
+        DSDPA_FWD_CASE(32)
+        DSDPA_FWD_CASE(64)
+        DSDPA_FWD_CASE(128)
+        DSDPA_FWD_CASE(256)
     }
+#undef DSDPA_FWD_CASE
     return DSDPA_ERR_HEAD_DIM;
 }
 
@@ -264,6 +319,8 @@ WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Himg, size
     return w;
 }
 
+// elements per lane in the cell kernel: one 16-byte load per tap; 8 fp32 elements per lane were
+// measured slower (211 VGPRs, 2 waves per SIMD, latency-bound)
 template <typename S, int D> struct CellChunk {
     static constexpr int value = Chunk<S, D>::value > 8 ? 8 : Chunk<S, D>::value;
 };
@@ -273,6 +330,31 @@ int launch_binning(const float *coords, const Dims &dm, const WorkspaceLayout &w
     unsigned *counters = (unsigned *)(ws + wl.counters);
     unsigned *start = (unsigned *)(ws + wl.start);
     unsigned *sorted = (unsigned *)(ws + wl.sorted);
+    const size_t hist_bytes = (size_t)dm.V * wl.NC * sizeof(unsigned);
+    if (2 * hist_bytes <= (size_t)kLdsBytes - 1024) {
+        // LDS-aggregated passes: a workgroup per run of about 8k samples of one (b, s1)
+        int lchunk = 8192 / dm.N;
+        if (lchunk < 1) lchunk = 1;
+        if (lchunk > dm.L) lchunk = dm.L;
+        const int nlc = (dm.L + lchunk - 1) / lchunk;
+        lchunk = (dm.L + nlc - 1) / nlc;
+        const long long blocks = (long long)dm.B * dm.V * nlc;
+        if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+        auto k0 = bin_samples_lds_kernel<0>;
+        auto k1 = bin_samples_lds_kernel<1>;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k0),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)hist_bytes);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k1),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * hist_bytes));
+        if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+        hipLaunchKernelGGL(k0, dim3((unsigned)blocks), dim3(kBinLdsThreads), hist_bytes, st,
+                           coords, dm, wl.NC, lchunk, nlc, counters, sorted);
+        hipLaunchKernelGGL(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st, counters, start, wl.NC);
+        hipLaunchKernelGGL(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
+                           coords, dm, wl.NC, lchunk, nlc, counters, sorted);
+        return check_launch();
+    }
     const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
     const long long blocks = (total + kBinThreads - 1) / kBinThreads;
     if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
@@ -329,6 +411,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const int path = g_path.load();
     const bool fused_atomics = path == DSDPA_PATH_GATHER;
     const bool cell_binned = path == DSDPA_PATH_AUTO;
+    const bool staged = plane_fits<S>(dm, D);
     const unsigned *start = (const unsigned *)(ws + wl.start);
     const unsigned *sorted = (const unsigned *)(ws + wl.sorted);
     if (cell_binned) {
@@ -340,7 +423,8 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
         if (fused_atomics) {                                                                                    \
             rc = launch_bwd_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st);         \
         } else {                                                                                                \
-            rc = launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dm, st);               \
+            rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dm, st)        \
+                        : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dm, st);      \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
                 rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, lse, delta, dout, start, sorted, dk_acc,      \
                                                  dv_acc, dm, wl.NC, st);                                        \

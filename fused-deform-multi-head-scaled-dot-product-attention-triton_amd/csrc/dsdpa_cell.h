@@ -65,6 +65,64 @@ __global__ __launch_bounds__(kBinThreads) void bin_samples_kernel(const float *_
     }
 }
 
+// LDS-aggregated variant of the two passes above, used when the V*NC counters of
+// one batch item fit in LDS. A workgroup takes a contiguous run of query rows of
+// one (b, s1) -- whose coordinates are one contiguous block covering all V key
+// views -- and histograms it in LDS first, so the contended global atomics drop
+// from one per sample to one per (workgroup, non-empty cell).
+// mode 0: global count[cell] += local count
+// mode 1: reserve [base, base+local count) from the global cursor of each cell,
+//         then place every sample at base + its local rank.
+constexpr int kBinLdsThreads = 1024;
+
+template <int MODE>
+__global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
+    const float *__restrict__ coords_, Dims dm, int NC, int lchunk, int nlc,
+    unsigned *__restrict__ counters, unsigned *__restrict__ sorted)
+{
+    extern __shared__ unsigned s_hist[];                 // [V][NC]; mode 1 adds [V][NC] bases
+    unsigned *s_base = s_hist + (size_t)dm.V * NC;
+    const int lc = blockIdx.x % nlc;
+    const int s1 = (blockIdx.x / nlc) % dm.V;
+    const int b = blockIdx.x / (nlc * dm.V);
+    const int l0 = lc * lchunk, l1 = min(dm.L, l0 + lchunk);
+    const int nhist = dm.V * NC;
+    for (int i = threadIdx.x; i < nhist; i += kBinLdsThreads) s_hist[i] = 0u;
+    __syncthreads();
+    const float2 *crd = reinterpret_cast<const float2 *>(coords_) + (((size_t)b * dm.V + s1) * dm.L + l0) * dm.N;
+    const int total = (l1 - l0) * dm.N;                  // samples of this workgroup, all key views
+    for (int i = threadIdx.x; i < total; i += kBinLdsThreads) {
+        const float2 xy = crd[i];
+        const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
+        if (taps_any(tp)) atomicAdd(&s_hist[((i / dm.P) % dm.V) * NC + cell_of(tp, dm.Wimg)], 1u);
+    }
+    __syncthreads();
+    unsigned *gctr = counters + (size_t)b * dm.V * NC;   // [s2][cell] of this batch item
+    if (MODE == 0) {
+        for (int i = threadIdx.x; i < nhist; i += kBinLdsThreads) {
+            const unsigned c = s_hist[i];
+            if (c) atomicAdd(gctr + i, c);
+        }
+    } else {
+        for (int i = threadIdx.x; i < nhist; i += kBinLdsThreads) {
+            const unsigned c = s_hist[i];
+            s_base[i] = c ? atomicAdd(gctr + i, c) : 0u;
+            s_hist[i] = 0u;
+        }
+        __syncthreads();
+        const size_t M = (size_t)dm.V * dm.L * dm.P;
+        for (int i = threadIdx.x; i < total; i += kBinLdsThreads) {
+            const float2 xy = crd[i];
+            const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
+            if (!taps_any(tp)) continue;
+            const int p = i % dm.P, s2 = (i / dm.P) % dm.V, l = l0 + i / dm.N;
+            const int hidx = s2 * NC + cell_of(tp, dm.Wimg);
+            const unsigned pos = s_base[hidx] + atomicAdd(&s_hist[hidx], 1u);
+            sorted[((size_t)b * dm.V + s2) * M + pos] = ((unsigned)s1 * dm.L + l) * (unsigned)dm.P + (unsigned)p;
+        }
+    }
+}
+
 // One workgroup per (b, s2): exclusive scan of the NC cell counts. Writes
 // start[grp*(NC+1) + c] (with the total at c = NC) and resets counters to the
 // same starts, so that the fill pass can use them as cursors.
@@ -113,7 +171,7 @@ __device__ __forceinline__ void load_tap_or_zero(const char *base, int pix, int 
 }
 
 template <typename S, int D, int DC>
-__global__ __launch_bounds__(kCellWaves *kWave) void bwd_dkdv_cell_kernel(
+__global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 4 : 2) void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float *__restrict__ lse_, const float *__restrict__ delta_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
@@ -162,14 +220,22 @@ __global__ __launch_bounds__(kCellWaves *kWave) void bwd_dkdv_cell_kernel(
     const unsigned *list = sorted + grp * M;
     const float2 *coords = reinterpret_cast<const float2 *>(coords_);
 
+    // Walk the list 64 entries at a time. Sample ids are fetched one chunk ahead
+    // (the coordinate load depends on them). A software-pipelined version of the
+    // inner loop (query rows of the next NS samples prefetched) was measured
+    // slower: the register copies it adds cost more VALU issue slots than the
+    // four resident waves per SIMD fail to hide.
+    auto load_id = [&](unsigned cstart) -> unsigned {
+        return cstart < hi ? list[min(cstart + (unsigned)lane, hi - 1u)] : 0u;
+    };
+    unsigned id_nxt = load_id(lo);
     for (unsigned c0 = lo; c0 < hi; c0 += kWave) {
+        const unsigned id = id_nxt;
+        id_nxt = load_id(c0 + kWave);
         // one list entry per lane: weights and query row
-        const unsigned idx = c0 + lane;
-        const bool in_range = idx < hi;
-        const unsigned id = list[in_range ? idx : hi - 1];
         const unsigned p = id % (unsigned)dm.P, ql = id / (unsigned)dm.P;      // ql = s1*L + l
         const unsigned s1 = ql / (unsigned)dm.L, l = ql % (unsigned)dm.L;
-        const size_t ci = ((((size_t)b * dm.V + s1) * dm.L + l) * dm.V + s2) * (size_t)dm.P + p;
+        const size_t ci = (((size_t)b * dm.V * dm.L + ql) * dm.V + s2) * (size_t)dm.P + p;
         const float2 xy = coords[ci];
         const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
         const unsigned row = (unsigned)((((size_t)b * dm.V + s1) * dm.H + h) * dm.L + l);

@@ -124,9 +124,11 @@ int dsdpa_version(void);
  * `path` is unknown. Process-wide; the reference's analogue is the autotune
  * table, ops/triton.py:10-25.
  */
-/* Backward dk/dv: AUTO = cell-binned register accumulation, LDS = tiles of the
+/* Forward and backward-dq: AUTO and LDS stage each key view's K/V planes in LDS
+ * when a plane pair fits, GATHER always reads the taps from global memory.
+ * Backward dk/dv: AUTO = cell-binned register accumulation, LDS = tiles of the
  * plane accumulated in LDS with fp64 atomics, GATHER = global float atomics per
- * tap as in the reference (ops/triton.py:345-360). Forward: one path so far. */
+ * tap as in the reference (ops/triton.py:345-360). */
 enum { DSDPA_PATH_AUTO = 0, DSDPA_PATH_GATHER = 1, DSDPA_PATH_LDS = 2 };
 int dsdpa_set_path(int path);
 
