@@ -8,8 +8,8 @@ A "step" is one forward + backward pass of the public operator
 resident in HBM. Prints ONE JSON line on stdout:
 
   metric/value   M query.samples/s of fwd+bwd (query.samples = B*V*H*L * V*P)
-  roofline       the dominant kernel against the 8 TB/s HBM roofline on its
-                 algorithmic (compulsory) bytes; its average duration is measured
+  roofline       the dominant (longest) kernel against the 8 TB/s HBM roofline on its
+                 own algorithmic (compulsory) bytes; its average duration is measured
                  here with HIP events recorded by the library around that kernel
                  on the launch stream, during the timed steps
   cpu_baseline   the same workload through the host-CPU PyTorch path
@@ -37,14 +37,21 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each counter
+# scaled by its reading for a plain 256 MiB copy: FETCH x 2.000, WRITE x 1.000. Source and commands:
+# profiles/hbm_traffic_C2.md. Only the kernels of the bench workload were measured.
+MEASURED_TRAFFIC_BYTES = {
+    "C2": {
+        "fwd": int((22307.3 * 2.0 + 4012.9) * 1024),
+        "bwd_dq": int((30338.5 * 2.0 + 4011.9) * 1024),
+        "bwd_dkdv": int((42932.1 * 2.0 + 110976.0) * 1024),
+    },
+}
+
+
 def load_traffic(workload, which):
-    """Measured HBM bytes per launch from profiles/hbm_traffic.json (rocprofv3 --pmc runs), or None."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    try:
-        with open(path) as f:
-            return json.load(f).get(workload, {}).get(which)
-    except (OSError, ValueError):
-        return None
+    """Measured HBM bytes per launch of a kernel of a workload, or None when it was not measured."""
+    return MEASURED_TRAFFIC_BYTES.get(workload, {}).get(which)
 
 
 def measure_gpu(wl, steps, warmup):
@@ -74,8 +81,10 @@ def measure_gpu(wl, steps, warmup):
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     _native.timer_enable(False)
-    fwd_ms, fwd_n = _native.timer_collect(0)
-    bwd_ms, bwd_n = _native.timer_collect(1)
+    kern = {}
+    for which, name in enumerate(("fwd", "bwd_dkdv", "bwd_dq", "bwd_bin")):
+        ms, n = _native.timer_collect(which)
+        kern[name] = {"ms": ms / max(n, 1), "launches": n}
     ms_step = (t1 - t0) * 1e3 / steps
 
     # forward alone (no autograd graph), timed separately
@@ -97,9 +106,7 @@ def measure_gpu(wl, steps, warmup):
     return {
         "ms_per_step": ms_step,
         "fwd_only_ms": fwd_only_ms,
-        "fwd_kernel_ms": fwd_ms / max(fwd_n, 1),
-        "bwd_kernel_ms": bwd_ms / max(bwd_n, 1),
-        "kernel_launches": [fwd_n, bwd_n],
+        "kernels": kern,
         "peak_extra_bytes": int(peak_extra),
     }
 
@@ -143,6 +150,9 @@ def main():
     ap.add_argument("--workload", default="C2")
     ap.add_argument("--all", action="store_true", help="also report the other workloads on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="first run a plain 256 MiB device copy a few times (known HBM traffic, used to scale "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU; run with --gpus 1 "
@@ -150,29 +160,56 @@ def main():
 
     from workloads import WORKLOADS
     wl = WORKLOADS[args.workload]
+    if args.copy_calibration:
+        import torch
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)          # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     g = measure_gpu(wl, args.steps, args.warmup)
     qs = wl.query_samples
     value = qs / (g["ms_per_step"] * 1e-3) / 1e6
 
-    dominant = "bwd" if g["bwd_kernel_ms"] >= g["fwd_kernel_ms"] else "fwd"
-    dom_ms = g[dominant + "_kernel_ms"]
-    dom_bytes = wl.algorithmic_bytes(dominant)
-    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    # Per-kernel algorithmic (compulsory) bytes: every tensor the kernel must read or write, once.
+    #   fwd      q,k,v read + out written + coords            = 4*N*e + C
+    #   bwd_dq   q,k,v,out,dout read + dq written + coords    = 6*N*e + C
+    #   bwd_dkdv q,k,v,dout read + dk,dv written + coords     = 6*N*e + C
+    # (whole backward, each tensor once: 8*N*e + C; the per-row lse/delta side buffers are left out.)
+    def kernel_bytes(w, name):
+        n = w.rows * w.D * w.esize
+        c = w.B * w.V * w.L * w.V * w.P * 8
+        return {"fwd": 4 * n + c, "bwd_dq": 6 * n + c, "bwd_dkdv": 6 * n + c}[name]
+
+    def kernel_report(w, gk):
+        rep = {}
+        for name in ("fwd", "bwd_dq", "bwd_dkdv"):
+            ms = gk[name]["ms"]
+            if gk[name]["launches"] == 0 or ms <= 0:
+                continue
+            ach = kernel_bytes(w, name) / (ms * 1e-3) / 1e9
+            rep[name] = {"kernel_ms": ms, "algorithmic_bytes": kernel_bytes(w, name), "achieved": ach,
+                         "frac": ach / HBM_PEAK_GBS}
+        return rep
+
+    rep = kernel_report(wl, g["kernels"])
+    dominant = max(rep, key=lambda k: rep[k]["kernel_ms"])
+    dom = rep[dominant]
     roofline = {
-        "bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": achieved / HBM_PEAK_GBS, "traffic": load_traffic(wl.name, dominant),
-        "algorithmic_bytes": dom_bytes, "kernel_ms": dom_ms,
+        "bound": "hbm", "kernel": dominant, "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": dom["frac"], "traffic": load_traffic(wl.name, dominant),
+        "algorithmic_bytes": dom["algorithmic_bytes"], "kernel_ms": dom["kernel_ms"],
     }
-    other = "fwd" if dominant == "bwd" else "bwd"
-    oth_bytes = wl.algorithmic_bytes(other)
-    oth_ach = oth_bytes / (g[other + "_kernel_ms"] * 1e-3) / 1e9
+    kernels_ms = sum(v["ms"] for v in g["kernels"].values())
     details = {
-        "workload": wl.name, "query_samples": qs, **g,
+        "workload": wl.name, "query_samples": qs, **g, "per_kernel": rep,
         "fwd_only_MQS_per_s": qs / (g["fwd_only_ms"] * 1e-3) / 1e6,
-        "roofline_" + other: {"achieved": oth_ach, "frac": oth_ach / HBM_PEAK_GBS,
-                              "algorithmic_bytes": oth_bytes, "kernel_ms": g[other + "_kernel_ms"]},
-        "fwd_bwd_kernels_frac_of_roofline":
-            wl.algorithmic_bytes("fwd+bwd") / ((g["fwd_kernel_ms"] + g["bwd_kernel_ms"]) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "all_kernels_ms": kernels_ms,
+        "fwd_bwd_frac_of_roofline_on_kernel_time":
+            wl.algorithmic_bytes("fwd+bwd") / (kernels_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "fwd_bwd_frac_of_roofline_on_step_time":
+            wl.algorithmic_bytes("fwd+bwd") / (g["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
     }
     log("[bench]", json.dumps(details))
 
@@ -184,8 +221,9 @@ def main():
             gg = measure_gpu(w, max(5, args.steps // 5), max(2, args.warmup // 2))
             d = {"workload": name, "query_samples": w.query_samples, **gg,
                  "MQS_per_s": w.query_samples / (gg["ms_per_step"] * 1e-3) / 1e6,
-                 "fwd_frac": w.algorithmic_bytes("fwd") / (gg["fwd_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                 "bwd_frac": w.algorithmic_bytes("bwd") / (gg["bwd_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+                 "per_kernel": kernel_report(w, gg["kernels"]),
+                 "fwd_bwd_frac_of_roofline_on_step_time":
+                     w.algorithmic_bytes("fwd+bwd") / (gg["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
             log("[bench]", json.dumps(d))
             all_details[name] = d
 
@@ -208,8 +246,10 @@ def main():
         "config": {"workload": f"{wl.name}: B{wl.B} V{wl.V} H{wl.H} D{wl.D} {wl.H_IMG}x{wl.W_IMG} P{wl.P} "
                                f"{wl.dtype} coords={wl.coords}, fwd+bwd through the autograd operator",
                    "query_samples_per_step": qs,
-                   "fwd_only_ms": g["fwd_only_ms"], "fwd_kernel_ms": g["fwd_kernel_ms"],
-                   "bwd_kernel_ms": g["bwd_kernel_ms"], "peak_extra_bytes": g["peak_extra_bytes"]},
+                   "fwd_only_ms": g["fwd_only_ms"],
+                   "kernel_ms": {k: round(v["ms"], 5) for k, v in g["kernels"].items()},
+                   "fwd_bwd_frac_of_hbm_roofline_on_step_time": details["fwd_bwd_frac_of_roofline_on_step_time"],
+                   "peak_extra_bytes": g["peak_extra_bytes"]},
         "roofline": roofline,
         "cpu_baseline": cpu,
     }

@@ -28,7 +28,7 @@ struct EventPair { hipEvent_t start, stop; };
 struct KernelTimer {
     std::atomic<bool> on{false};
     std::mutex mu;
-    std::vector<EventPair> pairs[2];   // [0] forward kernels, [1] backward kernels
+    std::vector<EventPair> pairs[4];   // [0] forward, [1] backward dk/dv, [2] backward dq, [3] cell binning
 };
 KernelTimer g_timer;
 
@@ -145,6 +145,7 @@ int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const floa
 {
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
+    ScopedKernelTimer timer(2, st);
     hipLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                        q, k, v, coords, out, lse, dout, dq, delta, dm);
     return check_launch();
@@ -250,6 +251,7 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    ScopedKernelTimer timer(2, st);
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
                        q, k, v, coords, out, lse, dout, dq, delta, dm);
     return check_launch();
@@ -331,6 +333,7 @@ int launch_binning(const float *coords, const Dims &dm, const WorkspaceLayout &w
     unsigned *start = (unsigned *)(ws + wl.start);
     unsigned *sorted = (unsigned *)(ws + wl.sorted);
     const size_t hist_bytes = (size_t)dm.V * wl.NC * sizeof(unsigned);
+    ScopedKernelTimer timer(3, st);
     if (2 * hist_bytes <= (size_t)kLdsBytes - 1024) {
         // LDS-aggregated passes: a workgroup per run of about 8k samples of one (b, s1)
         int lchunk = 8192 / dm.N;
@@ -532,7 +535,7 @@ int dsdpa_timer_enable(int on)
 
 int dsdpa_timer_collect(int which, double *total_ms, int *launches)
 {
-    if (which < 0 || which > 1 || !total_ms || !launches) return DSDPA_ERR_NULL_POINTER;
+    if (which < 0 || which > 3 || !total_ms || !launches) return DSDPA_ERR_NULL_POINTER;
     double sum = 0.0;
     int n = 0, rc = DSDPA_OK;
     std::vector<EventPair> taken;

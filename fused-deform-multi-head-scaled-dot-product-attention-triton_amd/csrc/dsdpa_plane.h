@@ -131,10 +131,6 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
 
     for (int s2 = 0; s2 < dm.V; ++s2) {
         const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;
-        // the first 64 coordinate pairs of every row: in flight while the planes are staged
-        float2 xy0[QW];
-#pragma unroll
-        for (int qi = 0; qi < QW; ++qi) xy0[qi] = coords[crow[qi] + (size_t)s2 * dm.P + min(lane, dm.P - 1)];
         __syncthreads();                                       // the previous view's readers are done
         stage_plane(sK, (const char *)k_ + plane, plane_bytes);
         stage_plane(sV, (const char *)v_ + plane, plane_bytes);
@@ -144,7 +140,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
             if (!have[qi]) continue;                           // wave-uniform
             const float2 *cq = coords + crow[qi] + (size_t)s2 * dm.P;
             for (int c0 = 0; c0 < dm.P; c0 += kWave) {
-                const float2 xy = c0 == 0 ? xy0[qi] : cq[min(c0 + lane, dm.P - 1)];
+                const float2 xy = cq[min(c0 + lane, dm.P - 1)];
                 stage_plane_descriptors<S, D>(xy, c0 + lane < dm.P, lane, dm.Wimg, dm.Himg, s_w, s_e);
                 const int cnt = min(kWave, dm.P - c0);
                 float sv[ITS];
@@ -265,9 +261,6 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
 
     for (int s2 = 0; s2 < dm.V; ++s2) {
         const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;
-        float2 xy0[QW];
-#pragma unroll
-        for (int qi = 0; qi < QW; ++qi) xy0[qi] = coords[crow[qi] + (size_t)s2 * dm.P + min(lane, dm.P - 1)];
         __syncthreads();
         stage_plane(sK, (const char *)k_ + plane, plane_bytes);
         stage_plane(sV, (const char *)v_ + plane, plane_bytes);
@@ -277,7 +270,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
             if (!have[qi]) continue;
             const float2 *cq = coords + crow[qi] + (size_t)s2 * dm.P;
             for (int c0 = 0; c0 < dm.P; c0 += kWave) {
-                const float2 xy = c0 == 0 ? xy0[qi] : cq[min(c0 + lane, dm.P - 1)];
+                const float2 xy = cq[min(c0 + lane, dm.P - 1)];
                 stage_plane_descriptors<S, D>(xy, c0 + lane < dm.P, lane, dm.Wimg, dm.Himg, s_w, s_e);
                 const int cnt = min(kWave, dm.P - c0);
                 for (int j0 = 0; j0 < cnt; j0 += NS) {

@@ -138,7 +138,8 @@ int dsdpa_set_path(int path);
  * every main forward / backward kernel launch is bracketed by a pair of
  * HIP events recorded on the launch stream. dsdpa_timer_collect waits for the
  * recorded events, returns the summed kernel time and the number of launches
- * for `which` (0 = forward kernels, 1 = backward kernels) and releases them.
+ * for `which` (0 = forward kernel, 1 = backward dk/dv kernel, 2 = backward dq
+ * kernel, 3 = the three cell-binning launches taken together) and releases them.
  * dsdpa_timer_enable returns the previous state.
  */
 int dsdpa_timer_enable(int on);
