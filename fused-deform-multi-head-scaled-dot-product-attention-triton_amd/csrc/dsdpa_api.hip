@@ -58,11 +58,15 @@ constexpr int kLdsBytes = 160 * 1024;                                   // LDS p
 template <int DC> struct PlaneRows { static constexpr int value = 16 / DC >= 1 ? 16 / DC : 1; };
 
 // ------------------------------------------------------------------ small kernels
-__global__ void fill_zero_kernel(float4 *__restrict__ p, size_t n4)
+// Zero up to three buffers in one launch (sizes in 16-byte units; unused slots have size 0).
+struct ZeroJob { float4 *p[3]; size_t n4[3]; };
+__global__ void fill_zero_kernel(ZeroJob job)
 {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; i < n4; i += stride) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+        for (size_t i = first; i < job.n4[k]; i += stride) job.p[k][i] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
 // fp32 accumulators -> 16-bit storage, 8 elements per thread
@@ -215,7 +219,7 @@ int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const floa
 template <typename S>
 bool plane_fits(const Dims &dm, int D)
 {
-    return (size_t)2 * dm.L * D * S::kBytes + kPlaneDescBytes <= (size_t)kLdsBytes;
+    return (size_t)(dm.L + 2) * 2 * D * S::kBytes + kPlaneDescBytes <= (size_t)kLdsBytes;
 }
 
 template <typename S, int D>
@@ -223,11 +227,13 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float *c
                      const Dims &dm, hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
-    const size_t smem = (size_t)2 * dm.L * D * S::kBytes + kPlaneDescBytes;
+    const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes;
     constexpr int QW = PlaneRows<DC>::value;
     const int rows_per_block = kPlaneWaves * QW;
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
-    auto kern = fwd_plane_kernel<S, D, DC, QW>;
+    constexpr bool kCanPair = QW % 2 == 0;
+    auto kern = (kCanPair && dm.P <= 32) ? fwd_plane_kernel<S, D, DC, QW, kCanPair>
+                                         : fwd_plane_kernel<S, D, DC, QW, false>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
@@ -243,11 +249,13 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
                         hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
-    const size_t smem = (size_t)2 * dm.L * D * S::kBytes + kPlaneDescBytes;
+    const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes;
     constexpr int QW = PlaneRows<DC>::value;
     const int rows_per_block = kPlaneWaves * QW;
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
-    auto kern = bwd_dq_plane_kernel<S, D, DC, QW>;
+    constexpr bool kCanPair = QW % 2 == 0;
+    auto kern = (kCanPair && dm.P <= 32) ? bwd_dq_plane_kernel<S, D, DC, QW, kCanPair>
+                                         : bwd_dq_plane_kernel<S, D, DC, QW, false>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
@@ -282,13 +290,17 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
     return DSDPA_ERR_HEAD_DIM;
 }
 
-int zero_fill(float *p, size_t n, hipStream_t st)   // n is a multiple of 4 (D >= 16)
+// element counts are multiples of 4 (D >= 16; workspace segments are 256-byte multiples)
+int zero_fill(float *a, size_t na, float *b, size_t nb, float *c, size_t nc, hipStream_t st)
 {
-    const size_t n4 = n / 4;
+    ZeroJob job{{(float4 *)a, (float4 *)b, (float4 *)c}, {na / 4, nb / 4, nc / 4}};
+    size_t big = job.n4[0] > job.n4[1] ? job.n4[0] : job.n4[1];
+    if (job.n4[2] > big) big = job.n4[2];
     const int threads = 256;
-    size_t blocks = (n4 + threads - 1) / threads;
+    size_t blocks = (big + threads - 1) / threads;
     if (blocks > 256 * 16) blocks = 256 * 16;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(threads), 0, st, (float4 *)p, n4);
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(threads), 0, st, job);
     return check_launch();
 }
 
@@ -400,27 +412,18 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const WorkspaceLayout wl = workspace_layout(B, V, H, Himg, Wimg, D, P, S::kBytes != 4);
     char *ws = (char *)workspace;
     float *delta = (float *)(ws + wl.delta);
-    float *dk_acc, *dv_acc;
-    if (S::kBytes == 4) {
-        dk_acc = (float *)dk;
-        dv_acc = (float *)dv;
-        if ((rc = zero_fill(dk_acc, n, st)) != DSDPA_OK) return rc;
-        if ((rc = zero_fill(dv_acc, n, st)) != DSDPA_OK) return rc;
-    } else {
-        dk_acc = (float *)(ws + wl.acc);
-        dv_acc = dk_acc + n;
-        if ((rc = zero_fill(dk_acc, 2 * n, st)) != DSDPA_OK) return rc;
-    }
     const int path = g_path.load();
     const bool fused_atomics = path == DSDPA_PATH_GATHER;
     const bool cell_binned = path == DSDPA_PATH_AUTO;
     const bool staged = plane_fits<S>(dm, D);
     const unsigned *start = (const unsigned *)(ws + wl.start);
     const unsigned *sorted = (const unsigned *)(ws + wl.sorted);
-    if (cell_binned) {
-        if ((rc = zero_fill((float *)(ws + wl.counters), wl.counters_bytes / 4, st)) != DSDPA_OK) return rc;
-        if ((rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
-    }
+    // one launch zeroes the dk/dv accumulators and, for the cell-binned path, the cell counters
+    float *dk_acc = S::kBytes == 4 ? (float *)dk : (float *)(ws + wl.acc);
+    float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
+    rc = zero_fill(dk_acc, n, dv_acc, n, (float *)(ws + wl.counters), cell_binned ? wl.counters_bytes / 4 : 0, st);
+    if (rc != DSDPA_OK) return rc;
+    if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
 #define DSDPA_BWD_CASE(DD)                                                                                      \
     case DD:                                                                                                    \
         if (fused_atomics) {                                                                                    \

@@ -1,74 +1,70 @@
 // "Plane" kernels: query-stationary forward and dq with the current key view's
 // K and V planes staged in LDS, for shapes where one (b, s2, h) plane pair
-// (2 * L * D * element size) fits next to the per-wave tap descriptors.
+// fits next to the per-wave tap descriptors.
 //
 // A workgroup of 16 waves owns 16*QW consecutive query rows of one (b, h) (rows
 // are counted over (s1, l), so a workgroup may straddle two query views) and
 // walks the V key views: stage K_s2 and V_s2 (coalesced 16-byte loads, kept in
 // the storage type), barrier, every wave runs its QW rows against the staged
-// planes -- the 4-tap gathers are ds_read_b128 of D-contiguous runs, G lanes per
-// sample as in the gather kernels -- barrier, next view. The online-softmax
-// state (forward) or dq accumulator (backward) of each row stays in registers
-// across the views.
+// planes, barrier, next view. The online-softmax state (forward) or the dq
+// accumulator (backward) of each row stays in registers across the views.
+//
+// LDS image of a view: pixel p of the plane sits at byte (p + 1) * 2*ROW, its K
+// row first and its V row right behind it (ROW = D * element size), with one
+// zeroed pad pixel before pixel 0 and one after pixel L-1. A sample's four taps
+// are then two base addresses -- (row0, x0) and (row1, x0), x0 in [-1, W-1] NOT
+// clamped -- plus compile-time offsets: +2*ROW for the right-hand tap, +ROW for
+// V. A tap that falls outside the image carries weight 0 and reads either a pad
+// or a neighbouring real pixel, never anything non-finite the caller did not
+// put there. The gathers are ds_read_b128 of D-contiguous runs, G lanes per
+// sample as in the gather kernels.
 #pragma once
 #include "dsdpa_common.h"
-#include "dsdpa_gather.h"
 
 namespace dsdpa {
 
 constexpr int kPlaneWaves = 16;
-constexpr int kPlaneDescBytes = kPlaneWaves * kWave * 32;   // float4 weights + int4 offsets per sample slot
+constexpr int kPlaneDescBytes = kPlaneWaves * kWave * (16 + 8);   // float4 weights + int2 base offsets
 
-__device__ __forceinline__ void stage_plane(unsigned char *dst, const char *src, int bytes)
+template <typename S, int D>
+__host__ __device__ constexpr int plane_lds_bytes(int L) { return (L + 2) * 2 * D * S::kBytes; }
+
+// global [L][D] plane -> LDS rows 1..L of the interleaved image (which = 0: K half, 1: V half)
+template <typename S, int D>
+__device__ __forceinline__ void stage_plane(unsigned char *lds, const char *src, int L, int which)
 {
+    constexpr int kRow = D * S::kBytes;
+    constexpr int kChunksPerRow = kRow / 16;
     const uint4 *s4 = reinterpret_cast<const uint4 *>(src);
-    uint4 *d4 = reinterpret_cast<uint4 *>(dst);
-    const int n16 = bytes >> 4;
-    for (int i = threadIdx.x; i < n16; i += kPlaneWaves * kWave) d4[i] = s4[i];
+    const int n16 = L * kChunksPerRow;
+    for (int i = threadIdx.x; i < n16; i += kPlaneWaves * kWave) {
+        const int pix = i / kChunksPerRow, c = i % kChunksPerRow;
+        *reinterpret_cast<uint4 *>(lds + (size_t)(pix + 1) * 2 * kRow + which * kRow + c * 16) = s4[i];
+    }
 }
 
-// Tap descriptors of one (query row, key view): lane n handles sample c0+n.
-// Offsets are BYTE offsets into the staged plane.
 template <typename S, int D>
-__device__ __forceinline__ void stage_plane_descriptors(float2 xy, bool valid, int lane,
-                                                        int Wimg, int Himg, float4 *s_w, int4 *s_e)
+__device__ __forceinline__ void zero_plane_pads(unsigned char *lds, int L)
+{
+    constexpr int kRow = D * S::kBytes;
+    constexpr int kChunks = 2 * kRow / 16;
+    for (int i = threadIdx.x; i < 2 * kChunks; i += kPlaneWaves * kWave) {
+        const int pad = i / kChunks, c = i % kChunks;
+        *reinterpret_cast<uint4 *>(lds + (size_t)(pad ? L + 1 : 0) * 2 * kRow + c * 16) = make_uint4(0, 0, 0, 0);
+    }
+}
+
+// Tap descriptor of one sample: 4 weights and the two base byte offsets (top and
+// bottom tap row) into the interleaved LDS image.
+template <typename S, int D>
+__device__ __forceinline__ void plane_descriptor(float2 xy, bool valid, int Wimg, int Himg, float4 &w, int2 &e)
 {
     const Taps tp = make_taps(xy.x, xy.y, Wimg, Himg);
-    constexpr int kRow = D * S::kBytes;
-    const float4 w = valid ? make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]) : make_float4(0.f, 0.f, 0.f, 0.f);
-    const int4 e = make_int4(tp.pix[0] * kRow, tp.pix[1] * kRow, tp.pix[2] * kRow, tp.pix[3] * kRow);
-    wave_lds_sync();
-    s_w[lane] = w;
-    s_e[lane] = e;
-    wave_lds_sync();
-}
-
-template <typename S, int DC>
-__device__ __forceinline__ void blend_taps_lds(const unsigned char *base, const int4 &e, const float4 &w,
-                                               int lane_byte, float (&dst)[DC])
-{
-    float t0[DC], t1[DC], t2[DC], t3[DC];
-    load_chunk<S, DC>(base + e.x + lane_byte, t0);
-    load_chunk<S, DC>(base + e.y + lane_byte, t1);
-    load_chunk<S, DC>(base + e.z + lane_byte, t2);
-    load_chunk<S, DC>(base + e.w + lane_byte, t3);
-#pragma unroll
-    for (int d = 0; d < DC; ++d)
-        dst[d] = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
-}
-
-template <typename S, int DC>
-__device__ __forceinline__ void accumulate_taps_lds(const unsigned char *base, const int4 &e, const float4 &c,
-                                                    int lane_byte, float (&acc)[DC])
-{
-    float t0[DC], t1[DC], t2[DC], t3[DC];
-    load_chunk<S, DC>(base + e.x + lane_byte, t0);
-    load_chunk<S, DC>(base + e.y + lane_byte, t1);
-    load_chunk<S, DC>(base + e.z + lane_byte, t2);
-    load_chunk<S, DC>(base + e.w + lane_byte, t3);
-#pragma unroll
-    for (int d = 0; d < DC; ++d)
-        acc[d] = fmaf(c.x, t0[d], fmaf(c.y, t1[d], fmaf(c.z, t2[d], fmaf(c.w, t3[d], acc[d]))));
+    constexpr int kPix = 2 * D * S::kBytes;
+    const int x0u = min(max(tp.x0, -1), Wimg - 1);
+    const int cy0 = min(max(tp.y0, 0), Himg - 1), cy1 = min(max(tp.y0 + 1, 0), Himg - 1);
+    w = valid ? make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]) : make_float4(0.f, 0.f, 0.f, 0.f);
+    e = make_int2((cy0 * Wimg + x0u + 1) * kPix, (cy1 * Wimg + x0u + 1) * kPix);
 }
 
 struct PlaneBlock {
@@ -88,28 +84,126 @@ __device__ __forceinline__ PlaneBlock decode_plane_block(const Dims &dm, int row
     return pb;
 }
 
+// Descriptors for two rows of a wave and one key view in one 64-lane pass (the
+// PAIR instantiations, launched when P <= 32 and QW is even): lanes 0-31 take
+// the even row, 32-63 the odd one, parked at descriptor slots 0.. and 32..
+template <typename S, int D>
+__device__ __forceinline__ void stage_pair_descriptors(const float2 *__restrict__ c_even,
+                                                       const float2 *__restrict__ c_odd, int P, int lane,
+                                                       int Wimg, int Himg, float4 *s_w, int2 *s_e)
+{
+    const int n = lane & 31;
+    const bool valid = n < P;
+    const float2 xy = ((lane < 32) ? c_even : c_odd)[valid ? n : P - 1];
+    float4 w;
+    int2 e;
+    plane_descriptor<S, D>(xy, valid, Wimg, Himg, w, e);
+    wave_lds_sync();
+    s_w[lane] = w;
+    s_e[lane] = e;
+    wave_lds_sync();
+}
+
+// One row, samples c0 .. c0+63.
+template <typename S, int D>
+__device__ __forceinline__ void stage_row_descriptors(const float2 *__restrict__ crow, int P, int c0, int lane,
+                                                      int Wimg, int Himg, float4 *s_w, int2 *s_e)
+{
+    const int n = c0 + lane;
+    const bool valid = n < P;
+    const float2 xy = crow[valid ? n : P - 1];
+    float4 w;
+    int2 e;
+    plane_descriptor<S, D>(xy, valid, Wimg, Himg, w, e);
+    wave_lds_sync();
+    s_w[lane] = w;
+    s_e[lane] = e;
+    wave_lds_sync();
+}
+
 // ------------------------------------------------------------------ forward
-template <typename S, int D, int DC, int QW>
+// One chunk (cnt <= 64 samples, descriptors at s_w/s_e[dbase ...]) of one row.
+template <typename S, int D, int DC>
+__device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const float4 *s_w, const int2 *s_e,
+                                                int dbase, int cnt, int slot, int lane_byte,
+                                                const float (&qf)[DC], float &m, float &lsum, float (&acc)[DC])
+{
+    constexpr int G = D / DC, NS = kWave / G, ITS = G;
+    constexpr int kRow = D * S::kBytes;
+    float sv[ITS];
+    float mc = kNegBig;
+#pragma unroll
+    for (int it = 0; it < ITS; ++it) {
+        sv[it] = kNegBig;
+        if (it * NS < cnt) {
+            const int j = it * NS + slot;
+            const float4 w = s_w[dbase + j];
+            const int2 e = s_e[dbase + j];
+            const unsigned char *top = lds + e.x + lane_byte, *bot = lds + e.y + lane_byte;
+            float t0[DC], t1[DC], t2[DC], t3[DC];
+            load_chunk<S, DC>(top, t0);
+            load_chunk<S, DC>(top + 2 * kRow, t1);
+            load_chunk<S, DC>(bot, t2);
+            load_chunk<S, DC>(bot + 2 * kRow, t3);
+            float dot = 0.f;
+#pragma unroll
+            for (int d = 0; d < DC; ++d) {
+                const float kk = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
+                dot = fmaf(qf[d], kk, dot);
+            }
+            dot = group_sum<G>(dot);
+            sv[it] = (j < cnt) ? dot : kNegBig;
+            mc = fmaxf(mc, sv[it]);
+        }
+    }
+    const float m_new = fmaxf(m, mc);
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+    m = m_new;
+    lsum *= alpha;
+#pragma unroll
+    for (int d = 0; d < DC; ++d) acc[d] *= alpha;
+#pragma unroll
+    for (int it = 0; it < ITS; ++it) {
+        if (it * NS < cnt) {
+            const int j = it * NS + slot;
+            const float p = (j < cnt) ? __builtin_amdgcn_exp2f(sv[it] - m_new) : 0.f;
+            lsum += p;
+            const float4 w = s_w[dbase + j];
+            const int2 e = s_e[dbase + j];
+            const unsigned char *top = lds + e.x + lane_byte + kRow, *bot = lds + e.y + lane_byte + kRow;
+            float t0[DC], t1[DC], t2[DC], t3[DC];
+            load_chunk<S, DC>(top, t0);
+            load_chunk<S, DC>(top + 2 * kRow, t1);
+            load_chunk<S, DC>(bot, t2);
+            load_chunk<S, DC>(bot + 2 * kRow, t3);
+            const float c0 = p * w.x, c1 = p * w.y, c2 = p * w.z, c3 = p * w.w;
+#pragma unroll
+            for (int d = 0; d < DC; ++d)
+                acc[d] = fmaf(c0, t0[d], fmaf(c1, t1[d], fmaf(c2, t2[d], fmaf(c3, t3[d], acc[d]))));
+        }
+    }
+}
+
+template <typename S, int D, int DC, int QW, bool PAIR>
 __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, void *__restrict__ out_, float *__restrict__ lse_, Dims dm)
 {
     constexpr int G = D / DC;
-    constexpr int NS = kWave / G;
-    constexpr int ITS = G;
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int plane_bytes = dm.L * D * S::kBytes;
-    unsigned char *sK = smem, *sV = smem + plane_bytes;
+    const int img_bytes = plane_lds_bytes<S, D>(dm.L);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    float4 *s_w = reinterpret_cast<float4 *>(smem + 2 * plane_bytes) + wave * kWave;
-    int4 *s_e = reinterpret_cast<int4 *>(smem + 2 * plane_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
+    float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
+    int2 *s_e = reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
 
     const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * QW);
     const int nq = dm.V * dm.L;
     const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
     const float qscale = dm.sm_scale * kLog2e;
     const float2 *coords = reinterpret_cast<const float2 *>(coords_);
+
+    zero_plane_pads<S, D>(smem, dm.L);
 
     float qf[QW][DC], acc[QW][DC], m[QW], lsum[QW];
     size_t row[QW], crow[QW];
@@ -132,53 +226,30 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
     for (int s2 = 0; s2 < dm.V; ++s2) {
         const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;
         __syncthreads();                                       // the previous view's readers are done
-        stage_plane(sK, (const char *)k_ + plane, plane_bytes);
-        stage_plane(sV, (const char *)v_ + plane, plane_bytes);
+        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, 0);
+        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
         __syncthreads();
+        if constexpr (PAIR) {
 #pragma unroll
-        for (int qi = 0; qi < QW; ++qi) {
-            if (!have[qi]) continue;                           // wave-uniform
-            const float2 *cq = coords + crow[qi] + (size_t)s2 * dm.P;
-            for (int c0 = 0; c0 < dm.P; c0 += kWave) {
-                const float2 xy = cq[min(c0 + lane, dm.P - 1)];
-                stage_plane_descriptors<S, D>(xy, c0 + lane < dm.P, lane, dm.Wimg, dm.Himg, s_w, s_e);
-                const int cnt = min(kWave, dm.P - c0);
-                float sv[ITS];
-                float mc = kNegBig;
+            for (int qp = 0; qp + 1 < QW; qp += 2) {
+                if (!have[qp]) continue;                       // wave-uniform; rows are consecutive
+                stage_pair_descriptors<S, D>(coords + crow[qp] + (size_t)s2 * dm.P,
+                                             coords + crow[qp + 1] + (size_t)s2 * dm.P, dm.P, lane,
+                                             dm.Wimg, dm.Himg, s_w, s_e);
+                fwd_plane_chunk<S, D, DC>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qf[qp], m[qp], lsum[qp], acc[qp]);
+                if (have[qp + 1])
+                    fwd_plane_chunk<S, D, DC>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qf[qp + 1], m[qp + 1],
+                                              lsum[qp + 1], acc[qp + 1]);
+            }
+        } else {
 #pragma unroll
-                for (int it = 0; it < ITS; ++it) {
-                    sv[it] = kNegBig;
-                    if (it * NS < cnt) {
-                        const int j = it * NS + slot;
-                        const float4 w = s_w[j];
-                        const int4 e = s_e[j];
-                        float kk[DC];
-                        blend_taps_lds<S, DC>(sK, e, w, lane_byte, kk);
-                        float dot = 0.f;
-#pragma unroll
-                        for (int d = 0; d < DC; ++d) dot = fmaf(qf[qi][d], kk[d], dot);
-                        dot = group_sum<G>(dot);
-                        sv[it] = (j < cnt) ? dot : kNegBig;
-                        mc = fmaxf(mc, sv[it]);
-                    }
-                }
-                const float m_new = fmaxf(m[qi], mc);
-                const float alpha = __builtin_amdgcn_exp2f(m[qi] - m_new);
-                m[qi] = m_new;
-                lsum[qi] *= alpha;
-#pragma unroll
-                for (int d = 0; d < DC; ++d) acc[qi][d] *= alpha;
-#pragma unroll
-                for (int it = 0; it < ITS; ++it) {
-                    if (it * NS < cnt) {
-                        const int j = it * NS + slot;
-                        const float p = (j < cnt) ? __builtin_amdgcn_exp2f(sv[it] - m_new) : 0.f;
-                        lsum[qi] += p;
-                        const float4 w = s_w[j];
-                        const int4 e = s_e[j];
-                        const float4 c = make_float4(p * w.x, p * w.y, p * w.z, p * w.w);
-                        accumulate_taps_lds<S, DC>(sV, e, c, lane_byte, acc[qi]);
-                    }
+            for (int qi = 0; qi < QW; ++qi) {
+                if (!have[qi]) continue;
+                const float2 *cq = coords + crow[qi] + (size_t)s2 * dm.P;
+                for (int c0 = 0; c0 < dm.P; c0 += kWave) {
+                    stage_row_descriptors<S, D>(cq, dm.P, c0, lane, dm.Wimg, dm.Himg, s_w, s_e);
+                    fwd_plane_chunk<S, D, DC>(smem, s_w, s_e, 0, min(kWave, dm.P - c0), slot, lane_byte, qf[qi],
+                                              m[qi], lsum[qi], acc[qi]);
                 }
             }
         }
@@ -213,27 +284,76 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
 }
 
 // ------------------------------------------------------------------ backward: dq and delta
-template <typename S, int D, int DC, int QW>
+template <typename S, int D, int DC>
+__device__ __forceinline__ void dq_plane_chunk(const unsigned char *lds, const float4 *s_w, const int2 *s_e,
+                                               int dbase, int cnt, int slot, int lane_byte, float qscale,
+                                               const float (&qf)[DC], const float (&dof)[DC], float lse,
+                                               float delta, float (&dqa)[DC])
+{
+    constexpr int G = D / DC, NS = kWave / G;
+    constexpr int kRow = D * S::kBytes;
+    for (int j0 = 0; j0 < cnt; j0 += NS) {
+        const int j = j0 + slot;
+        const float4 w = s_w[dbase + j];
+        const int2 e = s_e[dbase + j];
+        const unsigned char *top = lds + e.x + lane_byte, *bot = lds + e.y + lane_byte;
+        float kk[DC];
+        float dot = 0.f, dp = 0.f;
+        {
+            float t0[DC], t1[DC], t2[DC], t3[DC];
+            load_chunk<S, DC>(top, t0);
+            load_chunk<S, DC>(top + 2 * kRow, t1);
+            load_chunk<S, DC>(bot, t2);
+            load_chunk<S, DC>(bot + 2 * kRow, t3);
+#pragma unroll
+            for (int d = 0; d < DC; ++d) {
+                kk[d] = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
+                dot = fmaf(qf[d], kk[d], dot);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);     // keep the V taps out of the K taps' live range (register budget)
+        {
+            float u0[DC], u1[DC], u2[DC], u3[DC];
+            load_chunk<S, DC>(top + kRow, u0);
+            load_chunk<S, DC>(top + 3 * kRow, u1);
+            load_chunk<S, DC>(bot + kRow, u2);
+            load_chunk<S, DC>(bot + 3 * kRow, u3);
+#pragma unroll
+            for (int d = 0; d < DC; ++d) {
+                const float vv = fmaf(w.x, u0[d], fmaf(w.y, u1[d], fmaf(w.z, u2[d], w.w * u3[d])));
+                dp = fmaf(dof[d], vv, dp);
+            }
+        }
+        dot = group_sum<G>(dot);
+        dp = group_sum<G>(dp);
+        const float p = (j < cnt) ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
+        const float ds = p * (dp - delta);
+#pragma unroll
+        for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
+    }
+}
+
+template <typename S, int D, int DC, int QW, bool PAIR>
 __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
     const void *__restrict__ dout_, void *__restrict__ dq_, float *__restrict__ delta_, Dims dm)
 {
     constexpr int G = D / DC;
-    constexpr int NS = kWave / G;
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int plane_bytes = dm.L * D * S::kBytes;
-    unsigned char *sK = smem, *sV = smem + plane_bytes;
+    const int img_bytes = plane_lds_bytes<S, D>(dm.L);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    float4 *s_w = reinterpret_cast<float4 *>(smem + 2 * plane_bytes) + wave * kWave;
-    int4 *s_e = reinterpret_cast<int4 *>(smem + 2 * plane_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
+    float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
+    int2 *s_e = reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
 
     const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * QW);
     const int nq = dm.V * dm.L;
     const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
     const float qscale = dm.sm_scale * kLog2e;
     const float2 *coords = reinterpret_cast<const float2 *>(coords_);
+
+    zero_plane_pads<S, D>(smem, dm.L);
 
     float qf[QW][DC], dof[QW][DC], dqa[QW][DC], lse[QW], delta[QW];
     size_t row[QW], crow[QW];
@@ -254,7 +374,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
         float dl = 0.f;
 #pragma unroll
         for (int d = 0; d < DC; ++d) { dl = fmaf(dof[qi][d], of[d], dl); dqa[qi][d] = 0.f; }
-        delta[qi] = group_sum<G>(dl);
+        delta[qi] = group_sum<G>(dl);          // the reference's _bwd_preprocess, fused
         lse[qi] = lse_[row[qi]];
         if (have[qi] && lane == 0) delta_[row[qi]] = delta[qi];
     }
@@ -262,36 +382,31 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
     for (int s2 = 0; s2 < dm.V; ++s2) {
         const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;
         __syncthreads();
-        stage_plane(sK, (const char *)k_ + plane, plane_bytes);
-        stage_plane(sV, (const char *)v_ + plane, plane_bytes);
+        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, 0);
+        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
         __syncthreads();
+        if constexpr (PAIR) {
 #pragma unroll
-        for (int qi = 0; qi < QW; ++qi) {
-            if (!have[qi]) continue;
-            const float2 *cq = coords + crow[qi] + (size_t)s2 * dm.P;
-            for (int c0 = 0; c0 < dm.P; c0 += kWave) {
-                const float2 xy = cq[min(c0 + lane, dm.P - 1)];
-                stage_plane_descriptors<S, D>(xy, c0 + lane < dm.P, lane, dm.Wimg, dm.Himg, s_w, s_e);
-                const int cnt = min(kWave, dm.P - c0);
-                for (int j0 = 0; j0 < cnt; j0 += NS) {
-                    const int j = j0 + slot;
-                    const float4 w = s_w[j];
-                    const int4 e = s_e[j];
-                    float kk[DC], vv[DC];
-                    blend_taps_lds<S, DC>(sK, e, w, lane_byte, kk);
-                    blend_taps_lds<S, DC>(sV, e, w, lane_byte, vv);
-                    float dot = 0.f, dp = 0.f;
+            for (int qp = 0; qp + 1 < QW; qp += 2) {
+                if (!have[qp]) continue;
+                stage_pair_descriptors<S, D>(coords + crow[qp] + (size_t)s2 * dm.P,
+                                             coords + crow[qp + 1] + (size_t)s2 * dm.P, dm.P, lane,
+                                             dm.Wimg, dm.Himg, s_w, s_e);
+                dq_plane_chunk<S, D, DC>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qscale, qf[qp], dof[qp], lse[qp],
+                                         delta[qp], dqa[qp]);
+                if (have[qp + 1])
+                    dq_plane_chunk<S, D, DC>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qscale, qf[qp + 1],
+                                             dof[qp + 1], lse[qp + 1], delta[qp + 1], dqa[qp + 1]);
+            }
+        } else {
 #pragma unroll
-                    for (int d = 0; d < DC; ++d) {
-                        dot = fmaf(qf[qi][d], kk[d], dot);
-                        dp = fmaf(dof[qi][d], vv[d], dp);
-                    }
-                    dot = group_sum<G>(dot);
-                    dp = group_sum<G>(dp);
-                    const float p = (j < cnt) ? __builtin_amdgcn_exp2f(dot * qscale - lse[qi]) : 0.f;
-                    const float ds = p * (dp - delta[qi]);
-#pragma unroll
-                    for (int d = 0; d < DC; ++d) dqa[qi][d] = fmaf(ds, kk[d], dqa[qi][d]);
+            for (int qi = 0; qi < QW; ++qi) {
+                if (!have[qi]) continue;
+                const float2 *cq = coords + crow[qi] + (size_t)s2 * dm.P;
+                for (int c0 = 0; c0 < dm.P; c0 += kWave) {
+                    stage_row_descriptors<S, D>(cq, dm.P, c0, lane, dm.Wimg, dm.Himg, s_w, s_e);
+                    dq_plane_chunk<S, D, DC>(smem, s_w, s_e, 0, min(kWave, dm.P - c0), slot, lane_byte, qscale,
+                                             qf[qi], dof[qi], lse[qi], delta[qi], dqa[qi]);
                 }
             }
         }
