@@ -333,10 +333,11 @@ WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Himg, size
     return w;
 }
 
-// elements per lane in the cell kernel: one 16-byte load per tap; 8 fp32 elements per lane were
-// measured slower (211 VGPRs, 2 waves per SIMD, latency-bound)
+// elements per lane in the cell kernel: 4 up to D = 128 (32 lanes per sample at most), 8 beyond.
+// With 4 the kernel holds 64 tap/accumulator registers and runs 4 waves per SIMD; 8 elements per
+// lane at D = 32/64 were measured slower (211 VGPRs, 2 waves per SIMD, latency-bound).
 template <typename S, int D> struct CellChunk {
-    static constexpr int value = Chunk<S, D>::value > 8 ? 8 : Chunk<S, D>::value;
+    static constexpr int value = D <= 128 ? 4 : 8;
 };
 
 int launch_binning(const float *coords, const Dims &dm, const WorkspaceLayout &wl, char *ws, hipStream_t st)

@@ -46,7 +46,8 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f)
     return (uint16_t)(u >> 16);
 }
 
-// Load DC consecutive elements starting at a 16-byte aligned address, widened to fp32.
+// Load DC consecutive elements, widened to fp32. The address is 16-byte aligned, or 8-byte aligned
+// for a 4-element 16-bit chunk.
 template <typename S, int DC>
 __device__ __forceinline__ void load_chunk(const void *p, float (&dst)[DC])
 {
@@ -59,23 +60,33 @@ __device__ __forceinline__ void load_chunk(const void *p, float (&dst)[DC])
             dst[4 * i + 0] = t.x; dst[4 * i + 1] = t.y; dst[4 * i + 2] = t.z; dst[4 * i + 3] = t.w;
         }
     } else {
-        static_assert(DC % 8 == 0, "16-bit chunks are multiples of 8 elements");
-        const uint4 *src = reinterpret_cast<const uint4 *>(p);
+        static_assert(DC % 4 == 0, "16-bit chunks are multiples of 4 elements");
+        uint32_t w[DC / 2];
+        if constexpr (DC % 8 == 0) {
+            const uint4 *src = reinterpret_cast<const uint4 *>(p);
 #pragma unroll
-        for (int i = 0; i < DC / 8; ++i) {
-            uint4 t = src[i];
-            uint32_t w[4] = { t.x, t.y, t.z, t.w };
+            for (int i = 0; i < DC / 8; ++i) {
+                uint4 t = src[i];
+                w[4 * i + 0] = t.x; w[4 * i + 1] = t.y; w[4 * i + 2] = t.z; w[4 * i + 3] = t.w;
+            }
+        } else {
+            const uint2 *src = reinterpret_cast<const uint2 *>(p);      // 8-byte aligned
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if constexpr (S::kBf16) {
-                    dst[8 * i + 2 * j + 0] = __uint_as_float(w[j] << 16);
-                    dst[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
-                } else {
-                    union { uint32_t u; _Float16 h[2]; } cv;
-                    cv.u = w[j];
-                    dst[8 * i + 2 * j + 0] = (float)cv.h[0];
-                    dst[8 * i + 2 * j + 1] = (float)cv.h[1];
-                }
+            for (int i = 0; i < DC / 4; ++i) {
+                uint2 t = src[i];
+                w[2 * i + 0] = t.x; w[2 * i + 1] = t.y;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < DC / 2; ++j) {
+            if constexpr (S::kBf16) {
+                dst[2 * j + 0] = __uint_as_float(w[j] << 16);
+                dst[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+            } else {
+                union { uint32_t u; _Float16 h[2]; } cv;
+                cv.u = w[j];
+                dst[2 * j + 0] = (float)cv.h[0];
+                dst[2 * j + 1] = (float)cv.h[1];
             }
         }
     }
@@ -172,7 +183,8 @@ __device__ __forceinline__ float group_sum(float x)
     if constexpr (G >= 4) x += dpp_f32<0x4E>(x);    // quad_perm [2,3,0,1]
     if constexpr (G >= 8) x += dpp_f32<0x141>(x);   // row_half_mirror
     if constexpr (G >= 16) x += dpp_f32<0x140>(x);  // row_mirror
-    if constexpr (G >= 32) x += __shfl_xor(x, 16, kWave);
+    if constexpr (G >= 32)                            // ds_swizzle, bit mode: lane ^ 16 within each half-wave
+        x += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(x), 0x401F));
     if constexpr (G >= 64) x += __shfl_xor(x, 32, kWave);
     return x;
 }
