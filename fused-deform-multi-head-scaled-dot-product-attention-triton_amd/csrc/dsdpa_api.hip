@@ -232,8 +232,9 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float *c
     const int rows_per_block = kPlaneWaves * QW;
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
     constexpr bool kCanPair = QW % 2 == 0;
-    auto kern = (kCanPair && dm.P <= 32) ? fwd_plane_kernel<S, D, DC, QW, kCanPair>
-                                         : fwd_plane_kernel<S, D, DC, QW, false>;
+    // (a P == 32 compile-time instantiation was tried: the unrolled chunk spills 432 bytes per lane)
+    auto kern = (kCanPair && dm.P <= 32) ? fwd_plane_kernel<S, D, DC, QW, kCanPair, 0>
+                                         : fwd_plane_kernel<S, D, DC, QW, false, 0>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
@@ -254,8 +255,8 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
     const int rows_per_block = kPlaneWaves * QW;
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
     constexpr bool kCanPair = QW % 2 == 0;
-    auto kern = (kCanPair && dm.P <= 32) ? bwd_dq_plane_kernel<S, D, DC, QW, kCanPair>
-                                         : bwd_dq_plane_kernel<S, D, DC, QW, false>;
+    auto kern = (kCanPair && dm.P <= 32) ? bwd_dq_plane_kernel<S, D, DC, QW, kCanPair, 0>
+                                         : bwd_dq_plane_kernel<S, D, DC, QW, false, 0>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }

@@ -171,7 +171,7 @@ __device__ __forceinline__ void load_tap_or_zero(const char *base, int pix, int 
 }
 
 template <typename S, int D, int DC>
-__global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 4 : 2) void bwd_dkdv_cell_kernel(
+__global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : 2) void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float *__restrict__ lse_, const float *__restrict__ delta_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 4 : 2) void bwd_dkdv_c
     __shared__ float4 s_w[kCellWaves][kWave];
     __shared__ unsigned s_row[kCellWaves][kWave];
 
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const long long work = (long long)xcd_logical_block(blockIdx.x, gridDim.x) * kCellWaves + wave;
     const long long nwork = (long long)dm.B * dm.H * dm.V * NC;
     if (work >= nwork) return;

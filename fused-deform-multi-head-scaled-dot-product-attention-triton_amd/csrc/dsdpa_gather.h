@@ -105,7 +105,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
     __shared__ float4 s_w[kGatherWaves][kWave];
     __shared__ int4 s_e[kGatherWaves][kWave];
 
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
     if (work >= dm.rows) return;
     const RowCtx rc = decode_row(work, dm, D);
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_gather_kernel(
     __shared__ float4 s_w[kGatherWaves][kWave];
     __shared__ int4 s_e[kGatherWaves][kWave];
 
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
     if (work >= dm.rows) return;
     const RowCtx rc = decode_row(work, dm, D);
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     __shared__ float4 s_w[kGatherWaves][kWave];
     __shared__ int4 s_e[kGatherWaves][kWave];
 
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
     if (work >= dm.rows) return;
     const RowCtx rc = decode_row(work, dm, D);

@@ -123,12 +123,15 @@ __device__ __forceinline__ void stage_row_descriptors(const float2 *__restrict__
 
 // ------------------------------------------------------------------ forward
 // One chunk (cnt <= 64 samples, descriptors at s_w/s_e[dbase ...]) of one row.
-template <typename S, int D, int DC>
+// CNT > 0 fixes the sample count at compile time (branch-free, fully unrolled chunk).
+template <typename S, int D, int DC, int CNT>
 __device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const float4 *s_w, const int2 *s_e,
-                                                int dbase, int cnt, int slot, int lane_byte,
+                                                int dbase, int cnt_rt, int slot, int lane_byte,
                                                 const float (&qf)[DC], float &m, float &lsum, float (&acc)[DC])
 {
-    constexpr int G = D / DC, NS = kWave / G, ITS = G;
+    constexpr int G = D / DC, NS = kWave / G;
+    constexpr int ITS = CNT > 0 ? (CNT + NS - 1) / NS : G;
+    const int cnt = CNT > 0 ? CNT : cnt_rt;
     constexpr int kRow = D * S::kBytes;
     float sv[ITS];
     float mc = kNegBig;
@@ -184,7 +187,8 @@ __device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const 
     }
 }
 
-template <typename S, int D, int DC, int QW, bool PAIR>
+// PAIR: two rows per descriptor pass (P <= 32); PCNT > 0: P is exactly PCNT, known at compile time.
+template <typename S, int D, int DC, int QW, bool PAIR, int PCNT>
 __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, void *__restrict__ out_, float *__restrict__ lse_, Dims dm)
@@ -193,7 +197,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int img_bytes = plane_lds_bytes<S, D>(dm.L);
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
     int2 *s_e = reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
 
@@ -236,9 +240,9 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
                 stage_pair_descriptors<S, D>(coords + crow[qp] + (size_t)s2 * dm.P,
                                              coords + crow[qp + 1] + (size_t)s2 * dm.P, dm.P, lane,
                                              dm.Wimg, dm.Himg, s_w, s_e);
-                fwd_plane_chunk<S, D, DC>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qf[qp], m[qp], lsum[qp], acc[qp]);
+                fwd_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qf[qp], m[qp], lsum[qp], acc[qp]);
                 if (have[qp + 1])
-                    fwd_plane_chunk<S, D, DC>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qf[qp + 1], m[qp + 1],
+                    fwd_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qf[qp + 1], m[qp + 1],
                                               lsum[qp + 1], acc[qp + 1]);
             }
         } else {
@@ -248,7 +252,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
                 const float2 *cq = coords + crow[qi] + (size_t)s2 * dm.P;
                 for (int c0 = 0; c0 < dm.P; c0 += kWave) {
                     stage_row_descriptors<S, D>(cq, dm.P, c0, lane, dm.Wimg, dm.Himg, s_w, s_e);
-                    fwd_plane_chunk<S, D, DC>(smem, s_w, s_e, 0, min(kWave, dm.P - c0), slot, lane_byte, qf[qi],
+                    fwd_plane_chunk<S, D, DC, 0>(smem, s_w, s_e, 0, min(kWave, dm.P - c0), slot, lane_byte, qf[qi],
                                               m[qi], lsum[qi], acc[qi]);
                 }
             }
@@ -284,14 +288,15 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
 }
 
 // ------------------------------------------------------------------ backward: dq and delta
-template <typename S, int D, int DC>
+template <typename S, int D, int DC, int CNT>
 __device__ __forceinline__ void dq_plane_chunk(const unsigned char *lds, const float4 *s_w, const int2 *s_e,
-                                               int dbase, int cnt, int slot, int lane_byte, float qscale,
+                                               int dbase, int cnt_rt, int slot, int lane_byte, float qscale,
                                                const float (&qf)[DC], const float (&dof)[DC], float lse,
                                                float delta, float (&dqa)[DC])
 {
     constexpr int G = D / DC, NS = kWave / G;
     constexpr int kRow = D * S::kBytes;
+    const int cnt = CNT > 0 ? CNT : cnt_rt;
     for (int j0 = 0; j0 < cnt; j0 += NS) {
         const int j = j0 + slot;
         const float4 w = s_w[dbase + j];
@@ -333,7 +338,7 @@ __device__ __forceinline__ void dq_plane_chunk(const unsigned char *lds, const f
     }
 }
 
-template <typename S, int D, int DC, int QW, bool PAIR>
+template <typename S, int D, int DC, int QW, bool PAIR, int PCNT>
 __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
@@ -343,7 +348,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int img_bytes = plane_lds_bytes<S, D>(dm.L);
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
     int2 *s_e = reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
 
@@ -392,10 +397,10 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
                 stage_pair_descriptors<S, D>(coords + crow[qp] + (size_t)s2 * dm.P,
                                              coords + crow[qp + 1] + (size_t)s2 * dm.P, dm.P, lane,
                                              dm.Wimg, dm.Himg, s_w, s_e);
-                dq_plane_chunk<S, D, DC>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qscale, qf[qp], dof[qp], lse[qp],
+                dq_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qscale, qf[qp], dof[qp], lse[qp],
                                          delta[qp], dqa[qp]);
                 if (have[qp + 1])
-                    dq_plane_chunk<S, D, DC>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qscale, qf[qp + 1],
+                    dq_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qscale, qf[qp + 1],
                                              dof[qp + 1], lse[qp + 1], delta[qp + 1], dqa[qp + 1]);
             }
         } else {
@@ -405,7 +410,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
                 const float2 *cq = coords + crow[qi] + (size_t)s2 * dm.P;
                 for (int c0 = 0; c0 < dm.P; c0 += kWave) {
                     stage_row_descriptors<S, D>(cq, dm.P, c0, lane, dm.Wimg, dm.Himg, s_w, s_e);
-                    dq_plane_chunk<S, D, DC>(smem, s_w, s_e, 0, min(kWave, dm.P - c0), slot, lane_byte, qscale,
+                    dq_plane_chunk<S, D, DC, 0>(smem, s_w, s_e, 0, min(kWave, dm.P - c0), slot, lane_byte, qscale,
                                              qf[qi], dof[qi], lse[qi], delta[qi], dqa[qi]);
                 }
             }

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(kTileWaves *kWave) void bwd_dkdv_tile_kernel(
     int4 *s_e_all = reinterpret_cast<int4 *>(s_w_all + kTileWaves * kWave);
     int *s_loc_all = reinterpret_cast<int *>(s_e_all + kTileWaves * kWave);
 
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     float4 *s_w = s_w_all + wave * kWave;
     int4 *s_e = s_e_all + wave * kWave;
     int *s_loc = s_loc_all + wave * kWave;
