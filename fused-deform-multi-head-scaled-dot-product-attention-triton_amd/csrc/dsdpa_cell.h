@@ -126,7 +126,7 @@ __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
 // One workgroup per (b, s2): exclusive scan of the NC cell counts. Writes
 // start[grp*(NC+1) + c] (with the total at c = NC) and resets counters to the
 // same starts, so that the fill pass can use them as cursors.
-__global__ __launch_bounds__(1024) void bin_scan_kernel(unsigned *__restrict__ counters,
+static __global__ __launch_bounds__(1024) void bin_scan_kernel(unsigned *__restrict__ counters,
                                                         unsigned *__restrict__ start, int NC)
 {
     __shared__ unsigned s_part[1024];

@@ -1,0 +1,10 @@
+// F32 storage: instantiates the forward and backward entry of libdsdpa.so for this type.
+#include "dsdpa_impl.h"
+
+namespace dsdpa {
+template int fwd_impl<F32>(const void *, const void *, const void *, const float *, void *, float *, int, int, int, int,
+                           int, int, int, float, void *);
+template int bwd_impl<F32>(const void *, const void *, const void *, const float *, const void *, const float *,
+                           const void *, void *, void *, void *, void *, int, int, int, int, int, int, int, float,
+                           void *);
+}  // namespace dsdpa

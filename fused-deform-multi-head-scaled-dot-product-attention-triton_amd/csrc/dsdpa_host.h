@@ -1,0 +1,99 @@
+// Host-side state shared by the translation units of libdsdpa.so: error slot, kernel-path selector,
+// kernel timer. Defined in dsdpa_api.hip.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <mutex>
+#include <vector>
+
+#include "../../include/dsdpa.h"
+
+namespace dsdpa {
+
+extern thread_local int g_last_hip_error;
+extern std::atomic<int> g_path;
+
+// Optional kernel timer: while enabled, every main forward/backward kernel
+// launch is bracketed by a pair of HIP events on the launch stream. Process-wide
+// (a framework may run the backward pass on another thread than the forward).
+struct EventPair { hipEvent_t start, stop; };
+struct KernelTimer {
+    std::atomic<bool> on{false};
+    std::mutex mu;
+    std::vector<EventPair> pairs[4];   // [0] forward, [1] backward dk/dv, [2] backward dq, [3] cell binning
+};
+extern KernelTimer g_timer;
+
+struct ScopedKernelTimer {
+    hipStream_t st;
+    EventPair ev{nullptr, nullptr};
+    int which;
+    bool armed = false;
+    ScopedKernelTimer(int which_, hipStream_t st_) : st(st_), which(which_)
+    {
+        if (!g_timer.on.load(std::memory_order_relaxed)) return;
+        if (hipEventCreate(&ev.start) != hipSuccess) return;
+        if (hipEventCreate(&ev.stop) != hipSuccess) { (void)hipEventDestroy(ev.start); return; }
+        armed = hipEventRecord(ev.start, st) == hipSuccess;
+    }
+    ~ScopedKernelTimer()
+    {
+        if (!armed) return;
+        (void)hipEventRecord(ev.stop, st);
+        std::lock_guard<std::mutex> lock(g_timer.mu);
+        g_timer.pairs[which].push_back(ev);
+    }
+};
+
+inline int check_launch()
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return DSDPA_ERR_HIP;
+    }
+    return DSDPA_OK;
+}
+
+// Backward workspace, every segment rounded up to 256 bytes:
+//   delta    rows floats                     dout.out per query row
+//   counters B*V*NC u32                      per (batch, key view) cell counts, then fill cursors
+//   start    B*V*(NC+1) u32                  exclusive scan of the counts
+//   sorted   B*V*(V*L*P) u32                 sample ids ordered by cell
+//   acc      2*n floats                      fp32 dk/dv accumulators (16-bit storage only)
+// with NC = (Himg+1)*(Wimg+1) cells.
+inline size_t round256(size_t b) { return (b + 255) / 256 * 256; }
+struct WorkspaceLayout {
+    size_t delta, counters, start, sorted, acc, total;
+    size_t counters_bytes;
+    int NC;
+};
+inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Himg, size_t Wimg, size_t D, size_t P,
+                                        bool storage16)
+{
+    WorkspaceLayout w;
+    const size_t rows = B * V * H * Himg * Wimg;
+    w.NC = (int)((Himg + 1) * (Wimg + 1));
+    size_t off = 0;
+    w.delta = off; off += round256(rows * 4);
+    w.counters = off; w.counters_bytes = round256(B * V * (size_t)w.NC * 4); off += w.counters_bytes;
+    w.start = off; off += round256(B * V * ((size_t)w.NC + 1) * 4);
+    w.sorted = off; off += round256(B * V * (V * Himg * Wimg * P) * 4);
+    w.acc = off; if (storage16) off += round256(2 * rows * D * 4);
+    w.total = off;
+    return w;
+}
+
+// One storage type's forward / backward entry (argument checks, kernel selection, launches); each is
+// instantiated in its own translation unit (dsdpa_f32.hip, dsdpa_bf16.hip, dsdpa_f16.hip) so that the
+// three compile in parallel.
+template <typename S>
+int fwd_impl(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream);
+template <typename S>
+int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
+             const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,
+             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream);
+
+}  // namespace dsdpa

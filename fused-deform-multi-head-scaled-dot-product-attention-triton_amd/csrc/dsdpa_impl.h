@@ -1,0 +1,383 @@
+// Launchers and per-storage-type entry points (argument checks, kernel selection, launches).
+// Included by one translation unit per storage type; no allocation, no synchronisation, no torch types.
+#pragma once
+#include "dsdpa_host.h"
+#include "dsdpa_common.h"
+#include "dsdpa_gather.h"
+#include "dsdpa_tile.h"
+#include "dsdpa_cell.h"
+#include "dsdpa_plane.h"
+
+namespace dsdpa {
+
+constexpr int kLdsBytes = 160 * 1024;                                   // LDS per workgroup on gfx950
+// query rows per wave in the plane kernels: rows * elements-per-lane = 16 keeps them at 128 VGPRs
+template <int DC> struct PlaneRows { static constexpr int value = 16 / DC >= 1 ? 16 / DC : 1; };
+
+// ------------------------------------------------------------------ small kernels
+// Zero up to three buffers in one launch (sizes in 16-byte units; unused slots have size 0).
+struct ZeroJob { float4 *p[3]; size_t n4[3]; };
+static __global__ void fill_zero_kernel(ZeroJob job)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+        for (size_t i = first; i < job.n4[k]; i += stride) job.p[k][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+// fp32 accumulators -> 16-bit storage, 8 elements per thread
+template <typename S>
+__global__ void cast_kernel(const float *__restrict__ src, void *__restrict__ dst, size_t n8)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n8; i += stride) {
+        float v[8];
+        const float4 *s4 = reinterpret_cast<const float4 *>(src) + 2 * i;
+        float4 a = s4[0], b = s4[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        store_chunk<S, 8>((char *)dst + i * 16, v);
+    }
+}
+
+static inline int make_dims(int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, Dims *dm)
+{
+    if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || P < 1) return DSDPA_ERR_BAD_SHAPE;
+    if (!(D == 16 || D == 32 || D == 64 || D == 128 || D == 256)) return DSDPA_ERR_HEAD_DIM;
+    const long long L = (long long)Himg * Wimg;
+    const long long slab = (long long)V * H * L * D;           // one batch item of k/v
+    const long long rows = (long long)B * V * H * L;
+    const long long N = (long long)V * P;
+    if (L > (1ll << 24) || slab > (1ll << 30) || rows > 0x7fffffffll - 1024 || N > (1ll << 24))
+        return DSDPA_ERR_TOO_LARGE;
+    dm->B = B; dm->V = V; dm->H = H; dm->Himg = Himg; dm->Wimg = Wimg;
+    dm->L = (int)L; dm->P = P; dm->N = (int)N; dm->rows = (int)rows; dm->sm_scale = sm_scale;
+    return DSDPA_OK;
+}
+
+// lanes per sample are D/DC; DC is chosen so that a lane moves 16 bytes per tap
+// (32 or 64 for the widest heads) and a sample never spans more than 16 lanes.
+template <typename S, int D> struct Chunk {
+    static constexpr int kMin = 16 / S::kBytes;
+    static constexpr int value = (D / kMin > 16) ? D / 16 : kMin;
+};
+
+template <typename S, int D>
+int launch_fwd_gather(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+                      const Dims &dm, hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
+    ScopedKernelTimer timer(0, st);
+    hipLaunchKernelGGL((fwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                       q, k, v, coords, out, lse, dm);
+    return check_launch();
+}
+
+template <typename S, int D>
+int launch_bwd_gather(const void *q, const void *k, const void *v, const float *coords, const void *out,
+                      const float *lse, const void *dout, void *dq, float *dk_acc, float *dv_acc,
+                      const Dims &dm, hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
+    ScopedKernelTimer timer(1, st);
+    hipLaunchKernelGGL((bwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                       q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm);
+    return check_launch();
+}
+
+template <typename S, int D>
+int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const float *coords, const void *out,
+                         const float *lse, const void *dout, void *dq, float *delta, const Dims &dm,
+                         hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
+    ScopedKernelTimer timer(2, st);
+    hipLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                       q, k, v, coords, out, lse, dout, dq, delta, dm);
+    return check_launch();
+}
+
+constexpr int kTileDescBytes = kTileWaves * kWave * (16 + 16 + 4);      // per-wave tap descriptors
+
+// Tile geometry for the dk/dv kernel: as few tiles per plane as the LDS budget allows
+// (every tile costs one more pass over the plane's coordinates and one halo ring).
+static inline TileGeom make_tile_geom(const Dims &dm, int D)
+{
+    const int maxpx = (kLdsBytes - kTileDescBytes) / (2 * (int)sizeof(double) * D);   // dK + dV, fp64
+    const int Hh = dm.Himg, Ww = dm.Wimg;
+    auto ceil_div = [](int a, int b) { return (a + b - 1) / b; };
+    // option A: full-width row bands
+    int a_nty = 1 << 30, a_th = 0;
+    if (Ww * 2 <= maxpx || Hh * Ww <= maxpx) {
+        const int rows = maxpx / Ww;                       // rows of pixels that fit
+        const int th_max = rows >= Hh ? Hh : rows - 1;     // one halo row unless the whole image fits
+        a_nty = ceil_div(Hh, th_max);
+        a_th = ceil_div(Hh, a_nty);
+    }
+    // option B: square-ish 2-D tiles
+    int side = 2;
+    while ((side + 1) * (side + 1) <= maxpx) ++side;
+    const int cells = side - 1 > 0 ? side - 1 : 1;
+    const int b_nty = ceil_div(Hh, cells), b_ntx = ceil_div(Ww, cells);
+    TileGeom tg;
+    if (a_nty <= b_nty * b_ntx) {
+        tg.th = a_th; tg.tw = Ww; tg.nty = a_nty; tg.ntx = 1;
+    } else {
+        tg.th = ceil_div(Hh, b_nty); tg.tw = ceil_div(Ww, b_ntx); tg.nty = b_nty; tg.ntx = b_ntx;
+    }
+    tg.lh = tg.nty == 1 ? Hh : tg.th + 1;
+    tg.lw = tg.ntx == 1 ? Ww : tg.tw + 1;
+    const long long groups = (long long)dm.B * dm.H * dm.V * tg.nty * tg.ntx;
+    long long qsplit = (1024 + groups - 1) / groups;
+    const long long max_split = ((long long)dm.V * dm.L + 63) / 64;    // keep >= 64 query rows per workgroup
+    if (qsplit > max_split) qsplit = max_split;
+    if (qsplit < 1) qsplit = 1;
+    tg.qsplit = (int)qsplit;
+    return tg;
+}
+
+template <typename S, int D>
+int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const float *coords, const float *lse,
+                         const float *delta, const void *dout, float *dk_acc, float *dv_acc, const Dims &dm,
+                         hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const TileGeom tg = make_tile_geom(dm, D);
+    const size_t smem = (size_t)2 * sizeof(double) * tg.lh * tg.lw * D + kTileDescBytes;
+    if (smem > (size_t)kLdsBytes) return DSDPA_ERR_TOO_LARGE;
+    const long long blocks = (long long)dm.B * dm.H * dm.V * tg.nty * tg.ntx * tg.qsplit;
+    if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+    auto kern = bwd_dkdv_tile_kernel<S, D, DC>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    ScopedKernelTimer timer(1, st);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kTileWaves * kWave), smem, st,
+                       q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, tg);
+    return check_launch();
+}
+
+// The plane kernels need one K and one V plane of a (b, s2, h) in LDS next to the descriptors.
+template <typename S>
+bool plane_fits(const Dims &dm, int D)
+{
+    return (size_t)(dm.L + 2) * 2 * D * S::kBytes + kPlaneDescBytes <= (size_t)kLdsBytes;
+}
+
+template <typename S, int D>
+int launch_fwd_plane(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+                     const Dims &dm, hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes;
+    constexpr int QW = PlaneRows<DC>::value;
+    const int rows_per_block = kPlaneWaves * QW;
+    const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
+    constexpr bool kCanPair = QW % 2 == 0;
+    // (a P == 32 compile-time instantiation was tried: the unrolled chunk spills 432 bytes per lane)
+    auto kern = (kCanPair && dm.P <= 32) ? fwd_plane_kernel<S, D, DC, QW, kCanPair, 0>
+                                         : fwd_plane_kernel<S, D, DC, QW, false, 0>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    ScopedKernelTimer timer(0, st);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
+                       q, k, v, coords, out, lse, dm);
+    return check_launch();
+}
+
+template <typename S, int D>
+int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float *coords, const void *out,
+                        const float *lse, const void *dout, void *dq, float *delta, const Dims &dm,
+                        hipStream_t st)
+{
+    constexpr int DC = Chunk<S, D>::value;
+    const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes;
+    constexpr int QW = PlaneRows<DC>::value;
+    const int rows_per_block = kPlaneWaves * QW;
+    const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
+    constexpr bool kCanPair = QW % 2 == 0;
+    auto kern = (kCanPair && dm.P <= 32) ? bwd_dq_plane_kernel<S, D, DC, QW, kCanPair, 0>
+                                         : bwd_dq_plane_kernel<S, D, DC, QW, false, 0>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    ScopedKernelTimer timer(2, st);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
+                       q, k, v, coords, out, lse, dout, dq, delta, dm);
+    return check_launch();
+}
+
+template <typename S>
+int fwd_impl(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    if (!q || !k || !v || !coords || !out || !lse) return DSDPA_ERR_NULL_POINTER;
+    Dims dm;
+    int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
+    if (rc != DSDPA_OK) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const bool staged = g_path.load() != DSDPA_PATH_GATHER && plane_fits<S>(dm, D);
+#define DSDPA_FWD_CASE(DD)                                                                        \
+    case DD:                                                                                      \
+        return staged ? launch_fwd_plane<S, DD>(q, k, v, coords, out, lse, dm, st)                \
+                      : launch_fwd_gather<S, DD>(q, k, v, coords, out, lse, dm, st);
+    switch (D) {
+        DSDPA_FWD_CASE(16)
+        DSDPA_FWD_CASE(32)
+        DSDPA_FWD_CASE(64)
+        DSDPA_FWD_CASE(128)
+        DSDPA_FWD_CASE(256)
+    }
+#undef DSDPA_FWD_CASE
+    return DSDPA_ERR_HEAD_DIM;
+}
+
+// element counts are multiples of 4 (D >= 16; workspace segments are 256-byte multiples)
+static inline int zero_fill(float *a, size_t na, float *b, size_t nb, float *c, size_t nc, hipStream_t st)
+{
+    ZeroJob job{{(float4 *)a, (float4 *)b, (float4 *)c}, {na / 4, nb / 4, nc / 4}};
+    size_t big = job.n4[0] > job.n4[1] ? job.n4[0] : job.n4[1];
+    if (job.n4[2] > big) big = job.n4[2];
+    const int threads = 256;
+    size_t blocks = (big + threads - 1) / threads;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(threads), 0, st, job);
+    return check_launch();
+}
+
+// elements per lane in the cell kernel: 4 up to D = 128 (32 lanes per sample at most), 8 beyond.
+// With 4 the kernel holds 64 tap/accumulator registers and runs 4 waves per SIMD; 8 elements per
+// lane at D = 32/64 were measured slower (211 VGPRs, 2 waves per SIMD, latency-bound).
+template <typename S, int D> struct CellChunk {
+    static constexpr int value = D <= 128 ? 4 : 8;
+};
+
+static inline int launch_binning(const float *coords, const Dims &dm, const WorkspaceLayout &wl, char *ws, hipStream_t st)
+{
+    unsigned *counters = (unsigned *)(ws + wl.counters);
+    unsigned *start = (unsigned *)(ws + wl.start);
+    unsigned *sorted = (unsigned *)(ws + wl.sorted);
+    const size_t hist_bytes = (size_t)dm.V * wl.NC * sizeof(unsigned);
+    ScopedKernelTimer timer(3, st);
+    if (2 * hist_bytes <= (size_t)kLdsBytes - 1024) {
+        // LDS-aggregated passes: a workgroup per run of about 8k samples of one (b, s1)
+        int lchunk = 8192 / dm.N;
+        if (lchunk < 1) lchunk = 1;
+        if (lchunk > dm.L) lchunk = dm.L;
+        const int nlc = (dm.L + lchunk - 1) / lchunk;
+        lchunk = (dm.L + nlc - 1) / nlc;
+        const long long blocks = (long long)dm.B * dm.V * nlc;
+        if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+        auto k0 = bin_samples_lds_kernel<0>;
+        auto k1 = bin_samples_lds_kernel<1>;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k0),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)hist_bytes);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k1),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * hist_bytes));
+        if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+        hipLaunchKernelGGL(k0, dim3((unsigned)blocks), dim3(kBinLdsThreads), hist_bytes, st,
+                           coords, dm, wl.NC, lchunk, nlc, counters, sorted);
+        hipLaunchKernelGGL(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st, counters, start, wl.NC);
+        hipLaunchKernelGGL(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
+                           coords, dm, wl.NC, lchunk, nlc, counters, sorted);
+        return check_launch();
+    }
+    const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
+    const long long blocks = (total + kBinThreads - 1) / kBinThreads;
+    if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(bin_samples_kernel<0>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
+                       coords, dm, wl.NC, counters, sorted);
+    hipLaunchKernelGGL(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st, counters, start, wl.NC);
+    hipLaunchKernelGGL(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
+                       coords, dm, wl.NC, counters, sorted);
+    return check_launch();
+}
+
+template <typename S, int D>
+int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const float *coords, const float *lse,
+                         const float *delta, const void *dout, const unsigned *start, const unsigned *sorted,
+                         float *dk_acc, float *dv_acc, const Dims &dm, int NC, hipStream_t st)
+{
+    constexpr int DC = CellChunk<S, D>::value;
+    const long long nwork = (long long)dm.B * dm.H * dm.V * NC;
+    const long long blocks = (nwork + kCellWaves - 1) / kCellWaves;
+    if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+    ScopedKernelTimer timer(1, st);
+    hipLaunchKernelGGL((bwd_dkdv_cell_kernel<S, D, DC>), dim3((unsigned)blocks), dim3(kCellWaves * kWave), 0, st,
+                       q, k, v, coords, lse, delta, dout, start, sorted, dk_acc, dv_acc, dm, NC);
+    return check_launch();
+}
+
+template <typename S>
+int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
+             const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,
+             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    if (!q || !k || !v || !coords || !out || !lse || !dout || !dq || !dk || !dv || !workspace)
+        return DSDPA_ERR_NULL_POINTER;
+    Dims dm;
+    int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
+    if (rc != DSDPA_OK) return rc;
+    if ((long long)dm.L * dm.N > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;   // sample ids are 32-bit
+    hipStream_t st = (hipStream_t)stream;
+    const size_t n = (size_t)dm.rows * D;
+    const WorkspaceLayout wl = workspace_layout(B, V, H, Himg, Wimg, D, P, S::kBytes != 4);
+    char *ws = (char *)workspace;
+    float *delta = (float *)(ws + wl.delta);
+    const int path = g_path.load();
+    const bool fused_atomics = path == DSDPA_PATH_GATHER;
+    const bool cell_binned = path == DSDPA_PATH_AUTO;
+    const bool staged = plane_fits<S>(dm, D);
+    const unsigned *start = (const unsigned *)(ws + wl.start);
+    const unsigned *sorted = (const unsigned *)(ws + wl.sorted);
+    // one launch zeroes the dk/dv accumulators and, for the cell-binned path, the cell counters
+    float *dk_acc = S::kBytes == 4 ? (float *)dk : (float *)(ws + wl.acc);
+    float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
+    rc = zero_fill(dk_acc, n, dv_acc, n, (float *)(ws + wl.counters), cell_binned ? wl.counters_bytes / 4 : 0, st);
+    if (rc != DSDPA_OK) return rc;
+    if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
+#define DSDPA_BWD_CASE(DD)                                                                                      \
+    case DD:                                                                                                    \
+        if (fused_atomics) {                                                                                    \
+            rc = launch_bwd_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st);         \
+        } else {                                                                                                \
+            rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dm, st)        \
+                        : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dm, st);      \
+            if (rc == DSDPA_OK && cell_binned)                                                                  \
+                rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, lse, delta, dout, start, sorted, dk_acc,      \
+                                                 dv_acc, dm, wl.NC, st);                                        \
+            else if (rc == DSDPA_OK)                                                                            \
+                rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, st);    \
+        }                                                                                                       \
+        break;
+    switch (D) {
+        DSDPA_BWD_CASE(16)
+        DSDPA_BWD_CASE(32)
+        DSDPA_BWD_CASE(64)
+        DSDPA_BWD_CASE(128)
+        DSDPA_BWD_CASE(256)
+    default: return DSDPA_ERR_HEAD_DIM;
+    }
+#undef DSDPA_BWD_CASE
+    if (rc != DSDPA_OK) return rc;
+    if (S::kBytes != 4) {
+        const size_t n8 = n / 8;
+        const int threads = 256;
+        size_t blocks = (n8 + threads - 1) / threads;
+        if (blocks > 256 * 16) blocks = 256 * 16;
+        hipLaunchKernelGGL((cast_kernel<S>), dim3((unsigned)blocks), dim3(threads), 0, st, dk_acc, dk, n8);
+        hipLaunchKernelGGL((cast_kernel<S>), dim3((unsigned)blocks), dim3(threads), 0, st, dv_acc, dv, n8);
+        rc = check_launch();
+    }
+    return rc;
+}
+
+}  // namespace dsdpa

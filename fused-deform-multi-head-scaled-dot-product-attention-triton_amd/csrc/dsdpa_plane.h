@@ -123,6 +123,9 @@ __device__ __forceinline__ void stage_row_descriptors(const float2 *__restrict__
 
 // ------------------------------------------------------------------ forward
 // One chunk (cnt <= 64 samples, descriptors at s_w/s_e[dbase ...]) of one row.
+// (Requesting the taps of slot-iteration it+1 before the arithmetic of iteration it -- a hand-made
+// software pipeline -- was measured: no gain for the forward, register spills for dq. The four waves
+// per SIMD already overlap the LDS pipe and the VALU.)
 // CNT > 0 fixes the sample count at compile time (branch-free, fully unrolled chunk).
 template <typename S, int D, int DC, int CNT>
 __device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const float4 *s_w, const int2 *s_e,
