@@ -233,14 +233,19 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : 2) void bwd_dkdv_c
         const unsigned id = id_nxt;
         id_nxt = load_id(c0 + kWave);
         // one list entry per lane: weights and query row
-        const unsigned p = id % (unsigned)dm.P, ql = id / (unsigned)dm.P;      // ql = s1*L + l
-        const unsigned s1 = ql / (unsigned)dm.L, l = ql % (unsigned)dm.L;
+        const unsigned ql = dm.divP.div(id), p = id - ql * (unsigned)dm.P;     // ql = s1*L + l
+        const unsigned s1 = dm.divL.div(ql), l = ql - s1 * (unsigned)dm.L;
         const size_t ci = (((size_t)b * dm.V * dm.L + ql) * dm.V + s2) * (size_t)dm.P + p;
         const float2 xy = coords[ci];
-        const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
+        // Plain bilinear weights, not masked: every sample of this list lies in this cell, whose taps
+        // outside the image were loaded as zeros above and are skipped by the flush below.
+        const float x = ((xy.x * 2.0f - 1.0f) + 1.0f) * ((float)(dm.Wimg - 1) * 0.5f);
+        const float y = ((xy.y * 2.0f - 1.0f) + 1.0f) * ((float)(dm.Himg - 1) * 0.5f);
+        const float fx = x - floorf(x), fy = y - floorf(y);
+        const float gx = 1.0f - fx, gy = 1.0f - fy;
         const unsigned row = (unsigned)((((size_t)b * dm.V + s1) * dm.H + h) * dm.L + l);
         wave_lds_sync();
-        s_w[wave][lane] = make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]);
+        s_w[wave][lane] = make_float4(gx * gy, fx * gy, gx * fy, fx * fy);
         s_row[wave][lane] = row;
         wave_lds_sync();
         const int cnt = (int)min((unsigned)kWave, hi - c0);

@@ -12,10 +12,30 @@ constexpr float kNegBig = -1.0e30f;   // finite stand-in for -inf in running max
 constexpr int kWave = 64;
 constexpr int kXcds = 8;              // MI355X: 8 XCDs, workgroups dealt round-robin
 
+// Division of a 31-bit unsigned by a run-time constant d: q = (n * mul) >> (31 + shift), exact for every
+// n < 2^31 (round-up method: shift = ceil(log2 d), mul = ceil(2^(31+shift) / d) <= 2^32 - 1, or 2^31 for d = 1).
+struct FastDiv {
+    unsigned mul, shift;
+    __host__ static FastDiv make(unsigned d)
+    {
+        FastDiv f;
+        unsigned s = 0;
+        while ((1ull << s) < d) ++s;
+        f.shift = s;
+        f.mul = (unsigned)(((1ull << (31 + s)) + d - 1) / d);
+        return f;
+    }
+    __device__ __forceinline__ unsigned div(unsigned n) const
+    {
+        return (unsigned)(((unsigned long long)n * mul) >> (31 + shift));
+    }
+};
+
 struct Dims {
     int B, V, H, Himg, Wimg, L, P, N;   // N = V*P samples per query row
     int rows;                           // B*V*H*L query rows
     float sm_scale;
+    FastDiv divP, divL;                 // for decoding sample ids (s1*L + l)*P + p
 };
 
 // ------------------------------------------------------------------ storage types

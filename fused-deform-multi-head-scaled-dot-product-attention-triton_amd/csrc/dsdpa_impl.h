@@ -54,6 +54,8 @@ static inline int make_dims(int B, int V, int H, int Himg, int Wimg, int D, int 
         return DSDPA_ERR_TOO_LARGE;
     dm->B = B; dm->V = V; dm->H = H; dm->Himg = Himg; dm->Wimg = Wimg;
     dm->L = (int)L; dm->P = P; dm->N = (int)N; dm->rows = (int)rows; dm->sm_scale = sm_scale;
+    dm->divP = FastDiv::make((unsigned)P);
+    dm->divL = FastDiv::make((unsigned)L);
     return DSDPA_OK;
 }
 
