@@ -112,6 +112,67 @@ __device__ __forceinline__ void load_chunk(const void *p, float (&dst)[DC])
     }
 }
 
+// ---- 16-bit storage: packed pairs straight into the dot-product instructions (no widening) ----
+// DC consecutive 16-bit elements as DC/2 packed pairs.
+template <typename S, int DC>
+__device__ __forceinline__ void load_packed(const void *p, uint32_t (&w)[DC / 2])
+{
+    static_assert(S::kBytes == 2 && DC % 4 == 0, "packed pairs exist for 16-bit storage only");
+    if constexpr (DC % 8 == 0) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(p);
+#pragma unroll
+        for (int i = 0; i < DC / 8; ++i) {
+            uint4 t = src[i];
+            w[4 * i + 0] = t.x; w[4 * i + 1] = t.y; w[4 * i + 2] = t.z; w[4 * i + 3] = t.w;
+        }
+    } else {
+        const uint2 *src = reinterpret_cast<const uint2 *>(p);
+#pragma unroll
+        for (int i = 0; i < DC / 4; ++i) {
+            uint2 t = src[i];
+            w[2 * i + 0] = t.x; w[2 * i + 1] = t.y;
+        }
+    }
+}
+
+typedef __attribute__((ext_vector_type(2))) __bf16 dsdpa_bf16x2;
+typedef __attribute__((ext_vector_type(2))) _Float16 dsdpa_f16x2;
+
+// sum_d a[d] * b[d] over DC elements held as packed pairs: v_dot2_f32_bf16 / v_dot2_f32_f16, products
+// exact in fp32, fp32 accumulation.
+template <typename S, int DC>
+__device__ __forceinline__ float packed_dot(const uint32_t (&a)[DC / 2], const uint32_t (&b)[DC / 2])
+{
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < DC / 2; ++i) {
+        if constexpr (S::kBf16)
+            acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(dsdpa_bf16x2, a[i]),
+                                                  __builtin_bit_cast(dsdpa_bf16x2, b[i]), acc, false);
+        else
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(dsdpa_f16x2, a[i]),
+                                         __builtin_bit_cast(dsdpa_f16x2, b[i]), acc, false);
+    }
+    return acc;
+}
+
+// x . (w.x*tap0 + w.y*tap1 + w.z*tap2 + w.w*tap3) for this lane's DC elements, 16-bit storage: four packed
+// dot products against the un-widened taps, then the bilinear weights on the four scalars (the blend is
+// linear, so it commutes with the dot product).
+template <typename S, int DC>
+__device__ __forceinline__ float tap_dot16(const void *p0, const void *p1, const void *p2, const void *p3,
+                                           const float4 &w, const uint32_t (&x)[DC / 2])
+{
+    uint32_t t0[DC / 2], t1[DC / 2], t2[DC / 2], t3[DC / 2];
+    load_packed<S, DC>(p0, t0);
+    load_packed<S, DC>(p1, t1);
+    load_packed<S, DC>(p2, t2);
+    load_packed<S, DC>(p3, t3);
+    const float d0 = packed_dot<S, DC>(x, t0), d1 = packed_dot<S, DC>(x, t1);
+    const float d2 = packed_dot<S, DC>(x, t2), d3 = packed_dot<S, DC>(x, t3);
+    return fmaf(w.x, d0, fmaf(w.y, d1, fmaf(w.z, d2, w.w * d3)));
+}
+
 // Store DC consecutive fp32 values, narrowed (RNE) to the storage type.
 template <typename S, int DC>
 __device__ __forceinline__ void store_chunk(void *p, const float (&src)[DC])

@@ -114,11 +114,19 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
     const char *vb = (const char *)v_ + rc.kv_base * S::kBytes;
     const float2 *coords = (const float2 *)coords_;
 
+    // fp32 storage: q widened and pre-scaled; 16-bit storage: q kept as packed pairs for the dot-product
+    // instructions and the scale applied to the logit
+    constexpr bool kPacked = S::kBytes == 2;
     float qf[DC];
-    load_chunk<S, DC>((const char *)q_ + (rc.row * D + lane_elem) * S::kBytes, qf);
+    uint32_t qp[kPacked ? DC / 2 : 1];
     const float qscale = dm.sm_scale * kLog2e;
+    if constexpr (kPacked) {
+        load_packed<S, DC>((const char *)q_ + (rc.row * D + lane_elem) * S::kBytes, qp);
+    } else {
+        load_chunk<S, DC>((const char *)q_ + (rc.row * D + lane_elem) * S::kBytes, qf);
 #pragma unroll
-    for (int d = 0; d < DC; ++d) qf[d] *= qscale;
+        for (int d = 0; d < DC; ++d) qf[d] *= qscale;
+    }
 
     float m = kNegBig, lsum = 0.f, acc[DC];
 #pragma unroll
@@ -136,11 +144,18 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
                 int j = it * NS + slot;
                 float4 w = s_w[wave][j];
                 int4 e = s_e[wave][j];
-                float kk[DC];
-                blend_taps<S, DC>(kb, e, w, lane_elem, kk);
                 float dot = 0.f;
+                if constexpr (kPacked) {
+                    dot = qscale * tap_dot16<S, DC>(kb + (size_t)(e.x + lane_elem) * S::kBytes,
+                                                    kb + (size_t)(e.y + lane_elem) * S::kBytes,
+                                                    kb + (size_t)(e.z + lane_elem) * S::kBytes,
+                                                    kb + (size_t)(e.w + lane_elem) * S::kBytes, w, qp);
+                } else {
+                    float kk[DC];
+                    blend_taps<S, DC>(kb, e, w, lane_elem, kk);
 #pragma unroll
-                for (int d = 0; d < DC; ++d) dot = fmaf(qf[d], kk[d], dot);
+                    for (int d = 0; d < DC; ++d) dot = fmaf(qf[d], kk[d], dot);
+                }
                 dot = group_sum<G>(dot);
                 sv[it] = (j < cnt) ? dot : kNegBig;
                 mc = fmaxf(mc, sv[it]);
@@ -314,11 +329,14 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     const char *vb = (const char *)v_ + rc.kv_base * S::kBytes;
     const float2 *coords = (const float2 *)coords_;
 
+    constexpr bool kPacked = S::kBytes == 2;
     float qf[DC], dof[DC], of[DC];
+    uint32_t dop[kPacked ? DC / 2 : 1];
     const size_t roff = (rc.row * D + lane_elem) * S::kBytes;
     load_chunk<S, DC>((const char *)q_ + roff, qf);
     load_chunk<S, DC>((const char *)dout_ + roff, dof);
     load_chunk<S, DC>((const char *)out_ + roff, of);
+    if constexpr (kPacked) load_packed<S, DC>((const char *)dout_ + roff, dop);
     float delta = 0.f;
 #pragma unroll
     for (int d = 0; d < DC; ++d) delta = fmaf(dof[d], of[d], delta);
@@ -340,14 +358,22 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                 int j = it * NS + slot;
                 float4 w = s_w[wave][j];
                 int4 e = s_e[wave][j];
-                float kk[DC], vv[DC];
+                float kk[DC];
                 blend_taps<S, DC>(kb, e, w, lane_elem, kk);
-                blend_taps<S, DC>(vb, e, w, lane_elem, vv);
                 float dot = 0.f, dp = 0.f;
 #pragma unroll
-                for (int d = 0; d < DC; ++d) {
-                    dot = fmaf(qf[d], kk[d], dot);
-                    dp = fmaf(dof[d], vv[d], dp);
+                for (int d = 0; d < DC; ++d) dot = fmaf(qf[d], kk[d], dot);
+                if constexpr (kPacked) {
+                    // dout . v~ needs no widened v~: four packed dot products on the raw taps
+                    dp = tap_dot16<S, DC>(vb + (size_t)(e.x + lane_elem) * S::kBytes,
+                                          vb + (size_t)(e.y + lane_elem) * S::kBytes,
+                                          vb + (size_t)(e.z + lane_elem) * S::kBytes,
+                                          vb + (size_t)(e.w + lane_elem) * S::kBytes, w, dop);
+                } else {
+                    float vv[DC];
+                    blend_taps<S, DC>(vb, e, w, lane_elem, vv);
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) dp = fmaf(dof[d], vv[d], dp);
                 }
                 dot = group_sum<G>(dot);
                 dp = group_sum<G>(dp);

@@ -130,8 +130,10 @@ __device__ __forceinline__ void stage_row_descriptors(const float2 *__restrict__
 template <typename S, int D, int DC, int CNT>
 __device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const float4 *s_w, const int2 *s_e,
                                                 int dbase, int cnt_rt, int slot, int lane_byte,
-                                                const float (&qf)[DC], float &m, float &lsum, float (&acc)[DC])
+                                                const float (&qf)[DC], const uint32_t *qp, float qscale,
+                                                float &m, float &lsum, float (&acc)[DC])
 {
+    constexpr bool kPacked = S::kBytes == 2;
     constexpr int G = D / DC, NS = kWave / G;
     constexpr int ITS = CNT > 0 ? (CNT + NS - 1) / NS : G;
     const int cnt = CNT > 0 ? CNT : cnt_rt;
@@ -146,16 +148,23 @@ __device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const 
             const float4 w = s_w[dbase + j];
             const int2 e = s_e[dbase + j];
             const unsigned char *top = lds + e.x + lane_byte, *bot = lds + e.y + lane_byte;
-            float t0[DC], t1[DC], t2[DC], t3[DC];
-            load_chunk<S, DC>(top, t0);
-            load_chunk<S, DC>(top + 2 * kRow, t1);
-            load_chunk<S, DC>(bot, t2);
-            load_chunk<S, DC>(bot + 2 * kRow, t3);
             float dot = 0.f;
+            if constexpr (kPacked) {
+                uint32_t qq[DC / 2];
 #pragma unroll
-            for (int d = 0; d < DC; ++d) {
-                const float kk = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
-                dot = fmaf(qf[d], kk, dot);
+                for (int i = 0; i < DC / 2; ++i) qq[i] = qp[i];
+                dot = qscale * tap_dot16<S, DC>(top, top + 2 * kRow, bot, bot + 2 * kRow, w, qq);
+            } else {
+                float t0[DC], t1[DC], t2[DC], t3[DC];
+                load_chunk<S, DC>(top, t0);
+                load_chunk<S, DC>(top + 2 * kRow, t1);
+                load_chunk<S, DC>(bot, t2);
+                load_chunk<S, DC>(bot + 2 * kRow, t3);
+#pragma unroll
+                for (int d = 0; d < DC; ++d) {
+                    const float kk = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
+                    dot = fmaf(qf[d], kk, dot);
+                }
             }
             dot = group_sum<G>(dot);
             sv[it] = (j < cnt) ? dot : kNegBig;
@@ -212,7 +221,10 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
 
     zero_plane_pads<S, D>(smem, dm.L);
 
+    // fp32 storage: q widened and pre-scaled (qf); 16-bit storage: q as packed pairs (qp), scale on the logit
+    constexpr bool kPacked = S::kBytes == 2;
     float qf[QW][DC], acc[QW][DC], m[QW], lsum[QW];
+    uint32_t qp[QW][kPacked ? DC / 2 : 1];
     size_t row[QW], crow[QW];
     bool have[QW];
 #pragma unroll
@@ -223,11 +235,17 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
         const int s1 = qc / dm.L, l = qc % dm.L;
         row[qi] = (((size_t)pb.b * dm.V + s1) * dm.H + pb.h) * dm.L + l;
         crow[qi] = (((size_t)pb.b * dm.V + s1) * dm.L + l) * (size_t)dm.N;
-        load_chunk<S, DC>((const char *)q_ + (row[qi] * D + lane_elem) * S::kBytes, qf[qi]);
+        if constexpr (kPacked) {
+            load_packed<S, DC>((const char *)q_ + (row[qi] * D + lane_elem) * S::kBytes, qp[qi]);
+        } else {
+            load_chunk<S, DC>((const char *)q_ + (row[qi] * D + lane_elem) * S::kBytes, qf[qi]);
+#pragma unroll
+            for (int d = 0; d < DC; ++d) qf[qi][d] *= qscale;
+        }
         m[qi] = kNegBig;
         lsum[qi] = 0.f;
 #pragma unroll
-        for (int d = 0; d < DC; ++d) { qf[qi][d] *= qscale; acc[qi][d] = 0.f; }
+        for (int d = 0; d < DC; ++d) acc[qi][d] = 0.f;
     }
 
     for (int s2 = 0; s2 < dm.V; ++s2) {
@@ -238,15 +256,16 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
         __syncthreads();
         if constexpr (PAIR) {
 #pragma unroll
-            for (int qp = 0; qp + 1 < QW; qp += 2) {
-                if (!have[qp]) continue;                       // wave-uniform; rows are consecutive
-                stage_pair_descriptors<S, D>(coords + crow[qp] + (size_t)s2 * dm.P,
-                                             coords + crow[qp + 1] + (size_t)s2 * dm.P, dm.P, lane,
+            for (int qr = 0; qr + 1 < QW; qr += 2) {
+                if (!have[qr]) continue;                       // wave-uniform; rows are consecutive
+                stage_pair_descriptors<S, D>(coords + crow[qr] + (size_t)s2 * dm.P,
+                                             coords + crow[qr + 1] + (size_t)s2 * dm.P, dm.P, lane,
                                              dm.Wimg, dm.Himg, s_w, s_e);
-                fwd_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qf[qp], m[qp], lsum[qp], acc[qp]);
-                if (have[qp + 1])
-                    fwd_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qf[qp + 1], m[qp + 1],
-                                              lsum[qp + 1], acc[qp + 1]);
+                fwd_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qf[qr], qp[qr], qscale,
+                                                m[qr], lsum[qr], acc[qr]);
+                if (have[qr + 1])
+                    fwd_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qf[qr + 1], qp[qr + 1],
+                                                    qscale, m[qr + 1], lsum[qr + 1], acc[qr + 1]);
             }
         } else {
 #pragma unroll
@@ -256,7 +275,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
                 for (int c0 = 0; c0 < dm.P; c0 += kWave) {
                     stage_row_descriptors<S, D>(cq, dm.P, c0, lane, dm.Wimg, dm.Himg, s_w, s_e);
                     fwd_plane_chunk<S, D, DC, 0>(smem, s_w, s_e, 0, min(kWave, dm.P - c0), slot, lane_byte, qf[qi],
-                                              m[qi], lsum[qi], acc[qi]);
+                                                 qp[qi], qscale, m[qi], lsum[qi], acc[qi]);
                 }
             }
         }
@@ -294,11 +313,12 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
 template <typename S, int D, int DC, int CNT>
 __device__ __forceinline__ void dq_plane_chunk(const unsigned char *lds, const float4 *s_w, const int2 *s_e,
                                                int dbase, int cnt_rt, int slot, int lane_byte, float qscale,
-                                               const float (&qf)[DC], const float (&dof)[DC], float lse,
-                                               float delta, float (&dqa)[DC])
+                                               const float (&qf)[DC], const float (&dof)[DC], const uint32_t *dop,
+                                               float lse, float delta, float (&dqa)[DC])
 {
     constexpr int G = D / DC, NS = kWave / G;
     constexpr int kRow = D * S::kBytes;
+    constexpr bool kPacked = S::kBytes == 2;
     const int cnt = CNT > 0 ? CNT : cnt_rt;
     for (int j0 = 0; j0 < cnt; j0 += NS) {
         const int j = j0 + slot;
@@ -320,7 +340,12 @@ __device__ __forceinline__ void dq_plane_chunk(const unsigned char *lds, const f
             }
         }
         __builtin_amdgcn_sched_barrier(0);     // keep the V taps out of the K taps' live range (register budget)
-        {
+        if constexpr (kPacked) {
+            uint32_t dd[DC / 2];
+#pragma unroll
+            for (int i = 0; i < DC / 2; ++i) dd[i] = dop[i];
+            dp = tap_dot16<S, DC>(top + kRow, top + 3 * kRow, bot + kRow, bot + 3 * kRow, w, dd);
+        } else {
             float u0[DC], u1[DC], u2[DC], u3[DC];
             load_chunk<S, DC>(top + kRow, u0);
             load_chunk<S, DC>(top + 3 * kRow, u1);
@@ -363,7 +388,9 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
 
     zero_plane_pads<S, D>(smem, dm.L);
 
+    constexpr bool kPacked = S::kBytes == 2;
     float qf[QW][DC], dof[QW][DC], dqa[QW][DC], lse[QW], delta[QW];
+    uint32_t dop[QW][kPacked ? DC / 2 : 1];      // 16-bit storage: dout as packed pairs for the dp dot products
     size_t row[QW], crow[QW];
     bool have[QW];
 #pragma unroll
@@ -378,6 +405,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
         float of[DC];
         load_chunk<S, DC>((const char *)q_ + roff, qf[qi]);
         load_chunk<S, DC>((const char *)dout_ + roff, dof[qi]);
+        if constexpr (kPacked) load_packed<S, DC>((const char *)dout_ + roff, dop[qi]);
         load_chunk<S, DC>((const char *)out_ + roff, of);
         float dl = 0.f;
 #pragma unroll
@@ -400,11 +428,11 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
                 stage_pair_descriptors<S, D>(coords + crow[qp] + (size_t)s2 * dm.P,
                                              coords + crow[qp + 1] + (size_t)s2 * dm.P, dm.P, lane,
                                              dm.Wimg, dm.Himg, s_w, s_e);
-                dq_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qscale, qf[qp], dof[qp], lse[qp],
-                                         delta[qp], dqa[qp]);
+                dq_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qscale, qf[qp], dof[qp],
+                                               dop[qp], lse[qp], delta[qp], dqa[qp]);
                 if (have[qp + 1])
                     dq_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qscale, qf[qp + 1],
-                                             dof[qp + 1], lse[qp + 1], delta[qp + 1], dqa[qp + 1]);
+                                                   dof[qp + 1], dop[qp + 1], lse[qp + 1], delta[qp + 1], dqa[qp + 1]);
             }
         } else {
 #pragma unroll
@@ -414,7 +442,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
                 for (int c0 = 0; c0 < dm.P; c0 += kWave) {
                     stage_row_descriptors<S, D>(cq, dm.P, c0, lane, dm.Wimg, dm.Himg, s_w, s_e);
                     dq_plane_chunk<S, D, DC, 0>(smem, s_w, s_e, 0, min(kWave, dm.P - c0), slot, lane_byte, qscale,
-                                             qf[qi], dof[qi], lse[qi], delta[qi], dqa[qi]);
+                                                qf[qi], dof[qi], dop[qi], lse[qi], delta[qi], dqa[qi]);
                 }
             }
         }
