@@ -171,7 +171,7 @@ __device__ __forceinline__ void load_tap_or_zero(const char *base, int pix, int 
 }
 
 template <typename S, int D, int DC>
-__global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : 2) void bwd_dkdv_cell_kernel(
+__global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 3 : 2)) void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float *__restrict__ lse_, const float *__restrict__ delta_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
@@ -207,11 +207,24 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : 2) void bwd_dkdv_c
     const size_t plane_base = ((grp * dm.H) + h) * (size_t)dm.L * D;          // elements; grp = b*V + s2
     const char *kb = (const char *)k_ + plane_base * S::kBytes;
     const char *vb = (const char *)v_ + plane_base * S::kBytes;
-    float kt[4][DC], vt[4][DC], aK[4][DC], aV[4][DC];
+    // fp32 storage: the taps widened in registers; 16-bit storage: the taps as packed pairs (half the
+    // registers) feeding the packed dot-product instructions
+    constexpr bool kPacked = S::kBytes == 2;
+    float kt[4][kPacked ? 1 : DC], vt[4][kPacked ? 1 : DC], aK[4][DC], aV[4][DC];
+    uint32_t ktp[4][kPacked ? DC / 2 : 1], vtp[4][kPacked ? DC / 2 : 1];
 #pragma unroll
     for (int tpi = 0; tpi < 4; ++tpi) {
-        load_tap_or_zero<S, DC>(kb, tpix[tpi], D, lane_elem, tv[tpi], kt[tpi]);
-        load_tap_or_zero<S, DC>(vb, tpix[tpi], D, lane_elem, tv[tpi], vt[tpi]);
+        if constexpr (kPacked) {
+#pragma unroll
+            for (int i = 0; i < DC / 2; ++i) { ktp[tpi][i] = 0u; vtp[tpi][i] = 0u; }
+            if (tv[tpi]) {
+                load_packed<S, DC>(kb + ((size_t)tpix[tpi] * D + lane_elem) * S::kBytes, ktp[tpi]);
+                load_packed<S, DC>(vb + ((size_t)tpix[tpi] * D + lane_elem) * S::kBytes, vtp[tpi]);
+            }
+        } else {
+            load_tap_or_zero<S, DC>(kb, tpix[tpi], D, lane_elem, tv[tpi], kt[tpi]);
+            load_tap_or_zero<S, DC>(vb, tpix[tpi], D, lane_elem, tv[tpi], vt[tpi]);
+        }
 #pragma unroll
         for (int d = 0; d < DC; ++d) { aK[tpi][d] = 0.f; aV[tpi][d] = 0.f; }
     }
@@ -260,12 +273,25 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : 2) void bwd_dkdv_c
             load_chunk<S, DC>((const char *)dout_ + (r * D + lane_elem) * S::kBytes, dof);
             const float lse = lse_[r], delta = delta_[r];
             float dot = 0.f, dp = 0.f;
+            if constexpr (kPacked) {
+                // q . k~ = sum_t w_t (q . K_t): packed dot products on the raw 16-bit pairs
+                uint32_t qp[DC / 2], dop[DC / 2];
+                load_packed<S, DC>((const char *)q_ + (r * D + lane_elem) * S::kBytes, qp);
+                load_packed<S, DC>((const char *)dout_ + (r * D + lane_elem) * S::kBytes, dop);
+                dot = fmaf(w.x, packed_dot<S, DC>(qp, ktp[0]),
+                           fmaf(w.y, packed_dot<S, DC>(qp, ktp[1]),
+                                fmaf(w.z, packed_dot<S, DC>(qp, ktp[2]), w.w * packed_dot<S, DC>(qp, ktp[3]))));
+                dp = fmaf(w.x, packed_dot<S, DC>(dop, vtp[0]),
+                          fmaf(w.y, packed_dot<S, DC>(dop, vtp[1]),
+                               fmaf(w.z, packed_dot<S, DC>(dop, vtp[2]), w.w * packed_dot<S, DC>(dop, vtp[3]))));
+            } else {
 #pragma unroll
-            for (int d = 0; d < DC; ++d) {
-                const float kk = fmaf(w.x, kt[0][d], fmaf(w.y, kt[1][d], fmaf(w.z, kt[2][d], w.w * kt[3][d])));
-                const float vv = fmaf(w.x, vt[0][d], fmaf(w.y, vt[1][d], fmaf(w.z, vt[2][d], w.w * vt[3][d])));
-                dot = fmaf(qf[d], kk, dot);
-                dp = fmaf(dof[d], vv, dp);
+                for (int d = 0; d < DC; ++d) {
+                    const float kk = fmaf(w.x, kt[0][d], fmaf(w.y, kt[1][d], fmaf(w.z, kt[2][d], w.w * kt[3][d])));
+                    const float vv = fmaf(w.x, vt[0][d], fmaf(w.y, vt[1][d], fmaf(w.z, vt[2][d], w.w * vt[3][d])));
+                    dot = fmaf(qf[d], kk, dot);
+                    dp = fmaf(dof[d], vv, dp);
+                }
             }
             dot = group_sum<G>(dot);
             dp = group_sum<G>(dp);

@@ -254,11 +254,12 @@ static inline int zero_fill(float *a, size_t na, float *b, size_t nb, float *c, 
     return check_launch();
 }
 
-// elements per lane in the cell kernel: 4 up to D = 128 (32 lanes per sample at most), 8 beyond.
-// With 4 the kernel holds 64 tap/accumulator registers and runs 4 waves per SIMD; 8 elements per
-// lane at D = 32/64 were measured slower (211 VGPRs, 2 waves per SIMD, latency-bound).
+// elements per lane in the cell kernel. fp32: 4 up to D = 128 (64 tap/accumulator registers, 5 waves per
+// SIMD; 8 elements per lane at D = 32/64 were measured slower: 211 VGPRs, 2 waves per SIMD). 16-bit storage
+// keeps the taps packed, so 8 elements per lane fit in ~150 VGPRs and pay off from D = 128 on, where 4 per
+// lane would spread one sample over 32 lanes and repeat the per-sample scalar work in all of them.
 template <typename S, int D> struct CellChunk {
-    static constexpr int value = D <= 128 ? 4 : 8;
+    static constexpr int value = S::kBytes == 2 ? (D <= 64 ? 4 : 8) : (D <= 128 ? 4 : 8);
 };
 
 static inline int launch_binning(const float *coords, const Dims &dm, const WorkspaceLayout &wl, char *ws, hipStream_t st)
