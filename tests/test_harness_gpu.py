@@ -77,3 +77,23 @@ def test_non_default_stream_and_back_to_back_calls():
     side.synchronize()
     assert rel(out, ro) < 1e-4
     assert rel(qg.grad, rdq) < 1e-3 and rel(kg.grad, rdk) < 1e-3 and rel(vg.grad, rdv) < 1e-3
+
+
+def test_large_image_uses_global_binning_path():
+    """A 96x128 image with 2 views has too many cells for the LDS-aggregated binning (V*NC counters do not
+    fit in LDS), so the backward takes the global-atomic counting passes; planes are too big for LDS too."""
+    print("[case] large image, global binning", flush=True)
+    g = torch.Generator().manual_seed(41)
+    B, V, H, Himg, Wimg, D, P = 1, 2, 1, 96, 128, 16, 3
+    L = Himg * Wimg
+    q, k, v = (torch.randn(B, V, H, L, D, generator=g) for _ in range(3))
+    c = torch.rand(B, V, L, V, P, 2, generator=g) * 1.06 - 0.03
+    do = torch.randn(B, V, H, L, D, generator=g)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = deform_sdpa_triton(qg, kg, vg, c.cuda(), Wimg, Himg, 0.25)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    ro, _ = oracle_fwd(q.numpy(), k.numpy(), v.numpy(), c.numpy(), Wimg, Himg, 0.25)
+    rdq, rdk, rdv = oracle_bwd(q.numpy(), k.numpy(), v.numpy(), c.numpy(), do.numpy(), Wimg, Himg, 0.25)
+    assert rel(out, ro) < 1e-4
+    assert rel(qg.grad, rdq) < 1e-3 and rel(kg.grad, rdk) < 1e-3 and rel(vg.grad, rdv) < 1e-3
