@@ -158,7 +158,7 @@ def main():
         sys.exit("bench.py: this build targets one GPU; run with --gpus 1 "
                  "(the operator shards over (batch, head) with no exchange, see DESIGN.md)")
 
-    from workloads import WORKLOADS
+    from workloads import WORKLOADS, oob_fractions
     wl = WORKLOADS[args.workload]
     if args.copy_calibration:
         import torch
@@ -210,6 +210,7 @@ def main():
             wl.algorithmic_bytes("fwd+bwd") / (kernels_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "fwd_bwd_frac_of_roofline_on_step_time":
             wl.algorithmic_bytes("fwd+bwd") / (g["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "coords_outside_image": oob_fractions(wl),
     }
     log("[bench]", json.dumps(details))
 
@@ -223,7 +224,8 @@ def main():
                  "MQS_per_s": w.query_samples / (gg["ms_per_step"] * 1e-3) / 1e6,
                  "per_kernel": kernel_report(w, gg["kernels"]),
                  "fwd_bwd_frac_of_roofline_on_step_time":
-                     w.algorithmic_bytes("fwd+bwd") / (gg["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+                     w.algorithmic_bytes("fwd+bwd") / (gg["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                 "coords_outside_image": oob_fractions(w)}
             log("[bench]", json.dumps(d))
             all_details[name] = d
 

@@ -102,3 +102,22 @@ def gen_inputs(wl, device="cpu", with_dout=True):
     outs = [t.to(dt) for t in outs]
     outs.insert(3, coords)
     return tuple(t.to(device) for t in outs)
+
+
+def oob_fractions(wl):
+    """Fraction of bilinear taps that fall outside the image, and of samples with all four taps outside,
+    for a workload's coordinates (per-tap zero padding: an outside tap contributes nothing)."""
+    gen = torch.Generator().manual_seed(wl.seed)
+    shape = (wl.B, wl.V, wl.H, wl.L, wl.D)
+    for _ in range(3):                      # q, k, v come first in the draw order
+        torch.randn(shape, generator=gen, dtype=torch.float32)
+    c = gen_coords(wl.coords, wl.B, wl.V, wl.L, wl.P, gen)
+    x0 = torch.floor(c[..., 0] * (wl.W_IMG - 1)).to(torch.int64)
+    y0 = torch.floor(c[..., 1] * (wl.H_IMG - 1)).to(torch.int64)
+    inside = []
+    for dy in (0, 1):
+        for dx in (0, 1):
+            inside.append((x0 + dx >= 0) & (x0 + dx < wl.W_IMG) & (y0 + dy >= 0) & (y0 + dy < wl.H_IMG))
+    inside = torch.stack(inside)
+    return {"taps_outside": 1.0 - inside.float().mean().item(),
+            "samples_fully_outside": (~inside.any(dim=0)).float().mean().item()}
