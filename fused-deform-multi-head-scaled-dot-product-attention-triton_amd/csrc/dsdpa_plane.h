@@ -9,15 +9,26 @@
 // planes, barrier, next view. The online-softmax state (forward) or the dq
 // accumulator (backward) of each row stays in registers across the views.
 //
-// LDS image of a view: pixel p of the plane sits at byte (p + 1) * 2*ROW, its K
-// row first and its V row right behind it (ROW = D * element size), with one
-// zeroed pad pixel before pixel 0 and one after pixel L-1. A sample's four taps
-// are then two base addresses -- (row0, x0) and (row1, x0), x0 in [-1, W-1] NOT
-// clamped -- plus compile-time offsets: +2*ROW for the right-hand tap, +ROW for
-// V. A tap that falls outside the image carries weight 0 and reads either a pad
-// or a neighbouring real pixel, never anything non-finite the caller did not
+// LDS image of a view: pixel p of the plane owns the 2*ROW bytes at (p + 1) * 2*ROW
+// (ROW = D * element size), with one zeroed pad pixel before pixel 0 and one after
+// pixel L-1. Slot q = p + 1 holds its K row in the first half when q is even and in
+// the second half when q is odd, the V row in the other half:
+//     K(q) = q*2*ROW + (q & 1)*ROW        V(q) = K(q) ^ ROW
+//     K(q+1) = V(q) + 2*ROW               V(q+1) = K(q) + 2*ROW
+// A sample's four taps are then two base addresses -- K of (row0, x0) and of
+// (row1, x0), x0 in [-1, W-1] NOT clamped -- one XOR each, and compile-time
+// offsets. A tap that falls outside the image carries weight 0 and reads either a
+// pad or a neighbouring real pixel, never anything non-finite the caller did not
 // put there. The gathers are ds_read_b128 of D-contiguous runs, G lanes per
 // sample as in the gather kernels.
+//
+// Why the alternation: the LDS has 64 four-byte banks (256 bytes per clock) and
+// serves a ds_read_b128 32 lanes at a time. A 128-byte row covers half the banks,
+// so four rows gathered by 32 lanes take 2 clocks when two of them lie in each
+// half and up to 4 when they share one (measured: 170 vs 103 bytes/clock/CU). With
+// K always in the first half every K gather would be the 4-clock case. With the
+// alternation the half is the parity of q, and the descriptors of a row are laid
+// out so that consecutive samples alternate parity (paired_position below).
 #pragma once
 #include "dsdpa_common.h"
 
@@ -38,8 +49,8 @@ __device__ __forceinline__ void stage_plane(unsigned char *lds, const char *src,
     const uint4 *s4 = reinterpret_cast<const uint4 *>(src);
     const int n16 = L * kChunksPerRow;
     for (int i = threadIdx.x; i < n16; i += kPlaneWaves * kWave) {
-        const int pix = i / kChunksPerRow, c = i % kChunksPerRow;
-        *reinterpret_cast<uint4 *>(lds + (size_t)(pix + 1) * 2 * kRow + which * kRow + c * 16) = s4[i];
+        const int q = i / kChunksPerRow + 1, c = i % kChunksPerRow;
+        *reinterpret_cast<uint4 *>(lds + (size_t)q * 2 * kRow + ((q & 1) ^ which) * kRow + c * 16) = s4[i];
     }
 }
 
@@ -54,17 +65,36 @@ __device__ __forceinline__ void zero_plane_pads(unsigned char *lds, int L)
     }
 }
 
-// Tap descriptor of one sample: 4 weights and the two base byte offsets (top and
-// bottom tap row) into the interleaved LDS image.
+// Tap descriptor of one sample: 4 weights and the byte offsets of K of the top-left and of the
+// bottom-left tap in the LDS image. Returns the parity of the top-left slot (which half of a 256-byte
+// bank line its K row occupies).
 template <typename S, int D>
-__device__ __forceinline__ void plane_descriptor(float2 xy, bool valid, int Wimg, int Himg, float4 &w, int2 &e)
+__device__ __forceinline__ int plane_descriptor(float2 xy, bool valid, int Wimg, int Himg, float4 &w, int2 &e)
 {
     const Taps tp = make_taps(xy.x, xy.y, Wimg, Himg);
-    constexpr int kPix = 2 * D * S::kBytes;
+    constexpr int kRow = D * S::kBytes;
     const int x0u = min(max(tp.x0, -1), Wimg - 1);
     const int cy0 = min(max(tp.y0, 0), Himg - 1), cy1 = min(max(tp.y0 + 1, 0), Himg - 1);
     w = valid ? make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]) : make_float4(0.f, 0.f, 0.f, 0.f);
-    e = make_int2((cy0 * Wimg + x0u + 1) * kPix, (cy1 * Wimg + x0u + 1) * kPix);
+    const int qt = cy0 * Wimg + x0u + 1, qb = cy1 * Wimg + x0u + 1;
+    e = make_int2((2 * qt + (qt & 1)) * kRow, (2 * qb + (qb & 1)) * kRow);
+    return qt & 1;
+}
+
+// Where lane `lane` parks its sample inside its block of descriptors (block = the lanes in `block`,
+// positions counted from 0): the valid samples first, alternating parity class 0, 1, 0, 1, ... for as
+// long as both classes last, then the rest of the larger class; the invalid lanes (beyond P) behind
+// them. Any four consecutive positions then gather two rows from each half of the bank line.
+__device__ __forceinline__ int paired_position(bool valid, int cls, int lane, unsigned long long block)
+{
+    const unsigned long long m0 = __ballot(valid && cls == 0) & block;
+    const unsigned long long m1 = __ballot(valid && cls != 0) & block;
+    const unsigned long long mi = __ballot(!valid) & block;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    const int n0 = __popcll(m0), n1 = __popcll(m1), np = min(n0, n1);
+    const int r = __popcll((cls ? m1 : m0) & below);
+    const int pos_valid = r < np ? 2 * r + (cls ? 1 : 0) : np + r;
+    return valid ? pos_valid : n0 + n1 + __popcll(mi & below);
 }
 
 struct PlaneBlock {
@@ -97,10 +127,11 @@ __device__ __forceinline__ void stage_pair_descriptors(const float2 *__restrict_
     const float2 xy = ((lane < 32) ? c_even : c_odd)[valid ? n : P - 1];
     float4 w;
     int2 e;
-    plane_descriptor<S, D>(xy, valid, Wimg, Himg, w, e);
+    const int cls = plane_descriptor<S, D>(xy, valid, Wimg, Himg, w, e);
+    const int pos = (lane & 32) + paired_position(valid, cls, lane, lane < 32 ? 0xffffffffull : 0xffffffff00000000ull);
     wave_lds_sync();
-    s_w[lane] = w;
-    s_e[lane] = e;
+    s_w[pos] = w;
+    s_e[pos] = e;
     wave_lds_sync();
 }
 
@@ -114,10 +145,11 @@ __device__ __forceinline__ void stage_row_descriptors(const float2 *__restrict__
     const float2 xy = crow[valid ? n : P - 1];
     float4 w;
     int2 e;
-    plane_descriptor<S, D>(xy, valid, Wimg, Himg, w, e);
+    const int cls = plane_descriptor<S, D>(xy, valid, Wimg, Himg, w, e);
+    const int pos = paired_position(valid, cls, lane, ~0ull);
     wave_lds_sync();
-    s_w[lane] = w;
-    s_e[lane] = e;
+    s_w[pos] = w;
+    s_e[pos] = e;
     wave_lds_sync();
 }
 
@@ -147,19 +179,21 @@ __device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const 
             const int j = it * NS + slot;
             const float4 w = s_w[dbase + j];
             const int2 e = s_e[dbase + j];
-            const unsigned char *top = lds + e.x + lane_byte, *bot = lds + e.y + lane_byte;
+            const int at = e.x + lane_byte, ab = e.y + lane_byte;
+            const unsigned char *top = lds + at, *bot = lds + ab;                                   // K, left taps
+            const unsigned char *topr = lds + (at ^ kRow) + 2 * kRow, *botr = lds + (ab ^ kRow) + 2 * kRow;   // K, right taps
             float dot = 0.f;
             if constexpr (kPacked) {
                 uint32_t qq[DC / 2];
 #pragma unroll
                 for (int i = 0; i < DC / 2; ++i) qq[i] = qp[i];
-                dot = qscale * tap_dot16<S, DC>(top, top + 2 * kRow, bot, bot + 2 * kRow, w, qq);
+                dot = qscale * tap_dot16<S, DC>(top, topr, bot, botr, w, qq);
             } else {
                 float t0[DC], t1[DC], t2[DC], t3[DC];
                 load_chunk<S, DC>(top, t0);
-                load_chunk<S, DC>(top + 2 * kRow, t1);
+                load_chunk<S, DC>(topr, t1);
                 load_chunk<S, DC>(bot, t2);
-                load_chunk<S, DC>(bot + 2 * kRow, t3);
+                load_chunk<S, DC>(botr, t3);
 #pragma unroll
                 for (int d = 0; d < DC; ++d) {
                     const float kk = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
@@ -185,12 +219,12 @@ __device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const 
             lsum += p;
             const float4 w = s_w[dbase + j];
             const int2 e = s_e[dbase + j];
-            const unsigned char *top = lds + e.x + lane_byte + kRow, *bot = lds + e.y + lane_byte + kRow;
+            const int at = e.x + lane_byte, ab = e.y + lane_byte;
             float t0[DC], t1[DC], t2[DC], t3[DC];
-            load_chunk<S, DC>(top, t0);
-            load_chunk<S, DC>(top + 2 * kRow, t1);
-            load_chunk<S, DC>(bot, t2);
-            load_chunk<S, DC>(bot + 2 * kRow, t3);
+            load_chunk<S, DC>(lds + (at ^ kRow), t0);                  // V, left taps
+            load_chunk<S, DC>(lds + at + 2 * kRow, t1);                // V, right taps
+            load_chunk<S, DC>(lds + (ab ^ kRow), t2);
+            load_chunk<S, DC>(lds + ab + 2 * kRow, t3);
             const float c0 = p * w.x, c1 = p * w.y, c2 = p * w.z, c3 = p * w.w;
 #pragma unroll
             for (int d = 0; d < DC; ++d)
@@ -324,15 +358,17 @@ __device__ __forceinline__ void dq_plane_chunk(const unsigned char *lds, const f
         const int j = j0 + slot;
         const float4 w = s_w[dbase + j];
         const int2 e = s_e[dbase + j];
-        const unsigned char *top = lds + e.x + lane_byte, *bot = lds + e.y + lane_byte;
+        const int at = e.x + lane_byte, ab = e.y + lane_byte;
+        const unsigned char *top = lds + at, *bot = lds + ab;                      // K left taps; V right taps at +2*ROW
+        const unsigned char *topx = lds + (at ^ kRow), *botx = lds + (ab ^ kRow);  // V left taps; K right taps at +2*ROW
         float kk[DC];
         float dot = 0.f, dp = 0.f;
         {
             float t0[DC], t1[DC], t2[DC], t3[DC];
             load_chunk<S, DC>(top, t0);
-            load_chunk<S, DC>(top + 2 * kRow, t1);
+            load_chunk<S, DC>(topx + 2 * kRow, t1);
             load_chunk<S, DC>(bot, t2);
-            load_chunk<S, DC>(bot + 2 * kRow, t3);
+            load_chunk<S, DC>(botx + 2 * kRow, t3);
 #pragma unroll
             for (int d = 0; d < DC; ++d) {
                 kk[d] = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
@@ -344,13 +380,13 @@ __device__ __forceinline__ void dq_plane_chunk(const unsigned char *lds, const f
             uint32_t dd[DC / 2];
 #pragma unroll
             for (int i = 0; i < DC / 2; ++i) dd[i] = dop[i];
-            dp = tap_dot16<S, DC>(top + kRow, top + 3 * kRow, bot + kRow, bot + 3 * kRow, w, dd);
+            dp = tap_dot16<S, DC>(topx, top + 2 * kRow, botx, bot + 2 * kRow, w, dd);
         } else {
             float u0[DC], u1[DC], u2[DC], u3[DC];
-            load_chunk<S, DC>(top + kRow, u0);
-            load_chunk<S, DC>(top + 3 * kRow, u1);
-            load_chunk<S, DC>(bot + kRow, u2);
-            load_chunk<S, DC>(bot + 3 * kRow, u3);
+            load_chunk<S, DC>(topx, u0);
+            load_chunk<S, DC>(top + 2 * kRow, u1);
+            load_chunk<S, DC>(botx, u2);
+            load_chunk<S, DC>(bot + 2 * kRow, u3);
 #pragma unroll
             for (int d = 0; d < DC; ++d) {
                 const float vv = fmaf(w.x, u0[d], fmaf(w.y, u1[d], fmaf(w.z, u2[d], w.w * u3[d])));
