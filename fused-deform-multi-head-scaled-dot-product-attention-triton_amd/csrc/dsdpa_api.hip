@@ -14,22 +14,22 @@ KernelTimer g_timer;
 
 extern "C" {
 
-int dsdpa_fwd_f32(const float *q, const float *k, const float *v, const float *coords, float *out, float *lse,
+int dsdpa_fwd_f32(const float *q, const float *k, const float *v, const float *coords, float *out, float *lse, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
 {
-    return fwd_impl<F32>(q, k, v, coords, out, lse, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+    return fwd_impl<F32>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
 }
 
-int dsdpa_fwd_bf16(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
-                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
-{
-    return fwd_impl<BF16>(q, k, v, coords, out, lse, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
-}
-
-int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+int dsdpa_fwd_bf16(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
 {
-    return fwd_impl<F16>(q, k, v, coords, out, lse, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+    return fwd_impl<BF16>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+}
+
+int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse, void *workspace,
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    return fwd_impl<F16>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
 }
 
 int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords, const float *out,
@@ -54,6 +54,13 @@ int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coor
 {
     return bwd_impl<F16>(q, k, v, coords, out, lse, dout, dq, dk, dv, workspace, B, V, H, Himg, Wimg, D, P,
                          sm_scale, stream);
+}
+
+size_t dsdpa_fwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P)
+{
+    if (dtype != DSDPA_F32 && dtype != DSDPA_BF16 && dtype != DSDPA_F16) return 0;
+    if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || D < 1 || P < 1) return 0;
+    return desc_layout(B, V, Himg, Wimg, D, P, dtype != DSDPA_F32 ? 2 : 4).bytes;
 }
 
 size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P)
@@ -88,7 +95,7 @@ int dsdpa_timer_enable(int on)
 
 int dsdpa_timer_collect(int which, double *total_ms, int *launches)
 {
-    if (which < 0 || which > 3 || !total_ms || !launches) return DSDPA_ERR_NULL_POINTER;
+    if (which < 0 || which > 4 || !total_ms || !launches) return DSDPA_ERR_NULL_POINTER;
     double sum = 0.0;
     int n = 0, rc = DSDPA_OK;
     std::vector<EventPair> taken;

@@ -231,6 +231,18 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
     const float qscale = dm.sm_scale * kLog2e;
     const size_t M = (size_t)dm.V * dm.L * dm.P;
     const unsigned *list = sorted + grp * M;
+    // Query rows of this wave's (b, h) are addressed as a uniform base plus a 32-bit byte offset
+    // (s1*H*L + l) * ROW < V*H*L*D*e <= 2^32 (the shape limits keep one batch item of a tensor below 2^30
+    // elements): one add per gather instead of 64-bit address arithmetic per lane.
+    constexpr unsigned kRowBytes = D * S::kBytes;
+    constexpr int kRowToFloatShift = __builtin_ctz(kRowBytes) - 2;         // row byte offset -> float offset
+    const size_t bh_row0 = ((size_t)b * dm.V * dm.H + h) * dm.L;              // row of (b, s1 = 0, h, l = 0)
+    const char *q_bh = (const char *)q_ + bh_row0 * kRowBytes;
+    const char *do_bh = (const char *)dout_ + bh_row0 * kRowBytes;
+    const char *lse_bh = (const char *)(lse_ + bh_row0);
+    const char *delta_bh = (const char *)(delta_ + bh_row0);
+    const unsigned lane_byte = (unsigned)lane_elem * S::kBytes;
+    const unsigned view_rows = (unsigned)dm.H * (unsigned)dm.L;
     const float2 *coords = reinterpret_cast<const float2 *>(coords_);
 
     // Walk the list 64 entries at a time. Sample ids are fetched one chunk ahead
@@ -256,28 +268,28 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
         const float y = ((xy.y * 2.0f - 1.0f) + 1.0f) * ((float)(dm.Himg - 1) * 0.5f);
         const float fx = x - floorf(x), fy = y - floorf(y);
         const float gx = 1.0f - fx, gy = 1.0f - fy;
-        const unsigned row = (unsigned)((((size_t)b * dm.V + s1) * dm.H + h) * dm.L + l);
+        // entries past the end of the list repeat its last sample with zero weights: they add nothing
+        const bool live = c0 + (unsigned)lane < hi;
         wave_lds_sync();
-        s_w[wave][lane] = make_float4(gx * gy, fx * gy, gx * fy, fx * fy);
-        s_row[wave][lane] = row;
+        s_w[wave][lane] = live ? make_float4(gx * gy, fx * gy, gx * fy, fx * fy) : make_float4(0.f, 0.f, 0.f, 0.f);
+        s_row[wave][lane] = (s1 * view_rows + l) * kRowBytes;
         wave_lds_sync();
         const int cnt = (int)min((unsigned)kWave, hi - c0);
         for (int j0 = 0; j0 < cnt; j0 += NS) {
-            const int j = j0 + slot;
-            const bool live = j < cnt;
-            const int jj = live ? j : cnt - 1;
-            const float4 w = s_w[wave][jj];
-            const size_t r = s_row[wave][jj];
+            const float4 w = s_w[wave][j0 + slot];
+            const unsigned r = s_row[wave][j0 + slot];
+            const unsigned roff = r + lane_byte, foff = r >> kRowToFloatShift;
             float qf[DC], dof[DC];
-            load_chunk<S, DC>((const char *)q_ + (r * D + lane_elem) * S::kBytes, qf);
-            load_chunk<S, DC>((const char *)dout_ + (r * D + lane_elem) * S::kBytes, dof);
-            const float lse = lse_[r], delta = delta_[r];
+            load_chunk<S, DC>(q_bh + roff, qf);
+            load_chunk<S, DC>(do_bh + roff, dof);
+            const float lse = *(const float *)(lse_bh + foff), delta = *(const float *)(delta_bh + foff);
+            __builtin_amdgcn_sched_barrier(0);     // all four gathers in flight before the arithmetic starts
             float dot = 0.f, dp = 0.f;
             if constexpr (kPacked) {
                 // q . k~ = sum_t w_t (q . K_t): packed dot products on the raw 16-bit pairs
                 uint32_t qp[DC / 2], dop[DC / 2];
-                load_packed<S, DC>((const char *)q_ + (r * D + lane_elem) * S::kBytes, qp);
-                load_packed<S, DC>((const char *)dout_ + (r * D + lane_elem) * S::kBytes, dop);
+                load_packed<S, DC>(q_bh + roff, qp);
+                load_packed<S, DC>(do_bh + roff, dop);
                 dot = fmaf(w.x, packed_dot<S, DC>(qp, ktp[0]),
                            fmaf(w.y, packed_dot<S, DC>(qp, ktp[1]),
                                 fmaf(w.z, packed_dot<S, DC>(qp, ktp[2]), w.w * packed_dot<S, DC>(qp, ktp[3]))));
@@ -295,7 +307,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
             }
             dot = group_sum<G>(dot);
             dp = group_sum<G>(dp);
-            const float p_n = live ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
+            const float p_n = __builtin_amdgcn_exp2f(dot * qscale - lse);
             const float dss = p_n * (dp - delta) * dm.sm_scale;
             const float ck[4] = { w.x * dss, w.y * dss, w.z * dss, w.w * dss };
             const float cv[4] = { w.x * p_n, w.y * p_n, w.z * p_n, w.w * p_n };

@@ -21,7 +21,7 @@ struct EventPair { hipEvent_t start, stop; };
 struct KernelTimer {
     std::atomic<bool> on{false};
     std::mutex mu;
-    std::vector<EventPair> pairs[4];   // [0] forward, [1] backward dk/dv, [2] backward dq, [3] cell binning
+    std::vector<EventPair> pairs[5];   // [0] forward, [1] backward dk/dv, [2] backward dq, [3] cell binning, [4] descriptor table
 };
 extern KernelTimer g_timer;
 
@@ -56,16 +56,43 @@ inline int check_launch()
     return DSDPA_OK;
 }
 
+// The plane kernels (forward, dq) keep one K and one V plane of a (b, s2, h) in LDS next to their
+// per-wave descriptors; they serve every shape for which that fits in the 160 KB of a gfx950 workgroup.
+constexpr size_t kLdsBytes = 160 * 1024;
+constexpr size_t kPlaneDescLdsBytes = 16 * 64 * (16 + 8);   // 16 waves x 64 samples x (4 weights + 2 offsets)
+inline bool plane_path_fits(size_t L, size_t D, size_t esize)
+{
+    return (L + 2) * 2 * D * esize + kPlaneDescLdsBytes <= kLdsBytes;
+}
+
+// Descriptor table of the plane kernels: per coordinate pair 16 bytes of weights and 4 of packed slot
+// codes, computed once per call by plane_descriptor_kernel. Empty when the plane kernels do not apply.
+struct DescLayout { size_t w, e, bytes; };
+inline size_t round256(size_t b) { return (b + 255) / 256 * 256; }
+inline DescLayout desc_layout(size_t B, size_t V, size_t Himg, size_t Wimg, size_t D, size_t P, size_t esize)
+{
+    DescLayout d{0, 0, 0};
+    const size_t L = Himg * Wimg;
+    if (!plane_path_fits(L, D, esize)) return d;
+    const size_t m = B * V * L * V * P;
+    d.w = 0;
+    d.e = round256(m * 16);
+    d.bytes = d.e + round256(m * 4);
+    return d;
+}
+
+// Forward workspace: the descriptor table alone.
 // Backward workspace, every segment rounded up to 256 bytes:
 //   delta    rows floats                     dout.out per query row
 //   counters B*V*NC u32                      per (batch, key view) cell counts, then fill cursors
 //   start    B*V*(NC+1) u32                  exclusive scan of the counts
 //   sorted   B*V*(V*L*P) u32                 sample ids ordered by cell
 //   acc      2*n floats                      fp32 dk/dv accumulators (16-bit storage only)
+//   desc     20 bytes per coordinate pair    descriptor table (only when the plane kernels apply)
 // with NC = (Himg+1)*(Wimg+1) cells.
-inline size_t round256(size_t b) { return (b + 255) / 256 * 256; }
 struct WorkspaceLayout {
-    size_t delta, counters, start, sorted, acc, total;
+    size_t delta, counters, start, sorted, acc, desc, total;
+    DescLayout dl;
     size_t counters_bytes;
     int NC;
 };
@@ -81,6 +108,8 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     w.start = off; off += round256(B * V * ((size_t)w.NC + 1) * 4);
     w.sorted = off; off += round256(B * V * (V * Himg * Wimg * P) * 4);
     w.acc = off; if (storage16) off += round256(2 * rows * D * 4);
+    w.dl = desc_layout(B, V, Himg, Wimg, D, P, storage16 ? 2 : 4);
+    w.desc = off; off += w.dl.bytes;
     w.total = off;
     return w;
 }
@@ -90,7 +119,7 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
 // three compile in parallel.
 template <typename S>
 int fwd_impl(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
-             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream);
+             void *workspace, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream);
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
              const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,

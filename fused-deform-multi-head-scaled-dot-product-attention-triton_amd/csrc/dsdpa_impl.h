@@ -10,7 +10,7 @@
 
 namespace dsdpa {
 
-constexpr int kLdsBytes = 160 * 1024;                                   // LDS per workgroup on gfx950
+static_assert(kPlaneDescLdsBytes == (size_t)kPlaneDescBytes, "host and device agree on the descriptor block");
 // query rows per wave in the plane kernels: rows * elements-per-lane = 16 keeps them at 128 VGPRs
 template <int DC> struct PlaneRows { static constexpr int value = 16 / DC >= 1 ? 16 / DC : 1; };
 
@@ -164,16 +164,29 @@ int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const floa
     return check_launch();
 }
 
-// The plane kernels need one K and one V plane of a (b, s2, h) in LDS next to the descriptors.
 template <typename S>
 bool plane_fits(const Dims &dm, int D)
 {
-    return (size_t)(dm.L + 2) * 2 * D * S::kBytes + kPlaneDescBytes <= (size_t)kLdsBytes;
+    return plane_path_fits((size_t)dm.L, (size_t)D, S::kBytes);
+}
+
+// Fill the descriptor table of the plane kernels (one thread per coordinate pair, padded to whole waves).
+static inline int launch_plane_descriptors(const float *coords, const Dims &dm, char *table, const DescLayout &dl,
+                                           int timer_slot, hipStream_t st)
+{
+    const long long nblk = (long long)dm.B * dm.V * dm.L * dm.V;
+    const long long waves = dm.P <= 32 ? (nblk + 1) / 2 : nblk * ((dm.P + 63) / 64);
+    const long long blocks = (waves * kWave + kDescThreads - 1) / kDescThreads;
+    if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+    ScopedKernelTimer timer(timer_slot, st);
+    hipLaunchKernelGGL(plane_descriptor_kernel, dim3((unsigned)blocks), dim3(kDescThreads), 0, st, coords, dm,
+                       (float4 *)(table + dl.w), (uint32_t *)(table + dl.e));
+    return check_launch();
 }
 
 template <typename S, int D>
-int launch_fwd_plane(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
-                     const Dims &dm, hipStream_t st)
+int launch_fwd_plane(const void *q, const void *k, const void *v, const float4 *desc_w, const uint32_t *desc_e,
+                     void *out, float *lse, const Dims &dm, hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
     const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes;
@@ -189,12 +202,13 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float *c
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(0, st);
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
-                       q, k, v, coords, out, lse, dm);
+                       q, k, v, desc_w, desc_e, out, lse, dm);
     return check_launch();
 }
 
 template <typename S, int D>
-int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float *coords, const void *out,
+int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float4 *desc_w,
+                        const uint32_t *desc_e, const void *out,
                         const float *lse, const void *dout, void *dq, float *delta, const Dims &dm,
                         hipStream_t st)
 {
@@ -211,23 +225,29 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(2, st);
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
-                       q, k, v, coords, out, lse, dout, dq, delta, dm);
+                       q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, dm);
     return check_launch();
 }
 
 template <typename S>
 int fwd_impl(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
-             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+             void *workspace, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
 {
     if (!q || !k || !v || !coords || !out || !lse) return DSDPA_ERR_NULL_POINTER;
     Dims dm;
     int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
     if (rc != DSDPA_OK) return rc;
     hipStream_t st = (hipStream_t)stream;
-    const bool staged = g_path.load() != DSDPA_PATH_GATHER && plane_fits<S>(dm, D);
+    const DescLayout dl = desc_layout(B, V, Himg, Wimg, D, P, S::kBytes);
+    if (dl.bytes && !workspace) return DSDPA_ERR_NULL_POINTER;
+    const bool staged = g_path.load() != DSDPA_PATH_GATHER && dl.bytes != 0;
+    char *ws = (char *)workspace;
+    if (staged && (rc = launch_plane_descriptors(coords, dm, ws, dl, 4, st)) != DSDPA_OK) return rc;
+    const float4 *desc_w = (const float4 *)(ws + dl.w);
+    const uint32_t *desc_e = (const uint32_t *)(ws + dl.e);
 #define DSDPA_FWD_CASE(DD)                                                                        \
     case DD:                                                                                      \
-        return staged ? launch_fwd_plane<S, DD>(q, k, v, coords, out, lse, dm, st)                \
+        return staged ? launch_fwd_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dm, st)        \
                       : launch_fwd_gather<S, DD>(q, k, v, coords, out, lse, dm, st);
     switch (D) {
         DSDPA_FWD_CASE(16)
@@ -270,8 +290,9 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
     const size_t hist_bytes = (size_t)dm.V * wl.NC * sizeof(unsigned);
     ScopedKernelTimer timer(3, st);
     if (2 * hist_bytes <= (size_t)kLdsBytes - 1024) {
-        // LDS-aggregated passes: a workgroup per run of about 8k samples of one (b, s1)
-        int lchunk = 8192 / dm.N;
+        // LDS-aggregated passes: a workgroup per run of about 4k samples of one (b, s1); 8k when the
+        // histogram is large, since every workgroup walks all of it twice (measured on 18x18 and 48x48)
+        int lchunk = (dm.V * wl.NC < 4096 ? 4096 : 8192) / dm.N;
         if (lchunk < 1) lchunk = 1;
         if (lchunk > dm.L) lchunk = dm.L;
         const int nlc = (dm.L + lchunk - 1) / lchunk;
@@ -338,7 +359,9 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const int path = g_path.load();
     const bool fused_atomics = path == DSDPA_PATH_GATHER;
     const bool cell_binned = path == DSDPA_PATH_AUTO;
-    const bool staged = plane_fits<S>(dm, D);
+    const bool staged = !fused_atomics && wl.dl.bytes != 0;
+    const float4 *desc_w = (const float4 *)(ws + wl.desc + wl.dl.w);
+    const uint32_t *desc_e = (const uint32_t *)(ws + wl.desc + wl.dl.e);
     const unsigned *start = (const unsigned *)(ws + wl.start);
     const unsigned *sorted = (const unsigned *)(ws + wl.sorted);
     // one launch zeroes the dk/dv accumulators and, for the cell-binned path, the cell counters
@@ -346,13 +369,14 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
     rc = zero_fill(dk_acc, n, dv_acc, n, (float *)(ws + wl.counters), cell_binned ? wl.counters_bytes / 4 : 0, st);
     if (rc != DSDPA_OK) return rc;
+    if (staged && (rc = launch_plane_descriptors(coords, dm, ws + wl.desc, wl.dl, 4, st)) != DSDPA_OK) return rc;
     if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
 #define DSDPA_BWD_CASE(DD)                                                                                      \
     case DD:                                                                                                    \
         if (fused_atomics) {                                                                                    \
             rc = launch_bwd_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st);         \
         } else {                                                                                                \
-            rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dm, st)        \
+            rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, dm, st) \
                         : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dm, st);      \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
                 rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, lse, delta, dout, start, sorted, dk_acc,      \

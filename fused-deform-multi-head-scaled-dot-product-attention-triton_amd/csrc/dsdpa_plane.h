@@ -35,6 +35,14 @@
 namespace dsdpa {
 
 constexpr int kPlaneWaves = 16;
+
+// LDS addresses as plain 32-bit numbers: the tap addresses are sums and XORs of byte offsets, and a
+// pointer made from the finished number costs no instruction (adding offsets to a generic pointer to
+// the dynamic LDS block costs an add per pointer). The XOR needs the block aligned to 2*ROW.
+using lds_bytes = __attribute__((address_space(3))) const unsigned char *;
+__device__ __forceinline__ uint32_t lds_offset(const void *p) { return (uint32_t)(size_t)(lds_bytes)p; }
+__device__ __forceinline__ const unsigned char *lds_at(uint32_t off) { return (const unsigned char *)(lds_bytes)(size_t)off; }
+constexpr int kPlaneLdsAlign = 2048;   // 2*ROW for the widest row (D = 256, fp32)
 constexpr int kPlaneDescBytes = kPlaneWaves * kWave * (16 + 8);   // float4 weights + int2 base offsets
 
 template <typename S, int D>
@@ -63,22 +71,6 @@ __device__ __forceinline__ void zero_plane_pads(unsigned char *lds, int L)
         const int pad = i / kChunks, c = i % kChunks;
         *reinterpret_cast<uint4 *>(lds + (size_t)(pad ? L + 1 : 0) * 2 * kRow + c * 16) = make_uint4(0, 0, 0, 0);
     }
-}
-
-// Tap descriptor of one sample: 4 weights and the byte offsets of K of the top-left and of the
-// bottom-left tap in the LDS image. Returns the parity of the top-left slot (which half of a 256-byte
-// bank line its K row occupies).
-template <typename S, int D>
-__device__ __forceinline__ int plane_descriptor(float2 xy, bool valid, int Wimg, int Himg, float4 &w, int2 &e)
-{
-    const Taps tp = make_taps(xy.x, xy.y, Wimg, Himg);
-    constexpr int kRow = D * S::kBytes;
-    const int x0u = min(max(tp.x0, -1), Wimg - 1);
-    const int cy0 = min(max(tp.y0, 0), Himg - 1), cy1 = min(max(tp.y0 + 1, 0), Himg - 1);
-    w = valid ? make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]) : make_float4(0.f, 0.f, 0.f, 0.f);
-    const int qt = cy0 * Wimg + x0u + 1, qb = cy1 * Wimg + x0u + 1;
-    e = make_int2((2 * qt + (qt & 1)) * kRow, (2 * qb + (qb & 1)) * kRow);
-    return qt & 1;
 }
 
 // Where lane `lane` parks its sample inside its block of descriptors (block = the lanes in `block`,
@@ -114,42 +106,86 @@ __device__ __forceinline__ PlaneBlock decode_plane_block(const Dims &dm, int row
     return pb;
 }
 
-// Descriptors for two rows of a wave and one key view in one 64-lane pass (the
-// PAIR instantiations, launched when P <= 32 and QW is even): lanes 0-31 take
-// the even row, 32-63 the odd one, parked at descriptor slots 0.. and 32..
-template <typename S, int D>
-__device__ __forceinline__ void stage_pair_descriptors(const float2 *__restrict__ c_even,
-                                                       const float2 *__restrict__ c_odd, int P, int lane,
-                                                       int Wimg, int Himg, float4 *s_w, int2 *s_e)
+// Descriptor table. The descriptors depend on the coordinates only, not on the head, and computing one
+// costs about as many instructions as consuming two samples; so one small kernel computes them once per
+// call -- one thread per coordinate pair, same order (b, s1, l, s2, p) as the coordinates -- and the
+// plane kernels of all H heads read them back: 16 bytes of weights and the two K slot codes
+// 2*q + (q & 1) (byte offset / ROW, so the table does not depend on the head width or storage type)
+// packed into one 32-bit word. Within every run of up to 64 samples of one (b, s1, l, s2) the entries
+// are stored in paired_position order.
+constexpr int kDescThreads = 256;
+
+static __global__ __launch_bounds__(kDescThreads) void plane_descriptor_kernel(
+    const float *__restrict__ coords_, Dims dm, float4 *__restrict__ desc_w, uint32_t *__restrict__ desc_e)
 {
+    const int lane = threadIdx.x & 63;
+    const long long wave = ((long long)blockIdx.x * kDescThreads + threadIdx.x) >> 6;
+    const long long nblk = (long long)dm.B * dm.V * dm.L * dm.V;        // (b, s1, l, s2) runs of P samples
+    long long blk;
+    int n;                                                              // sample index inside the run
+    unsigned long long group;                                           // lanes that share a run
+    if (dm.P <= 32) {                                                   // two runs per wave
+        blk = wave * 2 + (lane >> 5);
+        n = lane & 31;
+        group = lane < 32 ? 0xffffffffull : 0xffffffff00000000ull;
+    } else {                                                            // one 64-sample piece of a run per wave
+        const int pieces = (dm.P + 63) / 64;
+        blk = wave / pieces;
+        n = (int)(wave % pieces) * 64 + lane;
+        group = ~0ull;
+    }
+    const bool valid = blk < nblk && n < dm.P;
+    const long long src = valid ? blk * dm.P + n : 0;
+    const float2 xy = reinterpret_cast<const float2 *>(coords_)[src];
+    const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
+    const int x0u = min(max(tp.x0, -1), dm.Wimg - 1);
+    const int cy0 = min(max(tp.y0, 0), dm.Himg - 1), cy1 = min(max(tp.y0 + 1, 0), dm.Himg - 1);
+    const int qt = cy0 * dm.Wimg + x0u + 1, qb = cy1 * dm.Wimg + x0u + 1;
+    const int pos = paired_position(valid, qt & 1, lane, group) + (dm.P <= 32 ? 0 : (n & ~63));
+    if (valid) {
+        const long long dst = blk * dm.P + pos;
+        desc_w[dst] = make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]);
+        desc_e[dst] = (uint32_t)(2 * qt + (qt & 1)) | ((uint32_t)(2 * qb + (qb & 1)) << 16);
+    }
+}
+
+// Descriptors for two rows of a wave and one key view in one 64-lane pass (the PAIR instantiations,
+// launched when P <= 32 and QW is even): lanes 0-31 take the even row, 32-63 the odd one, parked at
+// descriptor slots 0.. and 32..   d_even / d_odd: index of the rows' first table entry for this view.
+template <typename S, int D>
+__device__ __forceinline__ void stage_pair_descriptors(const float4 *__restrict__ desc_w,
+                                                       const uint32_t *__restrict__ desc_e, size_t d_even,
+                                                       size_t d_odd, int P, int lane, float4 *s_w, int2 *s_e)
+{
+    constexpr int kRow = D * S::kBytes;
     const int n = lane & 31;
     const bool valid = n < P;
-    const float2 xy = ((lane < 32) ? c_even : c_odd)[valid ? n : P - 1];
-    float4 w;
-    int2 e;
-    const int cls = plane_descriptor<S, D>(xy, valid, Wimg, Himg, w, e);
-    const int pos = (lane & 32) + paired_position(valid, cls, lane, lane < 32 ? 0xffffffffull : 0xffffffff00000000ull);
+    const size_t i = ((lane < 32) ? d_even : d_odd) + (valid ? n : 0);
+    float4 w = desc_w[i];
+    const uint32_t c = desc_e[i];
+    if (!valid) w = make_float4(0.f, 0.f, 0.f, 0.f);
     wave_lds_sync();
-    s_w[pos] = w;
-    s_e[pos] = e;
+    s_w[lane] = w;
+    s_e[lane] = make_int2((int)(c & 0xffffu) * kRow, (int)(c >> 16) * kRow);
     wave_lds_sync();
 }
 
 // One row, samples c0 .. c0+63.
 template <typename S, int D>
-__device__ __forceinline__ void stage_row_descriptors(const float2 *__restrict__ crow, int P, int c0, int lane,
-                                                      int Wimg, int Himg, float4 *s_w, int2 *s_e)
+__device__ __forceinline__ void stage_row_descriptors(const float4 *__restrict__ desc_w,
+                                                      const uint32_t *__restrict__ desc_e, size_t d_row, int P,
+                                                      int c0, int lane, float4 *s_w, int2 *s_e)
 {
+    constexpr int kRow = D * S::kBytes;
     const int n = c0 + lane;
     const bool valid = n < P;
-    const float2 xy = crow[valid ? n : P - 1];
-    float4 w;
-    int2 e;
-    const int cls = plane_descriptor<S, D>(xy, valid, Wimg, Himg, w, e);
-    const int pos = paired_position(valid, cls, lane, ~0ull);
+    const size_t i = d_row + (valid ? n : 0);
+    float4 w = desc_w[i];
+    const uint32_t c = desc_e[i];
+    if (!valid) w = make_float4(0.f, 0.f, 0.f, 0.f);
     wave_lds_sync();
-    s_w[pos] = w;
-    s_e[pos] = e;
+    s_w[lane] = w;
+    s_e[lane] = make_int2((int)(c & 0xffffu) * kRow, (int)(c >> 16) * kRow);
     wave_lds_sync();
 }
 
@@ -160,8 +196,8 @@ __device__ __forceinline__ void stage_row_descriptors(const float2 *__restrict__
 // per SIMD already overlap the LDS pipe and the VALU.)
 // CNT > 0 fixes the sample count at compile time (branch-free, fully unrolled chunk).
 template <typename S, int D, int DC, int CNT>
-__device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const float4 *s_w, const int2 *s_e,
-                                                int dbase, int cnt_rt, int slot, int lane_byte,
+__device__ __forceinline__ void fwd_plane_chunk(uint32_t lbase, const float4 *s_w, const int2 *s_e,
+                                                int dbase, int cnt_rt, int slot,
                                                 const float (&qf)[DC], const uint32_t *qp, float qscale,
                                                 float &m, float &lsum, float (&acc)[DC])
 {
@@ -179,9 +215,9 @@ __device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const 
             const int j = it * NS + slot;
             const float4 w = s_w[dbase + j];
             const int2 e = s_e[dbase + j];
-            const int at = e.x + lane_byte, ab = e.y + lane_byte;
-            const unsigned char *top = lds + at, *bot = lds + ab;                                   // K, left taps
-            const unsigned char *topr = lds + (at ^ kRow) + 2 * kRow, *botr = lds + (ab ^ kRow) + 2 * kRow;   // K, right taps
+            const uint32_t at = e.x + lbase, ab = e.y + lbase;     // lbase: LDS address of the image + this lane's byte
+            const unsigned char *top = lds_at(at), *bot = lds_at(ab);                                          // K, left taps
+            const unsigned char *topr = lds_at((at ^ kRow) + 2 * kRow), *botr = lds_at((ab ^ kRow) + 2 * kRow);   // K, right taps
             float dot = 0.f;
             if constexpr (kPacked) {
                 uint32_t qq[DC / 2];
@@ -219,12 +255,12 @@ __device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const 
             lsum += p;
             const float4 w = s_w[dbase + j];
             const int2 e = s_e[dbase + j];
-            const int at = e.x + lane_byte, ab = e.y + lane_byte;
+            const uint32_t at = e.x + lbase, ab = e.y + lbase;
             float t0[DC], t1[DC], t2[DC], t3[DC];
-            load_chunk<S, DC>(lds + (at ^ kRow), t0);                  // V, left taps
-            load_chunk<S, DC>(lds + at + 2 * kRow, t1);                // V, right taps
-            load_chunk<S, DC>(lds + (ab ^ kRow), t2);
-            load_chunk<S, DC>(lds + ab + 2 * kRow, t3);
+            load_chunk<S, DC>(lds_at(at ^ kRow), t0);                  // V, left taps
+            load_chunk<S, DC>(lds_at(at + 2 * kRow), t1);              // V, right taps
+            load_chunk<S, DC>(lds_at(ab ^ kRow), t2);
+            load_chunk<S, DC>(lds_at(ab + 2 * kRow), t3);
             const float c0 = p * w.x, c1 = p * w.y, c2 = p * w.z, c3 = p * w.w;
 #pragma unroll
             for (int d = 0; d < DC; ++d)
@@ -237,11 +273,12 @@ __device__ __forceinline__ void fwd_plane_chunk(const unsigned char *lds, const 
 template <typename S, int D, int DC, int QW, bool PAIR, int PCNT>
 __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
-    const float *__restrict__ coords_, void *__restrict__ out_, float *__restrict__ lse_, Dims dm)
+    const float4 *__restrict__ desc_w, const uint32_t *__restrict__ desc_e, void *__restrict__ out_,
+    float *__restrict__ lse_, Dims dm)
 {
     constexpr int G = D / DC;
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    extern __shared__ __attribute__((aligned(kPlaneLdsAlign))) unsigned char smem[];
     const int img_bytes = plane_lds_bytes<S, D>(dm.L);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
@@ -251,7 +288,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
     const int nq = dm.V * dm.L;
     const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
     const float qscale = dm.sm_scale * kLog2e;
-    const float2 *coords = reinterpret_cast<const float2 *>(coords_);
+    const uint32_t lbase = lds_offset(smem) + lane_byte;
 
     zero_plane_pads<S, D>(smem, dm.L);
 
@@ -292,23 +329,22 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
 #pragma unroll
             for (int qr = 0; qr + 1 < QW; qr += 2) {
                 if (!have[qr]) continue;                       // wave-uniform; rows are consecutive
-                stage_pair_descriptors<S, D>(coords + crow[qr] + (size_t)s2 * dm.P,
-                                             coords + crow[qr + 1] + (size_t)s2 * dm.P, dm.P, lane,
-                                             dm.Wimg, dm.Himg, s_w, s_e);
-                fwd_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qf[qr], qp[qr], qscale,
+                stage_pair_descriptors<S, D>(desc_w, desc_e, crow[qr] + (size_t)s2 * dm.P,
+                                             crow[qr + 1] + (size_t)s2 * dm.P, dm.P, lane, s_w, s_e);
+                fwd_plane_chunk<S, D, DC, PCNT>(lbase, s_w, s_e, 0, dm.P, slot, qf[qr], qp[qr], qscale,
                                                 m[qr], lsum[qr], acc[qr]);
                 if (have[qr + 1])
-                    fwd_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qf[qr + 1], qp[qr + 1],
+                    fwd_plane_chunk<S, D, DC, PCNT>(lbase, s_w, s_e, 32, dm.P, slot, qf[qr + 1], qp[qr + 1],
                                                     qscale, m[qr + 1], lsum[qr + 1], acc[qr + 1]);
             }
         } else {
 #pragma unroll
             for (int qi = 0; qi < QW; ++qi) {
                 if (!have[qi]) continue;
-                const float2 *cq = coords + crow[qi] + (size_t)s2 * dm.P;
+                const size_t cq = crow[qi] + (size_t)s2 * dm.P;
                 for (int c0 = 0; c0 < dm.P; c0 += kWave) {
-                    stage_row_descriptors<S, D>(cq, dm.P, c0, lane, dm.Wimg, dm.Himg, s_w, s_e);
-                    fwd_plane_chunk<S, D, DC, 0>(smem, s_w, s_e, 0, min(kWave, dm.P - c0), slot, lane_byte, qf[qi],
+                    stage_row_descriptors<S, D>(desc_w, desc_e, cq, dm.P, c0, lane, s_w, s_e);
+                    fwd_plane_chunk<S, D, DC, 0>(lbase, s_w, s_e, 0, min(kWave, dm.P - c0), slot, qf[qi],
                                                  qp[qi], qscale, m[qi], lsum[qi], acc[qi]);
                 }
             }
@@ -345,8 +381,8 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
 
 // ------------------------------------------------------------------ backward: dq and delta
 template <typename S, int D, int DC, int CNT>
-__device__ __forceinline__ void dq_plane_chunk(const unsigned char *lds, const float4 *s_w, const int2 *s_e,
-                                               int dbase, int cnt_rt, int slot, int lane_byte, float qscale,
+__device__ __forceinline__ void dq_plane_chunk(uint32_t lbase, const float4 *s_w, const int2 *s_e,
+                                               int dbase, int cnt_rt, int slot, float qscale,
                                                const float (&qf)[DC], const float (&dof)[DC], const uint32_t *dop,
                                                float lse, float delta, float (&dqa)[DC])
 {
@@ -358,9 +394,9 @@ __device__ __forceinline__ void dq_plane_chunk(const unsigned char *lds, const f
         const int j = j0 + slot;
         const float4 w = s_w[dbase + j];
         const int2 e = s_e[dbase + j];
-        const int at = e.x + lane_byte, ab = e.y + lane_byte;
-        const unsigned char *top = lds + at, *bot = lds + ab;                      // K left taps; V right taps at +2*ROW
-        const unsigned char *topx = lds + (at ^ kRow), *botx = lds + (ab ^ kRow);  // V left taps; K right taps at +2*ROW
+        const uint32_t at = e.x + lbase, ab = e.y + lbase;
+        const unsigned char *top = lds_at(at), *bot = lds_at(ab);                      // K left taps; V right taps at +2*ROW
+        const unsigned char *topx = lds_at(at ^ kRow), *botx = lds_at(ab ^ kRow);      // V left taps; K right taps at +2*ROW
         float kk[DC];
         float dot = 0.f, dp = 0.f;
         {
@@ -405,12 +441,13 @@ __device__ __forceinline__ void dq_plane_chunk(const unsigned char *lds, const f
 template <typename S, int D, int DC, int QW, bool PAIR, int PCNT>
 __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
-    const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
-    const void *__restrict__ dout_, void *__restrict__ dq_, float *__restrict__ delta_, Dims dm)
+    const float4 *__restrict__ desc_w, const uint32_t *__restrict__ desc_e, const void *__restrict__ out_,
+    const float *__restrict__ lse_, const void *__restrict__ dout_, void *__restrict__ dq_,
+    float *__restrict__ delta_, Dims dm)
 {
     constexpr int G = D / DC;
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    extern __shared__ __attribute__((aligned(kPlaneLdsAlign))) unsigned char smem[];
     const int img_bytes = plane_lds_bytes<S, D>(dm.L);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
@@ -420,7 +457,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
     const int nq = dm.V * dm.L;
     const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
     const float qscale = dm.sm_scale * kLog2e;
-    const float2 *coords = reinterpret_cast<const float2 *>(coords_);
+    const uint32_t lbase = lds_offset(smem) + lane_byte;
 
     zero_plane_pads<S, D>(smem, dm.L);
 
@@ -461,23 +498,22 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
 #pragma unroll
             for (int qp = 0; qp + 1 < QW; qp += 2) {
                 if (!have[qp]) continue;
-                stage_pair_descriptors<S, D>(coords + crow[qp] + (size_t)s2 * dm.P,
-                                             coords + crow[qp + 1] + (size_t)s2 * dm.P, dm.P, lane,
-                                             dm.Wimg, dm.Himg, s_w, s_e);
-                dq_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 0, dm.P, slot, lane_byte, qscale, qf[qp], dof[qp],
+                stage_pair_descriptors<S, D>(desc_w, desc_e, crow[qp] + (size_t)s2 * dm.P,
+                                             crow[qp + 1] + (size_t)s2 * dm.P, dm.P, lane, s_w, s_e);
+                dq_plane_chunk<S, D, DC, PCNT>(lbase, s_w, s_e, 0, dm.P, slot, qscale, qf[qp], dof[qp],
                                                dop[qp], lse[qp], delta[qp], dqa[qp]);
                 if (have[qp + 1])
-                    dq_plane_chunk<S, D, DC, PCNT>(smem, s_w, s_e, 32, dm.P, slot, lane_byte, qscale, qf[qp + 1],
+                    dq_plane_chunk<S, D, DC, PCNT>(lbase, s_w, s_e, 32, dm.P, slot, qscale, qf[qp + 1],
                                                    dof[qp + 1], dop[qp + 1], lse[qp + 1], delta[qp + 1], dqa[qp + 1]);
             }
         } else {
 #pragma unroll
             for (int qi = 0; qi < QW; ++qi) {
                 if (!have[qi]) continue;
-                const float2 *cq = coords + crow[qi] + (size_t)s2 * dm.P;
+                const size_t cq = crow[qi] + (size_t)s2 * dm.P;
                 for (int c0 = 0; c0 < dm.P; c0 += kWave) {
-                    stage_row_descriptors<S, D>(cq, dm.P, c0, lane, dm.Wimg, dm.Himg, s_w, s_e);
-                    dq_plane_chunk<S, D, DC, 0>(smem, s_w, s_e, 0, min(kWave, dm.P - c0), slot, lane_byte, qscale,
+                    stage_row_descriptors<S, D>(desc_w, desc_e, cq, dm.P, c0, lane, s_w, s_e);
+                    dq_plane_chunk<S, D, DC, 0>(lbase, s_w, s_e, 0, min(kWave, dm.P - c0), slot, qscale,
                                                 qf[qi], dof[qi], dop[qi], lse[qi], delta[qi], dqa[qi]);
                 }
             }

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libdsdpa.so")
 SYMBOLS = (
     "dsdpa_fwd_f32", "dsdpa_fwd_bf16", "dsdpa_fwd_f16",
     "dsdpa_bwd_f32", "dsdpa_bwd_bf16", "dsdpa_bwd_f16",
-    "dsdpa_bwd_workspace_bytes", "dsdpa_error_string", "dsdpa_last_hip_error",
+    "dsdpa_fwd_workspace_bytes", "dsdpa_bwd_workspace_bytes", "dsdpa_error_string", "dsdpa_last_hip_error",
     "dsdpa_version", "dsdpa_set_path", "dsdpa_timer_enable", "dsdpa_timer_collect",
 )
 
@@ -42,11 +42,13 @@ def load():
     dims = [i, i, i, i, i, i, i, f, vp]            # B V H Himg Wimg D P sm_scale stream
     for sfx in ("f32", "bf16", "f16"):
         fwd = getattr(lib, "dsdpa_fwd_" + sfx)
-        fwd.argtypes = [vp] * 6 + dims
+        fwd.argtypes = [vp] * 7 + dims          # q k v coords out lse workspace
         fwd.restype = i
         bwd = getattr(lib, "dsdpa_bwd_" + sfx)
         bwd.argtypes = [vp] * 11 + dims
         bwd.restype = i
+    lib.dsdpa_fwd_workspace_bytes.argtypes = [i] * 8
+    lib.dsdpa_fwd_workspace_bytes.restype = ctypes.c_size_t
     lib.dsdpa_bwd_workspace_bytes.argtypes = [i] * 8
     lib.dsdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.dsdpa_error_string.argtypes = [i]

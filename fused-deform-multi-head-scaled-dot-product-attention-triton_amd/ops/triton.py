@@ -76,9 +76,12 @@ class _fused_deform_sdpa(torch.autograd.Function):
             coords = coords.float()
         out = torch.empty_like(q)
         lse = torch.empty((B, V, H, L), device=q.device, dtype=torch.float32)
+        ws_bytes = lib.dsdpa_fwd_workspace_bytes(_DTYPE_CODE[q.dtype], B, V, H, HEIGHT, WIDTH, D, P)
+        ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)     # scratch, not saved for backward
         with torch.cuda.device(q.device):
             rc = getattr(lib, "dsdpa_fwd_" + sfx)(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), coords.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                ws.data_ptr() if ws_bytes else None,
                 B, V, H, HEIGHT, WIDTH, D, P, float(sm_scale), _stream_ptr(q.device))
         _native.check(rc)
         ctx.save_for_backward(q, k, v, coords, out, lse)

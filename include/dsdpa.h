@@ -59,17 +59,22 @@ enum { DSDPA_F32 = 0, DSDPA_BF16 = 1, DSDPA_F16 = 2 };
  * Forward: replaces the `_fwd_kernel[grid](...)` launch, ops/triton.py:396-411,
  * including the coords clone/scale (:381-383) and the zero-fill of `o` (:389).
  * Writes out (storage dtype) and lse (fp32).
+ *
+ * `workspace` must hold dsdpa_fwd_workspace_bytes(...) bytes (256-byte aligned; may be NULL when that is
+ * 0). It is scratch for the duration of the call on `stream`: a table of the bilinear weights and tap
+ * addresses of every coordinate pair, computed once from coords and shared by all H heads (the
+ * reference recomputes them per head inside `_fwd_kernel`, ops/triton.py:118-140).
  */
 int dsdpa_fwd_f32(const float *q, const float *k, const float *v, const float *coords,
-                  float *out, float *lse,
+                  float *out, float *lse, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
                   float sm_scale, void *stream);
 int dsdpa_fwd_bf16(const void *q, const void *k, const void *v, const float *coords,
-                   void *out, float *lse,
+                   void *out, float *lse, void *workspace,
                    int B, int V, int H, int Himg, int Wimg, int D, int P,
                    float sm_scale, void *stream);
 int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coords,
-                  void *out, float *lse,
+                  void *out, float *lse, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
                   float sm_scale, void *stream);
 
@@ -86,7 +91,7 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
  * bilinear cell (one u32 per coordinate pair plus the cell offsets; it depends on
  * coords only and is shared by all heads) and, for bf16/fp16, the fp32 dk/dv
  * accumulators that are rounded to the storage type at the end (fp32: dk and dv
- * are themselves the accumulators). Accumulation order into dk/dv is not deterministic (float atomics,
+ * are themselves the accumulators), and the same per-coordinate table as the forward's. Accumulation order into dk/dv is not deterministic (float atomics,
  * as in the reference, ops/triton.py:345-360).
  */
 int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords,
@@ -104,6 +109,11 @@ int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coor
                   void *dq, void *dk, void *dv, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
                   float sm_scale, void *stream);
+
+/* Bytes of device workspace dsdpa_fwd_* needs for a storage dtype: 20 bytes per coordinate pair when the
+ * K and V planes of one view fit in LDS (the staged kernels), else 0; 0 also if an argument is invalid.
+ * No counterpart in the reference. */
+size_t dsdpa_fwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P);
 
 /* Bytes of device workspace dsdpa_bwd_* needs for a storage dtype (0 if an argument is invalid).
  * Counterpart of the reference's delta and dk32/dv32 temporaries, ops/triton.py:428-430. */
@@ -139,7 +149,8 @@ int dsdpa_set_path(int path);
  * HIP events recorded on the launch stream. dsdpa_timer_collect waits for the
  * recorded events, returns the summed kernel time and the number of launches
  * for `which` (0 = forward kernel, 1 = backward dk/dv kernel, 2 = backward dq
- * kernel, 3 = the three cell-binning launches taken together) and releases them.
+ * kernel, 3 = the three cell-binning launches taken together, 4 = the launches
+ * that fill the per-coordinate table, one per forward and one per backward call) and releases them.
  * dsdpa_timer_enable returns the previous state.
  */
 int dsdpa_timer_enable(int on);

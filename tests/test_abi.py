@@ -40,14 +40,27 @@ def test_workspace_bytes():
     lib = _native.load()
     r256 = lambda b: (b + 255) // 256 * 256
 
+    def table(B, V, Himg, Wimg, D, P, storage16):
+        """per-coordinate table of the staged kernels: only when one K and one V plane fit in LDS"""
+        L, e = Himg * Wimg, 2 if storage16 else 4
+        if (L + 2) * 2 * D * e + 16 * 64 * 24 > 160 * 1024:
+            return 0
+        m = B * V * L * V * P
+        return r256(m * 16) + r256(m * 4)
+
     def expect(B, V, H, Himg, Wimg, D, P, storage16):
         rows, NC = B * V * H * Himg * Wimg, (Himg + 1) * (Wimg + 1)
         total = r256(rows * 4) + r256(B * V * NC * 4) + r256(B * V * (NC + 1) * 4) + r256(B * V * V * Himg * Wimg * P * 4)
-        return total + (r256(2 * rows * D * 4) if storage16 else 0)
+        total += r256(2 * rows * D * 4) if storage16 else 0
+        return total + table(B, V, Himg, Wimg, D, P, storage16)
 
     assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32) == expect(2, 6, 8, 18, 18, 32, 32, False)
     assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64, 32) == expect(2, 6, 8, 48, 48, 64, 32, True)
     assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F16, 1, 2, 1, 3, 5, 16, 7) == expect(1, 2, 1, 3, 5, 16, 7, True)
+    assert lib.dsdpa_fwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32) == table(2, 6, 18, 18, 32, 32, False) > 0
+    assert lib.dsdpa_fwd_workspace_bytes(_native.DSDPA_F16, 1, 2, 1, 3, 5, 16, 7) == table(1, 2, 3, 5, 16, 7, True) > 0
+    assert lib.dsdpa_fwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64, 32) == 0      # planes too large for LDS
+    assert lib.dsdpa_fwd_workspace_bytes(7, 2, 6, 8, 18, 18, 32, 32) == 0
     assert lib.dsdpa_bwd_workspace_bytes(7, 2, 6, 8, 48, 48, 64, 32) == 0
     assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 0, 6, 8, 48, 48, 64, 32) == 0
 
@@ -57,11 +70,12 @@ def test_argument_validation_before_launch():
     lib = _native.load()
     fake = ctypes.c_void_p(0x1000)   # never dereferenced: validation fails first
     ok_dims = (1, 2, 2, 3, 4, 32, 2, 0.5, None)
-    assert lib.dsdpa_fwd_f32(None, fake, fake, fake, fake, fake, *ok_dims) == 1
-    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, 0, 2, 2, 3, 4, 32, 2, 0.5, None) == 2
-    assert lib.dsdpa_fwd_bf16(fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 48, 2, 0.5, None) == 3
-    assert lib.dsdpa_fwd_f16(fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 8, 2, 0.5, None) == 3
-    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, 1, 64, 64, 1024, 1024, 256, 2, 0.5, None) == 4
+    assert lib.dsdpa_fwd_f32(None, fake, fake, fake, fake, fake, fake, *ok_dims) == 1
+    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, None, *ok_dims) == 1    # this shape needs the workspace
+    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 0, 2, 2, 3, 4, 32, 2, 0.5, None) == 2
+    assert lib.dsdpa_fwd_bf16(fake, fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 48, 2, 0.5, None) == 3
+    assert lib.dsdpa_fwd_f16(fake, fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 8, 2, 0.5, None) == 3
+    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 1, 64, 64, 1024, 1024, 256, 2, 0.5, None) == 4
     # backward: the workspace is required
     args = [fake] * 10
     assert lib.dsdpa_bwd_bf16(*args, None, *ok_dims) == 1

@@ -122,8 +122,12 @@ def test_lse_through_c_abi():
     qg, kg, vg, cg = (t.to(dev).contiguous() for t in (q, k, v, c))
     out = torch.empty_like(qg)
     lse = torch.empty(q.shape[:4], device=dev, dtype=torch.float32)
+    ws = torch.empty(lib.dsdpa_fwd_workspace_bytes(_native.DSDPA_F32, 2, 3, 2, 6, 4, 32, 23), device=dev,
+                     dtype=torch.uint8)
+    assert ws.numel() > 0
     rc = lib.dsdpa_fwd_f32(qg.data_ptr(), kg.data_ptr(), vg.data_ptr(), cg.data_ptr(), out.data_ptr(),
-                           lse.data_ptr(), 2, 3, 2, 6, 4, 32, 23, 0.2, torch.cuda.current_stream().cuda_stream)
+                           lse.data_ptr(), ws.data_ptr(), 2, 3, 2, 6, 4, 32, 23, 0.2,
+                           torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
     ro, rl = oracle_fwd(q.numpy(), k.numpy(), v.numpy(), c.numpy(), 4, 6, 0.2)
@@ -213,8 +217,10 @@ def test_named_workloads_full_size(name):
 
 
 def test_peak_memory_is_linear_in_tensor_size():
-    """No sampled-tensor materialisation: fwd+bwd peak stays within a small multiple of
-    the q/k/v/out/grad tensors (the eager path needs 2*QS*D*4 bytes = 1.5 GB here)."""
+    """No sampled-tensor materialisation: the fwd+bwd peak is out, dq, dk, dv plus scratch proportional to
+    the coordinates (20 bytes of tap table and 4 of cell ordering per 8-byte coordinate pair, shared by all
+    heads) -- nothing that scales with samples x head width (the eager path needs 2*QS*D*4 bytes = 1.5 GB
+    here)."""
     wl = WORKLOADS["C2"]
     say("[case] peak memory C2")
     q, k, v, c, do = gen_inputs(wl, device="cuda")
@@ -227,4 +233,5 @@ def test_peak_memory_is_linear_in_tensor_size():
     torch.cuda.synchronize()
     extra = torch.cuda.max_memory_allocated() - base
     tensor_bytes = q.numel() * q.element_size()
-    assert extra <= 8 * tensor_bytes, (extra, tensor_bytes)
+    coords_bytes = c.numel() * c.element_size()
+    assert extra <= 5 * tensor_bytes + 4 * coords_bytes, (extra, tensor_bytes, coords_bytes)
