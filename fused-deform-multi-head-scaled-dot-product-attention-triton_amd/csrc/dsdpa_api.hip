@@ -33,26 +33,26 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
 }
 
 int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords, const float *out,
-                  const float *lse, const float *dout, float *dq, float *dk, float *dv, void *workspace,
+                  const float *lse, const float *dout, float *dq, float *dk, float *dv, float *dcoords, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
 {
-    return bwd_impl<F32>(q, k, v, coords, out, lse, dout, dq, dk, dv, workspace, B, V, H, Himg, Wimg, D, P,
+    return bwd_impl<F32>(q, k, v, coords, out, lse, dout, dq, dk, dv, dcoords, workspace, B, V, H, Himg, Wimg, D, P,
                          sm_scale, stream);
 }
 
 int dsdpa_bwd_bf16(const void *q, const void *k, const void *v, const float *coords, const void *out,
-                   const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,
+                   const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
                    int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
 {
-    return bwd_impl<BF16>(q, k, v, coords, out, lse, dout, dq, dk, dv, workspace, B, V, H, Himg, Wimg, D, P,
+    return bwd_impl<BF16>(q, k, v, coords, out, lse, dout, dq, dk, dv, dcoords, workspace, B, V, H, Himg, Wimg, D, P,
                           sm_scale, stream);
 }
 
 int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coords, const void *out,
-                  const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,
+                  const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
 {
-    return bwd_impl<F16>(q, k, v, coords, out, lse, dout, dq, dk, dv, workspace, B, V, H, Himg, Wimg, D, P,
+    return bwd_impl<F16>(q, k, v, coords, out, lse, dout, dq, dk, dv, dcoords, workspace, B, V, H, Himg, Wimg, D, P,
                          sm_scale, stream);
 }
 

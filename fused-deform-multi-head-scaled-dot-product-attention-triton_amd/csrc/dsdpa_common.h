@@ -248,6 +248,43 @@ __device__ __forceinline__ Taps make_taps(float cx, float cy, int Wimg, int Himg
     return t;
 }
 
+// Derivatives of the four masked weights of make_taps by the NORMALISED coordinates: with the tap order
+// 00, 01, 10, 11 and x_pix = x*(W-1), y_pix = y*(Himg-1),
+//   d w/dx = (W-1)    * [-(1-fy), (1-fy), -fy, fy]      d w/dy = (Himg-1) * [-(1-fx), -fx, (1-fx), fx]
+// each zeroed for a tap outside the image (that tap contributes nothing, so it has no gradient
+// either: the rule of ATen's bilinear grid_sampler backward, which ops/torch.py:14-15 differentiates
+// through). floor() makes the sample piecewise smooth; on a cell border this is the one-sided
+// derivative of the cell floor() picks, as in ATen.
+struct TapGrads { float gx[4], gy[4]; };
+
+__device__ __forceinline__ TapGrads make_tap_grads(float cx, float cy, int Wimg, int Himg)
+{
+    float gxn = cx * 2.0f - 1.0f;
+    float gyn = cy * 2.0f - 1.0f;
+    float x = (gxn + 1.0f) * ((float)(Wimg - 1) * 0.5f);
+    float y = (gyn + 1.0f) * ((float)(Himg - 1) * 0.5f);
+    float x0f = floorf(x), y0f = floorf(y);
+    float fx = x - x0f, fy = y - y0f;
+    x0f = fminf(fmaxf(x0f, -2.0f), (float)Wimg + 1.0f);
+    y0f = fminf(fmaxf(y0f, -2.0f), (float)Himg + 1.0f);
+    int x0 = (int)x0f, y0 = (int)y0f;
+    int x1 = x0 + 1, y1 = y0 + 1;
+    bool vx0 = (x0 >= 0) & (x0 < Wimg), vx1 = (x1 >= 0) & (x1 < Wimg);
+    bool vy0 = (y0 >= 0) & (y0 < Himg), vy1 = (y1 >= 0) & (y1 < Himg);
+    bool fin = (x == x) & (y == y);                       // NaN coordinates: no taps, no gradient
+    const float sx = (float)(Wimg - 1), sy = (float)(Himg - 1);
+    const bool m[4] = { vx0 && vy0 && fin, vx1 && vy0 && fin, vx0 && vy1 && fin, vx1 && vy1 && fin };
+    const float ax[4] = { -(1.0f - fy), 1.0f - fy, -fy, fy };
+    const float ay[4] = { -(1.0f - fx), -fx, 1.0f - fx, fx };
+    TapGrads t;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        t.gx[i] = m[i] ? sx * ax[i] : 0.0f;
+        t.gy[i] = m[i] ? sy * ay[i] : 0.0f;
+    }
+    return t;
+}
+
 // ------------------------------------------------------------------ wave-level helpers
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float x)

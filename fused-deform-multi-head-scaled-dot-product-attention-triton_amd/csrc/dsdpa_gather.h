@@ -306,12 +306,21 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_gather_kernel(
 
 // ------------------------------------------------------------------ backward, dq only
 // Same walk as bwd_gather_kernel without the dk/dv scatter: writes dq and the
-// per-row delta = dout.out (consumed by the tile kernel that produces dk/dv).
-template <typename S, int D, int DC>
+// per-row delta = dout.out (consumed by the kernels that produce dk/dv).
+//
+// CG: also the gradient of the coordinates (the reference's fused operator returns None there,
+// ops/triton.py:464; its eager operator gets it through grid_sample, ops/torch.py:14-15). With
+// g_t = sm_scale*ds*(q.K_t) + p*(dout.V_t) per tap, dL/dx = sum_t (d w_t/dx) g_t, likewise y. The per-tap
+// dot products replace the blend-then-dot of the plain kernel; a lane keeps partial sums over its DC
+// elements, combines them with the (slot-uniform) ds, p and tap derivatives and only the two results
+// are reduced over the slot. The H heads share the coordinates: float atomics into dcoords (zeroed by
+// the caller of the kernel).
+template <typename S, int D, int DC, bool CG>
 __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
-    const void *__restrict__ dout_, void *__restrict__ dq_, float *__restrict__ delta_, Dims dm)
+    const void *__restrict__ dout_, void *__restrict__ dq_, float *__restrict__ delta_,
+    float *__restrict__ dcoords_, Dims dm)
 {
     constexpr int G = D / DC;
     constexpr int NS = kWave / G;
@@ -319,6 +328,8 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
     __shared__ float4 s_w[kGatherWaves][kWave];
     __shared__ int4 s_e[kGatherWaves][kWave];
+    __shared__ float4 s_gx[CG ? kGatherWaves : 1][kWave];
+    __shared__ float4 s_gy[CG ? kGatherWaves : 1][kWave];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
@@ -329,7 +340,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     const char *vb = (const char *)v_ + rc.kv_base * S::kBytes;
     const float2 *coords = (const float2 *)coords_;
 
-    constexpr bool kPacked = S::kBytes == 2;
+    constexpr bool kPacked = S::kBytes == 2 && !CG;
     float qf[DC], dof[DC], of[DC];
     uint32_t dop[kPacked ? DC / 2 : 1];
     const size_t roff = (rc.row * D + lane_elem) * S::kBytes;
@@ -351,6 +362,16 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
 
     for (int c0 = 0; c0 < dm.N; c0 += kWave) {
         stage_descriptors<D>(coords, rc, dm, c0, lane, s_w[wave], s_e[wave]);
+        if constexpr (CG) {
+            // (stage_descriptors ends with a wave-level LDS sync; these two arrays are read after the
+            // next one, and their previous readers finished before the sync at its start)
+            const int n = min(c0 + lane, dm.N - 1);
+            const float2 xy = coords[rc.crow + n];
+            const TapGrads tg = make_tap_grads(xy.x, xy.y, dm.Wimg, dm.Himg);
+            s_gx[wave][lane] = make_float4(tg.gx[0], tg.gx[1], tg.gx[2], tg.gx[3]);
+            s_gy[wave][lane] = make_float4(tg.gy[0], tg.gy[1], tg.gy[2], tg.gy[3]);
+            wave_lds_sync();
+        }
         const int cnt = min(kWave, dm.N - c0);
 #pragma unroll
         for (int it = 0; it < ITS; ++it) {
@@ -359,8 +380,54 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                 float4 w = s_w[wave][j];
                 int4 e = s_e[wave][j];
                 float kk[DC];
-                blend_taps<S, DC>(kb, e, w, lane_elem, kk);
                 float dot = 0.f, dp = 0.f;
+                if constexpr (CG) {
+                    float t[4][DC], u[4][DC];
+                    const int eo[4] = { e.x, e.y, e.z, e.w };
+                    const float wt[4] = { w.x, w.y, w.z, w.w };
+                    float dk_t[4], dv_t[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        load_chunk<S, DC>(kb + (size_t)(eo[i] + lane_elem) * S::kBytes, t[i]);
+                        load_chunk<S, DC>(vb + (size_t)(eo[i] + lane_elem) * S::kBytes, u[i]);
+                    }
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) kk[d] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        dk_t[i] = 0.f;
+                        dv_t[i] = 0.f;
+#pragma unroll
+                        for (int d = 0; d < DC; ++d) {
+                            dk_t[i] = fmaf(qf[d], t[i][d], dk_t[i]);
+                            dv_t[i] = fmaf(dof[d], u[i][d], dv_t[i]);
+                            kk[d] = fmaf(wt[i], t[i][d], kk[d]);
+                        }
+                        dot = fmaf(wt[i], dk_t[i], dot);
+                        dp = fmaf(wt[i], dv_t[i], dp);
+                    }
+                    dot = group_sum<G>(dot);
+                    dp = group_sum<G>(dp);
+                    const float p = (j < cnt) ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
+                    const float ds = p * (dp - delta);
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
+                    const float4 ax = s_gx[wave][j], ay = s_gy[wave][j];
+                    const float a = ds * dm.sm_scale;
+                    const float g0 = fmaf(a, dk_t[0], p * dv_t[0]), g1 = fmaf(a, dk_t[1], p * dv_t[1]);
+                    const float g2 = fmaf(a, dk_t[2], p * dv_t[2]), g3 = fmaf(a, dk_t[3], p * dv_t[3]);
+                    float gx = fmaf(ax.x, g0, fmaf(ax.y, g1, fmaf(ax.z, g2, ax.w * g3)));
+                    float gy = fmaf(ay.x, g0, fmaf(ay.y, g1, fmaf(ay.z, g2, ay.w * g3)));
+                    gx = group_sum<G>(gx);
+                    gy = group_sum<G>(gy);
+                    if (g == 0 && j < cnt) {
+                        float *dst = dcoords_ + 2 * (rc.crow + (size_t)(c0 + j));
+                        atomicAdd(dst, gx);
+                        atomicAdd(dst + 1, gy);
+                    }
+                    continue;
+                }
+                blend_taps<S, DC>(kb, e, w, lane_elem, kk);
 #pragma unroll
                 for (int d = 0; d < DC; ++d) dot = fmaf(qf[d], kk[d], dot);
                 if constexpr (kPacked) {

@@ -122,7 +122,7 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
              void *workspace, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream);
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
-             const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,
+             const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
              int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream);
 
 }  // namespace dsdpa

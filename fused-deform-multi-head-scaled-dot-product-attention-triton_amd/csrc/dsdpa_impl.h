@@ -15,15 +15,19 @@ static_assert(kPlaneDescLdsBytes == (size_t)kPlaneDescBytes, "host and device ag
 template <int DC> struct PlaneRows { static constexpr int value = 16 / DC >= 1 ? 16 / DC : 1; };
 
 // ------------------------------------------------------------------ small kernels
-// Zero up to three buffers in one launch (sizes in 16-byte units; unused slots have size 0).
-struct ZeroJob { float4 *p[3]; size_t n4[3]; };
+// Zero up to four 16-byte aligned float buffers in one launch (sizes in floats; unused slots have size 0).
+struct ZeroJob { float *p[4]; size_t n[4]; };
 static __global__ void fill_zero_kernel(ZeroJob job)
 {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
 #pragma unroll
-    for (int k = 0; k < 3; ++k)
-        for (size_t i = first; i < job.n4[k]; i += stride) job.p[k][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k = 0; k < 4; ++k) {
+        const size_t n4 = job.n[k] / 4;
+        float4 *p4 = reinterpret_cast<float4 *>(job.p[k]);
+        for (size_t i = first; i < n4; i += stride) p4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (size_t i = 4 * n4 + first; i < job.n[k]; i += stride) job.p[k][i] = 0.f;
+    }
 }
 
 // fp32 accumulators -> 16-bit storage, 8 elements per thread
@@ -93,14 +97,18 @@ int launch_bwd_gather(const void *q, const void *k, const void *v, const float *
 
 template <typename S, int D>
 int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const float *coords, const void *out,
-                         const float *lse, const void *dout, void *dq, float *delta, const Dims &dm,
-                         hipStream_t st)
+                         const float *lse, const void *dout, void *dq, float *delta, float *dcoords,
+                         const Dims &dm, hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(2, st);
-    hipLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
-                       q, k, v, coords, out, lse, dout, dq, delta, dm);
+    if (dcoords)
+        hipLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                           q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm);
+    else
+        hipLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                           q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm);
     return check_launch();
 }
 
@@ -260,12 +268,12 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
     return DSDPA_ERR_HEAD_DIM;
 }
 
-// element counts are multiples of 4 (D >= 16; workspace segments are 256-byte multiples)
-static inline int zero_fill(float *a, size_t na, float *b, size_t nb, float *c, size_t nc, hipStream_t st)
+static inline int zero_fill(float *a, size_t na, float *b, size_t nb, float *c, size_t nc, float *d, size_t nd,
+                            hipStream_t st)
 {
-    ZeroJob job{{(float4 *)a, (float4 *)b, (float4 *)c}, {na / 4, nb / 4, nc / 4}};
-    size_t big = job.n4[0] > job.n4[1] ? job.n4[0] : job.n4[1];
-    if (job.n4[2] > big) big = job.n4[2];
+    ZeroJob job{{a, b, c, d}, {na, nb, nc, d ? nd : 0}};
+    size_t big = 0;
+    for (int i = 0; i < 4; ++i) big = job.n[i] / 4 > big ? job.n[i] / 4 : big;
     const int threads = 256;
     size_t blocks = (big + threads - 1) / threads;
     if (blocks > 256 * 16) blocks = 256 * 16;
@@ -342,7 +350,7 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
 
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
-             const float *lse, const void *dout, void *dq, void *dk, void *dv, void *workspace,
+             const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
              int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
 {
     if (!q || !k || !v || !coords || !out || !lse || !dout || !dq || !dk || !dv || !workspace)
@@ -359,7 +367,8 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const int path = g_path.load();
     const bool fused_atomics = path == DSDPA_PATH_GATHER;
     const bool cell_binned = path == DSDPA_PATH_AUTO;
-    const bool staged = !fused_atomics && wl.dl.bytes != 0;
+    // the coordinate gradient lives in the gather dq kernel only: dq leaves the staged kernels when it is asked for
+    const bool staged = !fused_atomics && wl.dl.bytes != 0 && !dcoords;
     const float4 *desc_w = (const float4 *)(ws + wl.desc + wl.dl.w);
     const uint32_t *desc_e = (const uint32_t *)(ws + wl.desc + wl.dl.e);
     const unsigned *start = (const unsigned *)(ws + wl.start);
@@ -367,17 +376,19 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     // one launch zeroes the dk/dv accumulators and, for the cell-binned path, the cell counters
     float *dk_acc = S::kBytes == 4 ? (float *)dk : (float *)(ws + wl.acc);
     float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
-    rc = zero_fill(dk_acc, n, dv_acc, n, (float *)(ws + wl.counters), cell_binned ? wl.counters_bytes / 4 : 0, st);
+    rc = zero_fill(dk_acc, n, dv_acc, n, (float *)(ws + wl.counters), cell_binned ? wl.counters_bytes / 4 : 0,
+                   dcoords, (size_t)dm.B * dm.V * dm.L * dm.N * 2, st);
     if (rc != DSDPA_OK) return rc;
     if (staged && (rc = launch_plane_descriptors(coords, dm, ws + wl.desc, wl.dl, 4, st)) != DSDPA_OK) return rc;
     if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
 #define DSDPA_BWD_CASE(DD)                                                                                      \
     case DD:                                                                                                    \
-        if (fused_atomics) {                                                                                    \
+        if (fused_atomics && !dcoords) {                                                                        \
             rc = launch_bwd_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st);         \
         } else {                                                                                                \
             rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, dm, st) \
-                        : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dm, st);      \
+                        : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm,  \
+                                                      st);                                                      \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
                 rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, lse, delta, dout, start, sorted, dk_acc,      \
                                                  dv_acc, dm, wl.NC, st);                                        \

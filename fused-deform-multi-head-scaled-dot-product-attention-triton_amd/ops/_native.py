@@ -45,7 +45,7 @@ def load():
         fwd.argtypes = [vp] * 7 + dims          # q k v coords out lse workspace
         fwd.restype = i
         bwd = getattr(lib, "dsdpa_bwd_" + sfx)
-        bwd.argtypes = [vp] * 11 + dims
+        bwd.argtypes = [vp] * 12 + dims         # q k v coords out lse dout dq dk dv dcoords workspace
         bwd.restype = i
     lib.dsdpa_fwd_workspace_bytes.argtypes = [i] * 8
     lib.dsdpa_fwd_workspace_bytes.restype = ctypes.c_size_t

@@ -66,7 +66,15 @@ def _check_inputs(q, k, v, coords, WIDTH, HEIGHT):
 
 class _fused_deform_sdpa(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, coords, WIDTH, HEIGHT, sm_scale):
+    def forward(ctx, q, k, v, coords, WIDTH, HEIGHT, sm_scale, *extra):
+        # extra = (coords_grad,): an eighth, optional argument the reference does not have. Left out (or False) the
+        # operator behaves like the reference's: no gradient for coords (ops/triton.py:464). True asks for
+        # the gradient of coords as well, the one the eager operator gets through grid_sample
+        # (ops/torch.py:14-15).
+        if len(extra) > 1:
+            raise TypeError("deform_sdpa_triton takes 7 arguments and an optional coords_grad flag")
+        ctx.n_inputs = 7 + len(extra)
+        ctx.coords_grad = bool(extra[0]) if extra else False
         sfx = _check_inputs(q, k, v, coords, WIDTH, HEIGHT)
         lib = _native.load()
         B, V, H, L, D = q.shape
@@ -100,16 +108,18 @@ class _fused_deform_sdpa(torch.autograd.Function):
         if do.dtype != q.dtype:
             do = do.to(q.dtype)
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dcoords = torch.empty_like(coords) if ctx.coords_grad and ctx.needs_input_grad[3] else None
         ws_bytes = lib.dsdpa_bwd_workspace_bytes(_DTYPE_CODE[q.dtype], B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P)
         ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
         with torch.cuda.device(q.device):
             rc = getattr(lib, "dsdpa_bwd_" + sfx)(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), coords.data_ptr(), out.data_ptr(), lse.data_ptr(),
                 do.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-                ws.data_ptr(),
+                dcoords.data_ptr() if dcoords is not None else None, ws.data_ptr(),
                 B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P, ctx.sm_scale, _stream_ptr(q.device))
         _native.check(rc)
-        return dq, dk, dv, None, None, None, None
+        grads = (dq, dk, dv, dcoords, None, None, None)
+        return grads if ctx.n_inputs == 7 else grads + (None,)
 
 
 deform_sdpa_triton = _fused_deform_sdpa.apply

@@ -85,6 +85,11 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
  * fp32 -> storage casts of dk/dv (:461-462).
  *
  * dq, dk, dv are fully overwritten (no pre-zeroing by the caller needed).
+ * `dcoords` may be NULL (the reference's behaviour: no gradient for coords, ops/triton.py:464). When it
+ * is given (fp32, shaped like coords) it receives the gradient of the normalised coordinates summed over
+ * the heads -- what the reference's eager operator gets by differentiating through grid_sample,
+ * ops/torch.py:14-15 -- and is fully overwritten too; the backward then takes the gather dq kernel for
+ * every shape (float atomics across heads: not deterministic either).
  * `workspace` must hold dsdpa_bwd_workspace_bytes(...) bytes (256-byte aligned):
  * the per-row delta = dout.out (one float per query row, the reference's `delta`,
  * ops/triton.py:430), the per-(batch, key view) ordering of the samples by
@@ -96,17 +101,17 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
  */
 int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords,
                   const float *out, const float *lse, const float *dout,
-                  float *dq, float *dk, float *dv, void *workspace,
+                  float *dq, float *dk, float *dv, float *dcoords, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
                   float sm_scale, void *stream);
 int dsdpa_bwd_bf16(const void *q, const void *k, const void *v, const float *coords,
                    const void *out, const float *lse, const void *dout,
-                   void *dq, void *dk, void *dv, void *workspace,
+                   void *dq, void *dk, void *dv, float *dcoords, void *workspace,
                    int B, int V, int H, int Himg, int Wimg, int D, int P,
                    float sm_scale, void *stream);
 int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coords,
                   const void *out, const float *lse, const void *dout,
-                  void *dq, void *dk, void *dv, void *workspace,
+                  void *dq, void *dk, void *dv, float *dcoords, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
                   float sm_scale, void *stream);
 

@@ -31,7 +31,7 @@ def _load():
         i, f = ctypes.c_int, ctypes.c_float
         lib.dsdpa_oracle_fwd.argtypes = [fp, fp, fp, fp, fp, fp, i, i, i, i, i, i, i, f]
         lib.dsdpa_oracle_fwd.restype = i
-        lib.dsdpa_oracle_bwd.argtypes = [fp, fp, fp, fp, fp, fp, fp, fp, i, i, i, i, i, i, i, f]
+        lib.dsdpa_oracle_bwd.argtypes = [fp, fp, fp, fp, fp, fp, fp, fp, fp, i, i, i, i, i, i, i, f]
         lib.dsdpa_oracle_bwd.restype = i
         lib.dsdpa_oracle_taps.argtypes = [f, f, i, i, ip, fp]
         lib.dsdpa_oracle_taps.restype = None
@@ -71,16 +71,18 @@ def oracle_fwd(q, k, v, coords, WIDTH, HEIGHT, sm_scale):
     return out, lse
 
 
-def oracle_bwd(q, k, v, coords, dout, WIDTH, HEIGHT, sm_scale):
-    """Backward. Returns ``(dq, dk, dv)`` as float32 arrays shaped like q."""
+def oracle_bwd(q, k, v, coords, dout, WIDTH, HEIGHT, sm_scale, with_coords=False):
+    """Backward. Returns ``(dq, dk, dv)`` as float32 arrays shaped like q; with ``with_coords`` also the
+    gradient of the normalised coordinates (shaped like coords, summed over heads)."""
     q, k, v, coords, dout = _f32(q), _f32(k), _f32(v), _f32(coords), _f32(dout)
     B, V, H, L, D, P = _dims(q, coords, WIDTH, HEIGHT)
     dq, dk, dv = np.empty_like(q), np.empty_like(q), np.empty_like(q)
+    dc = np.empty_like(coords) if with_coords else None
     rc = _load().dsdpa_oracle_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(coords), _ptr(dout),
-                                  _ptr(dq), _ptr(dk), _ptr(dv),
+                                  _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dc) if with_coords else None,
                                   B, V, H, HEIGHT, WIDTH, D, P, float(sm_scale))
     assert rc == 0
-    return dq, dk, dv
+    return (dq, dk, dv, dc) if with_coords else (dq, dk, dv)
 
 
 def oracle_taps(cx, cy, WIDTH, HEIGHT):

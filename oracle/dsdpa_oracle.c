@@ -44,6 +44,7 @@
 typedef struct {
     int pix[4];   /* row*W + col of the 4 taps, -1 when the tap is outside the image */
     float w[4];   /* bilinear weight of each tap (kept even for outside taps) */
+    float fx, fy; /* fractional position inside the cell, for the coordinate gradient */
 } taps_t;
 
 /*
@@ -81,6 +82,8 @@ static void sample_taps(float cx, float cy, int Wimg, int Himg, taps_t *t)
             t->pix[j * 2 + i] = inb ? ys[j] * Wimg + xs[i] : -1;
             t->w[j * 2 + i] = wx[i] * wy[j];
         }
+    t->fx = fx;
+    t->fy = fy;
     /* NaN coordinates: comparisons above are false -> all taps dropped */
     if (!(x == x) || !(y == y))
         for (int i = 0; i < 4; ++i) t->pix[i] = -1;
@@ -165,13 +168,24 @@ int dsdpa_oracle_fwd(const float *q, const float *k, const float *v,
  *   dK[tap pixel] += w_tap * sm_scale * ds_n * q     (inside-image taps only)
  *   dV[tap pixel] += w_tap * p_n * dout
  * p_n is recomputed from the row's own logits (not from a stored lse) so the
- * backward oracle does not inherit a forward rounding. coords, W, H and
- * sm_scale get no gradient. Parallel over (b, h): each pair owns its dK/dV
- * planes, so there are no races and the result is deterministic.
+ * backward oracle does not inherit a forward rounding. W, H and sm_scale
+ * get no gradient. Parallel over (b, h): each pair owns its dK/dV planes, so
+ * there are no races and the result is deterministic.
+ *
+ * dcoords (may be NULL; [B][V][L][V][P][2] like coords): the gradient the
+ * eager operator gets for free because grid_sample is differentiable in its
+ * grid (ops/torch.py:14-15; the fused reference returns None there,
+ * ops/triton.py:464). With g_t = sm_scale*ds_n*(q.K_t) + p_n*(dout.V_t) for
+ * the taps t = nw, ne, sw, se that lie inside the image (0 for the others)
+ * ATen's bilinear backward (GridSampler.cpp, grid_sampler_2d_backward) gives
+ *   dL/dx_pix = (1-fy)*(g_ne - g_nw) + fy*(g_se - g_sw)
+ *   dL/dy_pix = (1-fx)*(g_sw - g_nw) + fx*(g_se - g_ne)
+ * and x_pix = x*(W-1), y_pix = y*(Himg-1), summed over the H heads that
+ * share the coordinates (double accumulation, atomic across threads).
  */
 int dsdpa_oracle_bwd(const float *q, const float *k, const float *v,
                      const float *coords, const float *dout,
-                     float *dq, float *dk, float *dv,
+                     float *dq, float *dk, float *dv, float *dcoords,
                      int B, int V, int H, int Himg, int Wimg, int D, int P,
                      float sm_scale)
 {
@@ -181,7 +195,9 @@ int dsdpa_oracle_bwd(const float *q, const float *k, const float *v,
     const double qs = (double)sm_scale * DSDPA_LOG2E;
     double *dk64 = (double *)calloc(total, sizeof(double));
     double *dv64 = (double *)calloc(total, sizeof(double));
-    if (!dk64 || !dv64) { free(dk64); free(dv64); return 1; }
+    const size_t ncoord = (size_t)B * V * L * V * P * 2;
+    double *dc64 = dcoords ? (double *)calloc(ncoord, sizeof(double)) : NULL;
+    if (!dk64 || !dv64 || (dcoords && !dc64)) { free(dk64); free(dv64); free(dc64); return 1; }
 #pragma omp parallel
     {
         double *kt = (double *)malloc(sizeof(double) * (size_t)N * D);
@@ -229,6 +245,29 @@ int dsdpa_oracle_bwd(const float *q, const float *k, const float *v,
                         double ds = p * (dp - delta);
                         for (int d = 0; d < D; ++d) dqa[d] += ds * kt[(size_t)n * D + d];
                         size_t plane = (((size_t)b * V + s2) * H + h) * (size_t)L * D;
+                        if (dc64) {
+                            double g[4] = { 0.0, 0.0, 0.0, 0.0 };
+                            for (int i = 0; i < 4; ++i) {
+                                if (tp[n].pix[i] < 0) continue;
+                                const float *kp = k + plane + (size_t)tp[n].pix[i] * D;
+                                const float *vp = v + plane + (size_t)tp[n].pix[i] * D;
+                                double qk = 0.0, dov = 0.0;
+                                for (int d = 0; d < D; ++d) {
+                                    qk += (double)qrow[d] * (double)kp[d];
+                                    dov += (double)dorow[d] * (double)vp[d];
+                                }
+                                g[i] = (double)sm_scale * ds * qk + p * dov;
+                            }
+                            double fx = (double)tp[n].fx, fy = (double)tp[n].fy;
+                            double gx = (1.0 - fy) * (g[1] - g[0]) + fy * (g[3] - g[2]);
+                            double gy = (1.0 - fx) * (g[2] - g[0]) + fx * (g[3] - g[1]);
+                            size_t ci = (size_t)(crow - coords) + 2 * (size_t)n;
+                            double ax = gx * (double)(Wimg - 1), ay = gy * (double)(Himg - 1);
+#pragma omp atomic
+                            dc64[ci] += ax;
+#pragma omp atomic
+                            dc64[ci + 1] += ay;
+                        }
                         for (int i = 0; i < 4; ++i) {
                             if (tp[n].pix[i] < 0) continue;
                             double w = (double)tp[n].w[i];
@@ -248,7 +287,8 @@ int dsdpa_oracle_bwd(const float *q, const float *k, const float *v,
         free(kt); free(vt); free(s); free(tp); free(dqa);
     }
     for (size_t i = 0; i < total; ++i) { dk[i] = (float)dk64[i]; dv[i] = (float)dv64[i]; }
-    free(dk64); free(dv64);
+    if (dc64) for (size_t i = 0; i < ncoord; ++i) dcoords[i] = (float)dc64[i];
+    free(dk64); free(dv64); free(dc64);
     return 0;
 }
 

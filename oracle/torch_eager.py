@@ -53,12 +53,15 @@ def deform_sdpa_eager_chunked(q, k, v, coords, WIDTH, HEIGHT, sm_scale):
     return out
 
 
-def eager_fwd_bwd(q, k, v, coords, dout, WIDTH, HEIGHT, sm_scale, dtype=torch.float32, chunked=False):
-    """out, dq, dk, dv through PyTorch autograd (used to pin the C oracle's backward)."""
+def eager_fwd_bwd(q, k, v, coords, dout, WIDTH, HEIGHT, sm_scale, dtype=torch.float32, chunked=False,
+                  with_coords=False):
+    """out, dq, dk, dv [, dcoords] through PyTorch autograd (used to pin the C oracle's backward)."""
     qd = q.detach().to(dtype).requires_grad_(True)
     kd = k.detach().to(dtype).requires_grad_(True)
     vd = v.detach().to(dtype).requires_grad_(True)
     cd = coords.detach().to(dtype)
+    if with_coords:
+        cd.requires_grad_(True)
     if chunked:
         B, V, H, L, D = q.shape
         outs = torch.empty_like(qd)
@@ -73,4 +76,6 @@ def eager_fwd_bwd(q, k, v, coords, dout, WIDTH, HEIGHT, sm_scale, dtype=torch.fl
         out = deform_sdpa_eager(qd, kd, vd, cd, WIDTH, HEIGHT, sm_scale, dtype)
         out.backward(dout.to(dtype))
         out = out.detach()
+    if with_coords:
+        return out, qd.grad, kd.grad, vd.grad, cd.grad
     return out, qd.grad, kd.grad, vd.grad

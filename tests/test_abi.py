@@ -78,10 +78,10 @@ def test_argument_validation_before_launch():
     assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 1, 64, 64, 1024, 1024, 256, 2, 0.5, None) == 4
     # backward: the workspace is required
     args = [fake] * 10
-    assert lib.dsdpa_bwd_bf16(*args, None, *ok_dims) == 1
-    assert lib.dsdpa_bwd_f32(*args, None, *ok_dims) == 1
-    assert lib.dsdpa_bwd_f32(*args[:9], None, fake, *ok_dims) == 1
-    assert lib.dsdpa_bwd_f32(*args, fake, 1, 2, 2, 3, 4, 33, 2, 0.5, None) == 3
+    assert lib.dsdpa_bwd_bf16(*args, None, None, *ok_dims) == 1
+    assert lib.dsdpa_bwd_f32(*args, fake, None, *ok_dims) == 1
+    assert lib.dsdpa_bwd_f32(*args[:9], None, None, fake, *ok_dims) == 1
+    assert lib.dsdpa_bwd_f32(*args, None, fake, 1, 2, 2, 3, 4, 33, 2, 0.5, None) == 3     # dcoords is optional
 
 
 def test_path_selector():

@@ -251,6 +251,77 @@ def test_bwd_finite_differences():
             assert abs(fd - grad[idx]) < 2e-3 * max(1.0, abs(fd)), (name, idx, fd, grad[idx])
 
 
+@pytest.mark.parametrize("case", CASES)
+def test_coords_gradient_matches_library_autograd(case):
+    """The gradient of the normalised coordinates, summed over the heads that share them, against
+    autograd through grid_sample (float64), out-of-bounds taps included."""
+    seed, B, V, H, Himg, Wimg, D, P, lo, hi = case
+    q, k, v, c, do = make_case(seed, B, V, H, Himg, Wimg, D, P, lo, hi)
+    *_, dc_r = eager_fwd_bwd(q, k, v, c, do, Wimg, Himg, 0.37, dtype=torch.float64, with_coords=True)
+    *_, dc = oracle_bwd(q.numpy(), k.numpy(), v.numpy(), c.numpy(), do.numpy(), Wimg, Himg, 0.37,
+                        with_coords=True)
+    assert dc.shape == tuple(c.shape)
+    assert np.abs(dc_r.numpy()).max() > 0
+    assert rel(dc, dc_r.numpy()) < 1e-5
+
+
+def test_coords_gradient_closed_form_linear_image():
+    """V = a*col + b*row per channel (a plane), sm_scale = 0: every p_n = 1/N and the bilinear sample of a
+    plane is exact, so dL/dx = (W-1)/N * sum_h dout_h.a_h and dL/dy = (Himg-1)/N * sum_h dout_h.b_h for
+    every in-bounds sample, whatever the coordinates."""
+    B, V, H, Himg, Wimg, D, P = 1, 2, 3, 4, 5, 16, 3
+    g = torch.Generator().manual_seed(77)
+    L, N = Himg * Wimg, V * P
+    a = torch.randn(V, H, D, generator=g)
+    b = torch.randn(V, H, D, generator=g)
+    col = torch.arange(L) % Wimg
+    row = torch.arange(L) // Wimg
+    v = (a[:, :, None, :] * col[None, None, :, None] + b[:, :, None, :] * row[None, None, :, None])[None]
+    q = torch.randn(B, V, H, L, D, generator=g)
+    k = torch.randn(B, V, H, L, D, generator=g)
+    do = torch.randn(B, V, H, L, D, generator=g)
+    c = torch.rand(B, V, L, V, P, 2, generator=g) * 0.98 + 0.01
+    *_, dc = oracle_bwd(q.numpy(), k.numpy(), v.contiguous().numpy(), c.numpy(), do.numpy(), Wimg, Himg, 0.0,
+                        with_coords=True)
+    # expect[b, s1, l, s2, :, 0] = (W-1)/N * sum_h dout[b,s1,h,l,:] . a[s2,h,:]
+    ex = torch.einsum("bshld,thd->bslt", do.double(), a.double()) * (Wimg - 1) / N
+    ey = torch.einsum("bshld,thd->bslt", do.double(), b.double()) * (Himg - 1) / N
+    assert np.abs(dc[..., 0] - ex[..., None].numpy()).max() < 1e-4 * float(ex.abs().max())
+    assert np.abs(dc[..., 1] - ey[..., None].numpy()).max() < 1e-4 * float(ey.abs().max())
+
+
+def test_coords_gradient_finite_differences():
+    """Central differences of the oracle's own forward in single coordinates (steps that stay inside
+    the bilinear cell, where the forward is smooth)."""
+    q, k, v, c, do = make_case(12, 1, 2, 2, 3, 4, 16, 2, 0.05, 0.95)
+    Wimg, Himg = 4, 3
+    qn, kn, vn, cn, don = (t.numpy().copy() for t in (q, k, v, c, do))
+    *_, dc = oracle_bwd(qn, kn, vn, cn, don, Wimg, Himg, 0.6, with_coords=True)
+
+    def loss(cc):
+        out, _ = oracle_fwd(qn, kn, vn, cc, Wimg, Himg, 0.6)
+        return float((out.astype(np.float64) * don).sum())
+
+    rng = np.random.default_rng(1)
+    eps, checked = 2e-3, 0
+    for _ in range(60):
+        idx = tuple(rng.integers(0, s) for s in cn.shape)
+        size = (Wimg if idx[-1] == 0 else Himg) - 1
+        pix = float(cn[idx]) * size
+        if min(pix - math.floor(pix), math.ceil(pix) - pix) < 3 * eps * size:
+            continue                                    # too close to a cell border
+        old = cn[idx]
+        cn[idx] = old + eps
+        lp = loss(cn)
+        cn[idx] = old - eps
+        lm = loss(cn)
+        cn[idx] = old
+        fd = (lp - lm) / (float(np.float32(old + eps)) - float(np.float32(old - eps)))
+        assert abs(fd - dc[idx]) < 5e-3 * max(1.0, abs(fd)), (idx, fd, dc[idx])
+        checked += 1
+    assert checked >= 20
+
+
 def test_bwd_homogeneity_identities():
     """Logits are bilinear in (q, K) and out is linear in V:
     <q,dq> = <K,dK> and <V,dV> = <dout,out>."""
