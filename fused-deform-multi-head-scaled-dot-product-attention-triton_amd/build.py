@@ -11,7 +11,7 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRCS = [os.path.join(HERE, "csrc", n) for n in ("dsdpa_api.hip", "dsdpa_f32.hip", "dsdpa_bf16.hip", "dsdpa_f16.hip")]
+SRCS = [os.path.join(HERE, "csrc", n) for n in ("dsdpa_api.hip", "dsdpa_sort.hip", "dsdpa_f32.hip", "dsdpa_bf16.hip", "dsdpa_f16.hip")]
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libdsdpa.so")
@@ -31,7 +31,7 @@ def _run(cmd):
 
 
 def build_library(verbose=True, extra_flags=()):
-    """Compile the four translation units in parallel (one per storage type + the C ABI) and link them."""
+    """Compile the translation units in parallel (one per storage type, the C ABI, the list sort) and link."""
     from concurrent.futures import ThreadPoolExecutor
     os.makedirs(LIB_DIR, exist_ok=True)
     os.makedirs(OBJ_DIR, exist_ok=True)

@@ -34,26 +34,26 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
 
 int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords, const float *out,
                   const float *lse, const float *dout, float *dq, float *dk, float *dv, float *dcoords, void *workspace,
-                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, unsigned flags, void *stream)
 {
     return bwd_impl<F32>(q, k, v, coords, out, lse, dout, dq, dk, dv, dcoords, workspace, B, V, H, Himg, Wimg, D, P,
-                         sm_scale, stream);
+                         sm_scale, flags, stream);
 }
 
 int dsdpa_bwd_bf16(const void *q, const void *k, const void *v, const float *coords, const void *out,
                    const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
-                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, unsigned flags, void *stream)
 {
     return bwd_impl<BF16>(q, k, v, coords, out, lse, dout, dq, dk, dv, dcoords, workspace, B, V, H, Himg, Wimg, D, P,
-                          sm_scale, stream);
+                          sm_scale, flags, stream);
 }
 
 int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coords, const void *out,
                   const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
-                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, unsigned flags, void *stream)
 {
     return bwd_impl<F16>(q, k, v, coords, out, lse, dout, dq, dk, dv, dcoords, workspace, B, V, H, Himg, Wimg, D, P,
-                         sm_scale, stream);
+                         sm_scale, flags, stream);
 }
 
 size_t dsdpa_fwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P)
@@ -63,11 +63,12 @@ size_t dsdpa_fwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int W
     return desc_layout(B, V, Himg, Wimg, D, P, dtype != DSDPA_F32 ? 2 : 4).bytes;
 }
 
-size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P)
+size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P, unsigned flags)
 {
     if (dtype != DSDPA_F32 && dtype != DSDPA_BF16 && dtype != DSDPA_F16) return 0;
     if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || D < 1 || P < 1) return 0;
-    return workspace_layout(B, V, H, Himg, Wimg, D, P, dtype != DSDPA_F32).total;
+    return workspace_layout(B, V, H, Himg, Wimg, D, P, dtype != DSDPA_F32,
+                            (flags & DSDPA_FLAG_DETERMINISTIC) != 0).total;
 }
 
 const char *dsdpa_error_string(int code)
@@ -79,6 +80,7 @@ const char *dsdpa_error_string(int code)
     case DSDPA_ERR_HEAD_DIM: return "head dim must be one of 16, 32, 64, 128, 256";
     case DSDPA_ERR_TOO_LARGE: return "shape exceeds the 32-bit indexing limits of the kernels";
     case DSDPA_ERR_HIP: return "a HIP launch failed (see dsdpa_last_hip_error)";
+    case DSDPA_ERR_UNSUPPORTED: return "unknown flag, or a combination of options that is not supported";
     case DSDPA_ERR_DTYPE: return "unknown dtype code";
     }
     return "unknown error code";

@@ -6,5 +6,5 @@ template int fwd_impl<BF16>(const void *, const void *, const void *, const floa
                            int, int, int, float, void *);
 template int bwd_impl<BF16>(const void *, const void *, const void *, const float *, const void *, const float *,
                            const void *, void *, void *, void *, float *, void *, int, int, int, int, int, int, int, float,
-                           void *);
+                           unsigned, void *);
 }  // namespace dsdpa

@@ -158,6 +158,19 @@ static __global__ __launch_bounds__(1024) void bin_scan_kernel(unsigned *__restr
     if (threadIdx.x == 0) st[NC] = s_carry;
 }
 
+// Deterministic backward: begin / end of every cell list as positions in the flat id array
+// [B*V][M] (one thread per (group, cell)), the segment bounds of the sort that orders each list.
+static __global__ void cell_segments_kernel(const unsigned *__restrict__ start, int NC, unsigned M, unsigned nseg,
+                                            unsigned *__restrict__ seg_begin, unsigned *__restrict__ seg_end)
+{
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nseg) return;
+    const unsigned grp = i / (unsigned)NC, cell = i - grp * (unsigned)NC;
+    const unsigned *st = start + (size_t)grp * (NC + 1) + cell;
+    seg_begin[i] = grp * M + st[0];
+    seg_end[i] = grp * M + st[1];
+}
+
 template <typename S, int DC>
 __device__ __forceinline__ void load_tap_or_zero(const char *base, int pix, int D, int lane_elem, bool valid,
                                                  float (&dst)[DC])
@@ -175,7 +188,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float *__restrict__ lse_, const float *__restrict__ delta_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
-    float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC)
+    float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC, int colour)
 {
     constexpr int G = D / DC;
     constexpr int NS = kWave / G;
@@ -185,11 +198,20 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const long long work = (long long)xcd_logical_block(blockIdx.x, gridDim.x) * kCellWaves + wave;
-    const long long nwork = (long long)dm.B * dm.H * dm.V * NC;
-    if (work >= nwork) return;
+    // colour < 0: all cells, per-cell sums flushed with float atomics (a pixel belongs to four cells).
+    // colour 0..3 (deterministic backward): only the cells with (row parity, column parity) = colour; no
+    // two of them share a pixel, so the flush is a plain read-add-write, and the four launches, one
+    // after the other, add every pixel's four contributions in a fixed order.
+    const int cw = dm.Wimg + 1, ch = dm.Himg + 1;
+    const int oy = colour < 0 ? 0 : colour >> 1, ox = colour < 0 ? 0 : colour & 1, step = colour < 0 ? 1 : 2;
+    const int ncx = (cw - ox + step - 1) / step, ncy = (ch - oy + step - 1) / step;
+    const int ncells = ncx * ncy;
+    const long long nwork = (long long)dm.B * dm.H * dm.V * ncells;
+    if (work >= nwork || ncells == 0) return;
     // plane-major: (b, h, s2, cell)
-    const int cell = (int)(work % NC);
-    long long t = work / NC;
+    const int ci = (int)(work % ncells);
+    const int cell = (ci / ncx * step + oy) * cw + (ci % ncx) * step + ox;
+    long long t = work / ncells;
     const int s2 = (int)(t % dm.V);
     t /= dm.V;
     const int h = (int)(t % dm.H);
@@ -340,8 +362,14 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
             if (tv[tpi]) {
 #pragma unroll
                 for (int d = 0; d < DC; ++d) {
-                    atomicAdd(dkb + (size_t)tpix[tpi] * D + d, aK[tpi][d]);
-                    atomicAdd(dvb + (size_t)tpix[tpi] * D + d, aV[tpi][d]);
+                    float *pk = dkb + (size_t)tpix[tpi] * D + d, *pv = dvb + (size_t)tpix[tpi] * D + d;
+                    if (colour < 0) {
+                        atomicAdd(pk, aK[tpi][d]);
+                        atomicAdd(pv, aV[tpi][d]);
+                    } else {
+                        *pk += aK[tpi][d];
+                        *pv += aV[tpi][d];
+                    }
                 }
             }
         }

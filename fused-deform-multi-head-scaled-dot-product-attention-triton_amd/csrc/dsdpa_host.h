@@ -89,15 +89,24 @@ inline DescLayout desc_layout(size_t B, size_t V, size_t Himg, size_t Wimg, size
 //   sorted   B*V*(V*L*P) u32                 sample ids ordered by cell
 //   acc      2*n floats                      fp32 dk/dv accumulators (16-bit storage only)
 //   desc     20 bytes per coordinate pair    descriptor table (only when the plane kernels apply)
+// deterministic backward only (DSDPA_FLAG_DETERMINISTIC):
+//   sorted2  as sorted                       the lists with every cell's ids in ascending order
+//   seg      2*B*V*NC u32                    begin / end of every list in the flat id array
+//   sorttmp  sort_temp_bytes()               scratch of the segmented sort
 // with NC = (Himg+1)*(Wimg+1) cells.
+size_t sort_temp_bytes(size_t n, size_t segments);                       // dsdpa_sort.hip
+int sort_cell_lists(void *temp, size_t temp_bytes, const unsigned *ids_in, unsigned *ids_out, size_t n,
+                    size_t segments, const unsigned *seg_begin, const unsigned *seg_end, unsigned id_bits,
+                    hipStream_t st);
+
 struct WorkspaceLayout {
-    size_t delta, counters, start, sorted, acc, desc, total;
+    size_t delta, counters, start, sorted, acc, desc, sorted2, seg, sorttmp, sorttmp_bytes, total;
     DescLayout dl;
     size_t counters_bytes;
     int NC;
 };
 inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Himg, size_t Wimg, size_t D, size_t P,
-                                        bool storage16)
+                                        bool storage16, bool deterministic)
 {
     WorkspaceLayout w;
     const size_t rows = B * V * H * Himg * Wimg;
@@ -110,6 +119,15 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     w.acc = off; if (storage16) off += round256(2 * rows * D * 4);
     w.dl = desc_layout(B, V, Himg, Wimg, D, P, storage16 ? 2 : 4);
     w.desc = off; off += w.dl.bytes;
+    w.sorted2 = w.seg = w.sorttmp = off;
+    w.sorttmp_bytes = 0;
+    if (deterministic) {
+        const size_t ids = B * V * (V * Himg * Wimg * P), segs = B * V * (size_t)w.NC;
+        w.sorted2 = off; off += round256(ids * 4);
+        w.seg = off; off += round256(2 * segs * 4);
+        w.sorttmp_bytes = round256(sort_temp_bytes(ids, segs));
+        w.sorttmp = off; off += w.sorttmp_bytes;
+    }
     w.total = off;
     return w;
 }
@@ -123,6 +141,6 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
              const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
-             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream);
+             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, unsigned flags, void *stream);
 
 }  // namespace dsdpa

@@ -333,38 +333,67 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
     return check_launch();
 }
 
+// deterministic: four launches, one per (row parity, column parity) of the cells, each with plain stores
 template <typename S, int D>
 int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const float *coords, const float *lse,
                          const float *delta, const void *dout, const unsigned *start, const unsigned *sorted,
-                         float *dk_acc, float *dv_acc, const Dims &dm, int NC, hipStream_t st)
+                         float *dk_acc, float *dv_acc, const Dims &dm, int NC, bool deterministic, hipStream_t st)
 {
     constexpr int DC = CellChunk<S, D>::value;
-    const long long nwork = (long long)dm.B * dm.H * dm.V * NC;
-    const long long blocks = (nwork + kCellWaves - 1) / kCellWaves;
-    if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
     ScopedKernelTimer timer(1, st);
-    hipLaunchKernelGGL((bwd_dkdv_cell_kernel<S, D, DC>), dim3((unsigned)blocks), dim3(kCellWaves * kWave), 0, st,
-                       q, k, v, coords, lse, delta, dout, start, sorted, dk_acc, dv_acc, dm, NC);
+    for (int colour = deterministic ? 0 : -1; colour < (deterministic ? 4 : 0); ++colour) {
+        const int cw = dm.Wimg + 1, ch = dm.Himg + 1;
+        const int oy = colour < 0 ? 0 : colour >> 1, ox = colour < 0 ? 0 : colour & 1, step = colour < 0 ? 1 : 2;
+        const long long ncells = (long long)((cw - ox + step - 1) / step) * ((ch - oy + step - 1) / step);
+        const long long nwork = (long long)dm.B * dm.H * dm.V * ncells;
+        const long long blocks = (nwork + kCellWaves - 1) / kCellWaves;
+        if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+        if (blocks == 0) continue;
+        hipLaunchKernelGGL((bwd_dkdv_cell_kernel<S, D, DC>), dim3((unsigned)blocks), dim3(kCellWaves * kWave), 0, st,
+                           q, k, v, coords, lse, delta, dout, start, sorted, dk_acc, dv_acc, dm, NC, colour);
+    }
     return check_launch();
+}
+
+// Deterministic backward: order every cell list by sample id (the counting sort leaves the order inside a
+// cell to its atomics).
+static inline int launch_list_ordering(const Dims &dm, const WorkspaceLayout &wl, char *ws, hipStream_t st)
+{
+    const size_t M = (size_t)dm.V * dm.L * dm.P, groups = (size_t)dm.B * dm.V;
+    const size_t ids = groups * M, segs = groups * (size_t)wl.NC;
+    if (ids > 0xffffffffull || segs > 0x7fffffffull) return DSDPA_ERR_TOO_LARGE;
+    unsigned *seg_begin = (unsigned *)(ws + wl.seg), *seg_end = seg_begin + segs;
+    ScopedKernelTimer timer(3, st);
+    hipLaunchKernelGGL(cell_segments_kernel, dim3((unsigned)((segs + 255) / 256)), dim3(256), 0, st,
+                       (const unsigned *)(ws + wl.start), wl.NC, (unsigned)M, (unsigned)segs, seg_begin, seg_end);
+    int rc = check_launch();
+    if (rc != DSDPA_OK) return rc;
+    unsigned bits = 1;
+    while (bits < 32 && (1ull << bits) < M) ++bits;
+    return sort_cell_lists(ws + wl.sorttmp, wl.sorttmp_bytes, (const unsigned *)(ws + wl.sorted),
+                           (unsigned *)(ws + wl.sorted2), ids, segs, seg_begin, seg_end, bits, st);
 }
 
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
              const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
-             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, unsigned flags, void *stream)
 {
     if (!q || !k || !v || !coords || !out || !lse || !dout || !dq || !dk || !dv || !workspace)
         return DSDPA_ERR_NULL_POINTER;
+    if (flags & ~(unsigned)DSDPA_FLAG_DETERMINISTIC) return DSDPA_ERR_UNSUPPORTED;
+    const bool deterministic = (flags & DSDPA_FLAG_DETERMINISTIC) != 0;
+    if (deterministic && dcoords) return DSDPA_ERR_UNSUPPORTED;   // dcoords sums over heads with float atomics
     Dims dm;
     int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
     if (rc != DSDPA_OK) return rc;
     if ((long long)dm.L * dm.N > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;   // sample ids are 32-bit
     hipStream_t st = (hipStream_t)stream;
     const size_t n = (size_t)dm.rows * D;
-    const WorkspaceLayout wl = workspace_layout(B, V, H, Himg, Wimg, D, P, S::kBytes != 4);
+    const WorkspaceLayout wl = workspace_layout(B, V, H, Himg, Wimg, D, P, S::kBytes != 4, deterministic);
     char *ws = (char *)workspace;
     float *delta = (float *)(ws + wl.delta);
-    const int path = g_path.load();
+    const int path = deterministic ? (int)DSDPA_PATH_AUTO : g_path.load();   // only the cell-binned path has a fixed order
     const bool fused_atomics = path == DSDPA_PATH_GATHER;
     const bool cell_binned = path == DSDPA_PATH_AUTO;
     // the coordinate gradient lives in the gather dq kernel only: dq leaves the staged kernels when it is asked for
@@ -372,7 +401,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const float4 *desc_w = (const float4 *)(ws + wl.desc + wl.dl.w);
     const uint32_t *desc_e = (const uint32_t *)(ws + wl.desc + wl.dl.e);
     const unsigned *start = (const unsigned *)(ws + wl.start);
-    const unsigned *sorted = (const unsigned *)(ws + wl.sorted);
+    const unsigned *sorted = (const unsigned *)(ws + (deterministic ? wl.sorted2 : wl.sorted));
     // one launch zeroes the dk/dv accumulators and, for the cell-binned path, the cell counters
     float *dk_acc = S::kBytes == 4 ? (float *)dk : (float *)(ws + wl.acc);
     float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
@@ -381,6 +410,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     if (rc != DSDPA_OK) return rc;
     if (staged && (rc = launch_plane_descriptors(coords, dm, ws + wl.desc, wl.dl, 4, st)) != DSDPA_OK) return rc;
     if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
+    if (deterministic && (rc = launch_list_ordering(dm, wl, ws, st)) != DSDPA_OK) return rc;
 #define DSDPA_BWD_CASE(DD)                                                                                      \
     case DD:                                                                                                    \
         if (fused_atomics && !dcoords) {                                                                        \
@@ -391,7 +421,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
                                                       st);                                                      \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
                 rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, lse, delta, dout, start, sorted, dk_acc,      \
-                                                 dv_acc, dm, wl.NC, st);                                        \
+                                                 dv_acc, dm, wl.NC, deterministic, st);                         \
             else if (rc == DSDPA_OK)                                                                            \
                 rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, st);    \
         }                                                                                                       \

@@ -20,6 +20,7 @@ SYMBOLS = (
 
 DSDPA_F32, DSDPA_BF16, DSDPA_F16 = 0, 1, 2
 PATH_AUTO, PATH_GATHER, PATH_LDS = 0, 1, 2
+FLAG_DETERMINISTIC = 1
 
 _lib = None
 
@@ -40,16 +41,17 @@ def load():
     lib = ctypes.CDLL(LIB_PATH)
     vp, i, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
     dims = [i, i, i, i, i, i, i, f, vp]            # B V H Himg Wimg D P sm_scale stream
+    u = ctypes.c_uint
     for sfx in ("f32", "bf16", "f16"):
         fwd = getattr(lib, "dsdpa_fwd_" + sfx)
         fwd.argtypes = [vp] * 7 + dims          # q k v coords out lse workspace
         fwd.restype = i
         bwd = getattr(lib, "dsdpa_bwd_" + sfx)
-        bwd.argtypes = [vp] * 12 + dims         # q k v coords out lse dout dq dk dv dcoords workspace
+        bwd.argtypes = [vp] * 12 + dims[:-1] + [u, vp]   # q k v coords out lse dout dq dk dv dcoords workspace, dims, flags, stream
         bwd.restype = i
     lib.dsdpa_fwd_workspace_bytes.argtypes = [i] * 8
     lib.dsdpa_fwd_workspace_bytes.restype = ctypes.c_size_t
-    lib.dsdpa_bwd_workspace_bytes.argtypes = [i] * 8
+    lib.dsdpa_bwd_workspace_bytes.argtypes = [i] * 8 + [u]
     lib.dsdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.dsdpa_error_string.argtypes = [i]
     lib.dsdpa_error_string.restype = ctypes.c_char_p

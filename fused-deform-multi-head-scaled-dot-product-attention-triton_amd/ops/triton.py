@@ -109,14 +109,19 @@ class _fused_deform_sdpa(torch.autograd.Function):
             do = do.to(q.dtype)
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         dcoords = torch.empty_like(coords) if ctx.coords_grad and ctx.needs_input_grad[3] else None
-        ws_bytes = lib.dsdpa_bwd_workspace_bytes(_DTYPE_CODE[q.dtype], B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P)
+        # torch.use_deterministic_algorithms(True) selects the bitwise reproducible backward
+        flags = _native.FLAG_DETERMINISTIC if torch.are_deterministic_algorithms_enabled() else 0
+        if flags and dcoords is not None:
+            raise RuntimeError("deform_sdpa_triton: the coordinate gradient has no deterministic implementation "
+                               "(it sums over heads with float atomics); turn one of the two off")
+        ws_bytes = lib.dsdpa_bwd_workspace_bytes(_DTYPE_CODE[q.dtype], B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P, flags)
         ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
         with torch.cuda.device(q.device):
             rc = getattr(lib, "dsdpa_bwd_" + sfx)(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), coords.data_ptr(), out.data_ptr(), lse.data_ptr(),
                 do.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                 dcoords.data_ptr() if dcoords is not None else None, ws.data_ptr(),
-                B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P, ctx.sm_scale, _stream_ptr(q.device))
+                B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P, ctx.sm_scale, flags, _stream_ptr(q.device))
         _native.check(rc)
         grads = (dq, dk, dv, dcoords, None, None, None)
         return grads if ctx.n_inputs == 7 else grads + (None,)

@@ -48,7 +48,8 @@ enum {
     DSDPA_ERR_TOO_LARGE = 4,      /* a per-batch slab V*H*L*D exceeds 2^30 elements or
                                      rows exceed 2^31-1                                   */
     DSDPA_ERR_HIP = 5,            /* a HIP launch failed; see dsdpa_last_hip_error()      */
-    DSDPA_ERR_DTYPE = 6           /* unknown dtype code                                   */
+    DSDPA_ERR_DTYPE = 6,          /* unknown dtype code                                   */
+    DSDPA_ERR_UNSUPPORTED = 7     /* unknown flag bit, or DSDPA_FLAG_DETERMINISTIC with dcoords */
 };
 
 /* Storage types (accumulation is always fp32). Mirrors the reference's dtype
@@ -78,6 +79,13 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
                   float sm_scale, void *stream);
 
+/* Flags of the backward. The reference has one backward, with float atomics (ops/triton.py:345-360).
+ * DSDPA_FLAG_DETERMINISTIC: bitwise reproducible dq, dk, dv: the samples of every bilinear cell are
+ * added up in ascending order of their index and the per-cell sums reach dk/dv in four passes of plain
+ * stores (cells of one row/column parity share no pixel) instead of float atomics. Needs a larger
+ * workspace (pass the same flags to dsdpa_bwd_workspace_bytes) and cannot be combined with dcoords. */
+enum { DSDPA_FLAG_DETERMINISTIC = 1 };
+
 /*
  * Backward: replaces everything `_fused_deform_sdpa.backward` enqueues,
  * ops/triton.py:427-462: the zero-fills (:427-430), the scaled copy of K
@@ -96,24 +104,25 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
  * bilinear cell (one u32 per coordinate pair plus the cell offsets; it depends on
  * coords only and is shared by all heads) and, for bf16/fp16, the fp32 dk/dv
  * accumulators that are rounded to the storage type at the end (fp32: dk and dv
- * are themselves the accumulators), and the same per-coordinate table as the forward's. Accumulation order into dk/dv is not deterministic (float atomics,
+ * are themselves the accumulators), and the same per-coordinate table as the forward's. Without
+ * DSDPA_FLAG_DETERMINISTIC the accumulation order into dk/dv is not deterministic (float atomics,
  * as in the reference, ops/triton.py:345-360).
  */
 int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords,
                   const float *out, const float *lse, const float *dout,
                   float *dq, float *dk, float *dv, float *dcoords, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
-                  float sm_scale, void *stream);
+                  float sm_scale, unsigned flags, void *stream);
 int dsdpa_bwd_bf16(const void *q, const void *k, const void *v, const float *coords,
                    const void *out, const float *lse, const void *dout,
                    void *dq, void *dk, void *dv, float *dcoords, void *workspace,
                    int B, int V, int H, int Himg, int Wimg, int D, int P,
-                   float sm_scale, void *stream);
+                   float sm_scale, unsigned flags, void *stream);
 int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coords,
                   const void *out, const float *lse, const void *dout,
                   void *dq, void *dk, void *dv, float *dcoords, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
-                  float sm_scale, void *stream);
+                  float sm_scale, unsigned flags, void *stream);
 
 /* Bytes of device workspace dsdpa_fwd_* needs for a storage dtype: 20 bytes per coordinate pair when the
  * K and V planes of one view fit in LDS (the staged kernels), else 0; 0 also if an argument is invalid.
@@ -122,7 +131,8 @@ size_t dsdpa_fwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int W
 
 /* Bytes of device workspace dsdpa_bwd_* needs for a storage dtype (0 if an argument is invalid).
  * Counterpart of the reference's delta and dk32/dv32 temporaries, ops/triton.py:428-430. */
-size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P);
+size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P,
+                                 unsigned flags);
 
 /* Human-readable text for a DSDPA_ERR_* code. */
 const char *dsdpa_error_string(int code);

@@ -54,15 +54,20 @@ def test_workspace_bytes():
         total += r256(2 * rows * D * 4) if storage16 else 0
         return total + table(B, V, Himg, Wimg, D, P, storage16)
 
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32) == expect(2, 6, 8, 18, 18, 32, 32, False)
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64, 32) == expect(2, 6, 8, 48, 48, 64, 32, True)
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F16, 1, 2, 1, 3, 5, 16, 7) == expect(1, 2, 1, 3, 5, 16, 7, True)
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32, 0) == expect(2, 6, 8, 18, 18, 32, 32, False)
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64, 32, 0) == expect(2, 6, 8, 48, 48, 64, 32, True)
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F16, 1, 2, 1, 3, 5, 16, 7, 0) == expect(1, 2, 1, 3, 5, 16, 7, True)
     assert lib.dsdpa_fwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32) == table(2, 6, 18, 18, 32, 32, False) > 0
     assert lib.dsdpa_fwd_workspace_bytes(_native.DSDPA_F16, 1, 2, 1, 3, 5, 16, 7) == table(1, 2, 3, 5, 16, 7, True) > 0
     assert lib.dsdpa_fwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64, 32) == 0      # planes too large for LDS
     assert lib.dsdpa_fwd_workspace_bytes(7, 2, 6, 8, 18, 18, 32, 32) == 0
-    assert lib.dsdpa_bwd_workspace_bytes(7, 2, 6, 8, 48, 48, 64, 32) == 0
-    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 0, 6, 8, 48, 48, 64, 32) == 0
+    assert lib.dsdpa_bwd_workspace_bytes(7, 2, 6, 8, 48, 48, 64, 32, 0) == 0
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 0, 6, 8, 48, 48, 64, 32, 0) == 0
+    # deterministic backward: a second id array and the list bounds on top (plus the sort's scratch, whose
+    # size the sort routine reports on a machine with a GPU)
+    plain = lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32, 0)
+    det = lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32, _native.FLAG_DETERMINISTIC)
+    assert det >= plain + r256(2 * 6 * 6 * 324 * 32 * 4) + r256(2 * 2 * 6 * 361 * 4)
 
 
 def test_argument_validation_before_launch():
@@ -70,6 +75,7 @@ def test_argument_validation_before_launch():
     lib = _native.load()
     fake = ctypes.c_void_p(0x1000)   # never dereferenced: validation fails first
     ok_dims = (1, 2, 2, 3, 4, 32, 2, 0.5, None)
+    bwd_dims = (1, 2, 2, 3, 4, 32, 2, 0.5, 0, None)          # ... sm_scale, flags, stream
     assert lib.dsdpa_fwd_f32(None, fake, fake, fake, fake, fake, fake, *ok_dims) == 1
     assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, None, *ok_dims) == 1    # this shape needs the workspace
     assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 0, 2, 2, 3, 4, 32, 2, 0.5, None) == 2
@@ -78,10 +84,12 @@ def test_argument_validation_before_launch():
     assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 1, 64, 64, 1024, 1024, 256, 2, 0.5, None) == 4
     # backward: the workspace is required
     args = [fake] * 10
-    assert lib.dsdpa_bwd_bf16(*args, None, None, *ok_dims) == 1
-    assert lib.dsdpa_bwd_f32(*args, fake, None, *ok_dims) == 1
-    assert lib.dsdpa_bwd_f32(*args[:9], None, None, fake, *ok_dims) == 1
-    assert lib.dsdpa_bwd_f32(*args, None, fake, 1, 2, 2, 3, 4, 33, 2, 0.5, None) == 3     # dcoords is optional
+    assert lib.dsdpa_bwd_bf16(*args, None, None, *bwd_dims) == 1
+    assert lib.dsdpa_bwd_f32(*args, fake, None, *bwd_dims) == 1
+    assert lib.dsdpa_bwd_f32(*args[:9], None, None, fake, *bwd_dims) == 1
+    assert lib.dsdpa_bwd_f32(*args, None, fake, 1, 2, 2, 3, 4, 33, 2, 0.5, 0, None) == 3     # dcoords is optional
+    assert lib.dsdpa_bwd_f32(*args, None, fake, 1, 2, 2, 3, 4, 32, 2, 0.5, 8, None) == 7     # unknown flag
+    assert lib.dsdpa_bwd_f32(*args, fake, fake, 1, 2, 2, 3, 4, 32, 2, 0.5, _native.FLAG_DETERMINISTIC, None) == 7
 
 
 def test_path_selector():
