@@ -2,6 +2,7 @@
 // kernel timer. Defined in dsdpa_api.hip.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <atomic>
 #include <mutex>
@@ -14,9 +15,12 @@ namespace dsdpa {
 extern thread_local int g_last_hip_error;
 extern std::atomic<int> g_path;
 
-// Optional kernel timer: while enabled, every main forward/backward kernel
-// launch is bracketed by a pair of HIP events on the launch stream. Process-wide
-// (a framework may run the backward pass on another thread than the forward).
+// Optional kernel timer: while enabled, every main forward/backward kernel launch carries a pair of HIP
+// events. Process-wide (a framework may run the backward pass on another thread than the forward).
+// The events ride on the kernel's own dispatch (hipExtLaunchKernelGGL's start/stop events: the start and
+// end timestamps of that dispatch), not on hipEventRecord: an event recorded between two kernels costs
+// about 5 us of idle GPU each (measured: 10 us gaps between timed kernels, none between untimed ones),
+// which would make the timed step slower than the untimed one.
 struct EventPair { hipEvent_t start, stop; };
 struct KernelTimer {
     std::atomic<bool> on{false};
@@ -25,22 +29,27 @@ struct KernelTimer {
 };
 extern KernelTimer g_timer;
 
+// One timed item: a single launch (pass start() and stop() to it) or a run of launches (start() to the
+// first, stop() to the last). record = true: the item contains launches made by a library routine, which
+// cannot carry events; then the pair is recorded around the run with hipEventRecord.
 struct ScopedKernelTimer {
     hipStream_t st;
     EventPair ev{nullptr, nullptr};
     int which;
-    bool armed = false;
-    ScopedKernelTimer(int which_, hipStream_t st_) : st(st_), which(which_)
+    bool armed = false, record;
+    ScopedKernelTimer(int which_, hipStream_t st_, bool record_ = false) : st(st_), which(which_), record(record_)
     {
         if (!g_timer.on.load(std::memory_order_relaxed)) return;
         if (hipEventCreate(&ev.start) != hipSuccess) return;
         if (hipEventCreate(&ev.stop) != hipSuccess) { (void)hipEventDestroy(ev.start); return; }
-        armed = hipEventRecord(ev.start, st) == hipSuccess;
+        armed = record ? hipEventRecord(ev.start, st) == hipSuccess : true;
     }
+    hipEvent_t start() const { return armed && !record ? ev.start : nullptr; }
+    hipEvent_t stop() const { return armed && !record ? ev.stop : nullptr; }
     ~ScopedKernelTimer()
     {
         if (!armed) return;
-        (void)hipEventRecord(ev.stop, st);
+        if (record) (void)hipEventRecord(ev.stop, st);
         std::lock_guard<std::mutex> lock(g_timer.mu);
         g_timer.pairs[which].push_back(ev);
     }

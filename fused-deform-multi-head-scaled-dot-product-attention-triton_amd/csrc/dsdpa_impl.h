@@ -77,7 +77,8 @@ int launch_fwd_gather(const void *q, const void *k, const void *v, const float *
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(0, st);
-    hipLaunchKernelGGL((fwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+    hipExtLaunchKernelGGL((fwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                          timer.start(), timer.stop(), 0,
                        q, k, v, coords, out, lse, dm);
     return check_launch();
 }
@@ -90,7 +91,8 @@ int launch_bwd_gather(const void *q, const void *k, const void *v, const float *
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(1, st);
-    hipLaunchKernelGGL((bwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+    hipExtLaunchKernelGGL((bwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                          timer.start(), timer.stop(), 0,
                        q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm);
     return check_launch();
 }
@@ -104,10 +106,12 @@ int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const floa
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(2, st);
     if (dcoords)
-        hipLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+        hipExtLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                              timer.start(), timer.stop(), 0,
                            q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm);
     else
-        hipLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+        hipExtLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                              timer.start(), timer.stop(), 0,
                            q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm);
     return check_launch();
 }
@@ -167,7 +171,8 @@ int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const floa
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(1, st);
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kTileWaves * kWave), smem, st,
+    hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kTileWaves * kWave), smem, st,
+                          timer.start(), timer.stop(), 0,
                        q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, tg);
     return check_launch();
 }
@@ -187,7 +192,8 @@ static inline int launch_plane_descriptors(const float *coords, const Dims &dm, 
     const long long blocks = (waves * kWave + kDescThreads - 1) / kDescThreads;
     if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
     ScopedKernelTimer timer(timer_slot, st);
-    hipLaunchKernelGGL(plane_descriptor_kernel, dim3((unsigned)blocks), dim3(kDescThreads), 0, st, coords, dm,
+    hipExtLaunchKernelGGL(plane_descriptor_kernel, dim3((unsigned)blocks), dim3(kDescThreads), 0, st,
+                          timer.start(), timer.stop(), 0, coords, dm,
                        (float4 *)(table + dl.w), (uint32_t *)(table + dl.e));
     return check_launch();
 }
@@ -209,7 +215,8 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float4 *
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(0, st);
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
+    hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
+                          timer.start(), timer.stop(), 0,
                        q, k, v, desc_w, desc_e, out, lse, dm);
     return check_launch();
 }
@@ -232,7 +239,8 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(2, st);
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
+    hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
+                          timer.start(), timer.stop(), 0,
                        q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, dm);
     return check_launch();
 }
@@ -290,7 +298,8 @@ template <typename S, int D> struct CellChunk {
     static constexpr int value = S::kBytes == 2 ? (D <= 64 ? 4 : 8) : (D <= 128 ? 4 : 8);
 };
 
-static inline int launch_binning(const float *coords, const Dims &dm, const WorkspaceLayout &wl, char *ws, hipStream_t st)
+static inline int launch_binning(const float *coords, const Dims &dm, const WorkspaceLayout &wl, char *ws,
+                                 hipStream_t st)
 {
     unsigned *counters = (unsigned *)(ws + wl.counters);
     unsigned *start = (unsigned *)(ws + wl.start);
@@ -315,20 +324,24 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(k1),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * hist_bytes));
         if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
-        hipLaunchKernelGGL(k0, dim3((unsigned)blocks), dim3(kBinLdsThreads), hist_bytes, st,
+        hipExtLaunchKernelGGL(k0, dim3((unsigned)blocks), dim3(kBinLdsThreads), hist_bytes, st,
+                              timer.start(), nullptr, 0,
                            coords, dm, wl.NC, lchunk, nlc, counters, sorted);
         hipLaunchKernelGGL(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st, counters, start, wl.NC);
-        hipLaunchKernelGGL(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
+        hipExtLaunchKernelGGL(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
+                              nullptr, timer.stop(), 0,
                            coords, dm, wl.NC, lchunk, nlc, counters, sorted);
         return check_launch();
     }
     const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
     const long long blocks = (total + kBinThreads - 1) / kBinThreads;
     if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(bin_samples_kernel<0>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
+    hipExtLaunchKernelGGL(bin_samples_kernel<0>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
+                          timer.start(), nullptr, 0,
                        coords, dm, wl.NC, counters, sorted);
     hipLaunchKernelGGL(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st, counters, start, wl.NC);
-    hipLaunchKernelGGL(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
+    hipExtLaunchKernelGGL(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
+                          nullptr, timer.stop(), 0,
                        coords, dm, wl.NC, counters, sorted);
     return check_launch();
 }
@@ -348,9 +361,10 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
         const long long nwork = (long long)dm.B * dm.H * dm.V * ncells;
         const long long blocks = (nwork + kCellWaves - 1) / kCellWaves;
         if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
-        if (blocks == 0) continue;
-        hipLaunchKernelGGL((bwd_dkdv_cell_kernel<S, D, DC>), dim3((unsigned)blocks), dim3(kCellWaves * kWave), 0, st,
-                           q, k, v, coords, lse, delta, dout, start, sorted, dk_acc, dv_acc, dm, NC, colour);
+        const bool first = colour <= 0, last = colour < 0 || colour == 3;
+        hipExtLaunchKernelGGL((bwd_dkdv_cell_kernel<S, D, DC>), dim3((unsigned)blocks), dim3(kCellWaves * kWave), 0, st,
+                              first ? timer.start() : nullptr, last ? timer.stop() : nullptr, 0, q, k, v, coords,
+                              lse, delta, dout, start, sorted, dk_acc, dv_acc, dm, NC, colour);
     }
     return check_launch();
 }
@@ -363,7 +377,7 @@ static inline int launch_list_ordering(const Dims &dm, const WorkspaceLayout &wl
     const size_t ids = groups * M, segs = groups * (size_t)wl.NC;
     if (ids > 0xffffffffull || segs > 0x7fffffffull) return DSDPA_ERR_TOO_LARGE;
     unsigned *seg_begin = (unsigned *)(ws + wl.seg), *seg_end = seg_begin + segs;
-    ScopedKernelTimer timer(3, st);
+    ScopedKernelTimer timer(3, st, /*record=*/true);      // the sort launches its own kernels
     hipLaunchKernelGGL(cell_segments_kernel, dim3((unsigned)((segs + 255) / 256)), dim3(256), 0, st,
                        (const unsigned *)(ws + wl.start), wl.NC, (unsigned)M, (unsigned)segs, seg_begin, seg_end);
     int rc = check_launch();
