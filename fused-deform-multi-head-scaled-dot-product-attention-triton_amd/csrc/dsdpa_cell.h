@@ -250,6 +250,22 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
 #pragma unroll
         for (int d = 0; d < DC; ++d) { aK[tpi][d] = 0.f; aV[tpi][d] = 0.f; }
     }
+    // fp32 storage: the cell's taps are turned, once, into the coefficients of the bilinear form
+    //   blend(fx, fy) = T00 + fx*(T01 - T00) + fy*(T10 - T00) + fx*fy*(T00 - T01 - T10 + T11)
+    // so that a sample's blend costs 3 multiply-adds per element instead of 4, and the sums are kept as the
+    // matching moments (sum c, sum c*fx, sum c*fy, sum c*fx*fy times the query row), turned back into the
+    // four pixels' sums after the loop. (Taps outside the image were loaded as zero rows.)
+    if constexpr (!kPacked) {
+#pragma unroll
+        for (int d = 0; d < DC; ++d) {
+            kt[3][d] = (kt[3][d] - kt[2][d]) - (kt[1][d] - kt[0][d]);
+            kt[1][d] -= kt[0][d];
+            kt[2][d] -= kt[0][d];
+            vt[3][d] = (vt[3][d] - vt[2][d]) - (vt[1][d] - vt[0][d]);
+            vt[1][d] -= vt[0][d];
+            vt[2][d] -= vt[0][d];
+        }
+    }
     const float qscale = dm.sm_scale * kLog2e;
     const size_t M = (size_t)dm.V * dm.L * dm.P;
     const unsigned *list = sorted + grp * M;
@@ -293,7 +309,10 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
         // entries past the end of the list repeat its last sample with zero weights: they add nothing
         const bool live = c0 + (unsigned)lane < hi;
         wave_lds_sync();
-        s_w[wave][lane] = live ? make_float4(gx * gy, fx * gy, gx * fy, fx * fy) : make_float4(0.f, 0.f, 0.f, 0.f);
+        if constexpr (kPacked)
+            s_w[wave][lane] = live ? make_float4(gx * gy, fx * gy, gx * fy, fx * fy) : make_float4(0.f, 0.f, 0.f, 0.f);
+        else
+            s_w[wave][lane] = make_float4(fx, fy, fx * fy, live ? 1.0f : 0.0f);
         s_row[wave][lane] = (s1 * view_rows + l) * kRowBytes;
         wave_lds_sync();
         const int cnt = (int)min((unsigned)kWave, hi - c0);
@@ -319,20 +338,25 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
                           fmaf(w.y, packed_dot<S, DC>(dop, vtp[1]),
                                fmaf(w.z, packed_dot<S, DC>(dop, vtp[2]), w.w * packed_dot<S, DC>(dop, vtp[3]))));
             } else {
+                // w = (fx, fy, fx*fy, live)
 #pragma unroll
                 for (int d = 0; d < DC; ++d) {
-                    const float kk = fmaf(w.x, kt[0][d], fmaf(w.y, kt[1][d], fmaf(w.z, kt[2][d], w.w * kt[3][d])));
-                    const float vv = fmaf(w.x, vt[0][d], fmaf(w.y, vt[1][d], fmaf(w.z, vt[2][d], w.w * vt[3][d])));
+                    const float kk = fmaf(w.z, kt[3][d], fmaf(w.y, kt[2][d], fmaf(w.x, kt[1][d], kt[0][d])));
+                    const float vv = fmaf(w.z, vt[3][d], fmaf(w.y, vt[2][d], fmaf(w.x, vt[1][d], vt[0][d])));
                     dot = fmaf(qf[d], kk, dot);
                     dp = fmaf(dof[d], vv, dp);
                 }
             }
             dot = group_sum<G>(dot);
             dp = group_sum<G>(dp);
-            const float p_n = __builtin_amdgcn_exp2f(dot * qscale - lse);
+            float p_n = __builtin_amdgcn_exp2f(dot * qscale - lse);
+            if constexpr (!kPacked) p_n *= w.w;                    // entries past the end of the list
             const float dss = p_n * (dp - delta) * dm.sm_scale;
-            const float ck[4] = { w.x * dss, w.y * dss, w.z * dss, w.w * dss };
-            const float cv[4] = { w.x * p_n, w.y * p_n, w.z * p_n, w.w * p_n };
+            // packed: per-tap weights; fp32: the moments 1, fx, fy, fx*fy
+            const float ck[4] = { kPacked ? w.x * dss : dss, kPacked ? w.y * dss : w.x * dss,
+                                  kPacked ? w.z * dss : w.y * dss, kPacked ? w.w * dss : w.z * dss };
+            const float cv[4] = { kPacked ? w.x * p_n : p_n, kPacked ? w.y * p_n : w.x * p_n,
+                                  kPacked ? w.z * p_n : w.y * p_n, kPacked ? w.w * p_n : w.z * p_n };
 #pragma unroll
             for (int tpi = 0; tpi < 4; ++tpi) {
 #pragma unroll
@@ -353,6 +377,18 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
                 aK[tpi][d] += __shfl_xor(aK[tpi][d], off, kWave);
                 aV[tpi][d] += __shfl_xor(aV[tpi][d], off, kWave);
             }
+        }
+    }
+    if constexpr (!kPacked) {
+        // moments -> pixels: w00 = 1 - fx - fy + fx*fy, w01 = fx - fx*fy, w10 = fy - fx*fy, w11 = fx*fy
+#pragma unroll
+        for (int d = 0; d < DC; ++d) {
+            aK[0][d] = (aK[0][d] - aK[1][d]) - (aK[2][d] - aK[3][d]);
+            aK[1][d] -= aK[3][d];
+            aK[2][d] -= aK[3][d];
+            aV[0][d] = (aV[0][d] - aV[1][d]) - (aV[2][d] - aV[3][d]);
+            aV[1][d] -= aV[3][d];
+            aV[2][d] -= aV[3][d];
         }
     }
     if (slot == 0) {
