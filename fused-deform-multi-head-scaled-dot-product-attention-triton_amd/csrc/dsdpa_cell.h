@@ -183,12 +183,25 @@ __device__ __forceinline__ void load_tap_or_zero(const char *base, int pix, int 
     }
 }
 
+// Which cells one launch of the dk/dv kernel covers, and the divisors that decode a work index into
+// (b, h, s2, cell) with multiply-shift instead of integer division (the decode is scalar code every
+// wave runs before it knows whether its cell is empty).
+// colour < 0: all cells, per-cell sums flushed with float atomics (a pixel belongs to four cells).
+// colour 0..3 (deterministic backward): only the cells with (row parity, column parity) = colour; no
+// two of them share a pixel, so the flush is a plain read-add-write, and the four launches, one
+// after the other, add every pixel's four contributions in a fixed order.
+struct CellGrid {
+    int colour, oy, ox, step, ncx, ncells;
+    unsigned nwork;                         // B*H*V*ncells < 2^31
+    FastDiv div_cells, div_ncx, div_v, div_h;
+};
+
 template <typename S, int D, int DC>
 __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 3 : 2)) void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float *__restrict__ lse_, const float *__restrict__ delta_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
-    float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC, int colour)
+    float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC, CellGrid cg)
 {
     constexpr int G = D / DC;
     constexpr int NS = kWave / G;
@@ -197,31 +210,25 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
     __shared__ unsigned s_row[kCellWaves][kWave];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
-    const long long work = (long long)xcd_logical_block(blockIdx.x, gridDim.x) * kCellWaves + wave;
-    // colour < 0: all cells, per-cell sums flushed with float atomics (a pixel belongs to four cells).
-    // colour 0..3 (deterministic backward): only the cells with (row parity, column parity) = colour; no
-    // two of them share a pixel, so the flush is a plain read-add-write, and the four launches, one
-    // after the other, add every pixel's four contributions in a fixed order.
-    const int cw = dm.Wimg + 1, ch = dm.Himg + 1;
-    const int oy = colour < 0 ? 0 : colour >> 1, ox = colour < 0 ? 0 : colour & 1, step = colour < 0 ? 1 : 2;
-    const int ncx = (cw - ox + step - 1) / step, ncy = (ch - oy + step - 1) / step;
-    const int ncells = ncx * ncy;
-    const long long nwork = (long long)dm.B * dm.H * dm.V * ncells;
-    if (work >= nwork || ncells == 0) return;
+    const unsigned work = (unsigned)xcd_logical_block(blockIdx.x, gridDim.x) * kCellWaves + wave;
+    if (work >= cg.nwork) return;
+    const int colour = cg.colour;
     // plane-major: (b, h, s2, cell)
-    const int ci = (int)(work % ncells);
-    const int cell = (ci / ncx * step + oy) * cw + (ci % ncx) * step + ox;
-    long long t = work / ncells;
-    const int s2 = (int)(t % dm.V);
-    t /= dm.V;
-    const int h = (int)(t % dm.H);
-    const int b = (int)(t / dm.H);
+    unsigned t = cg.div_cells.div(work);
+    const int ci = (int)(work - t * (unsigned)cg.ncells);
+    const int cyi = (int)cg.div_ncx.div((unsigned)ci);
+    const int cy = cyi * cg.step + cg.oy, cx = (ci - cyi * cg.ncx) * cg.step + cg.ox;   // on the (Himg+1) x (Wimg+1) grid
+    const int cell = cy * (dm.Wimg + 1) + cx;
+    const unsigned bh = cg.div_v.div(t);
+    const int s2 = (int)(t - bh * (unsigned)dm.V);
+    const int b = (int)cg.div_h.div(bh);
+    const int h = (int)(bh - (unsigned)b * (unsigned)dm.H);
     const size_t grp = (size_t)b * dm.V + s2;
     const unsigned lo = start[grp * (NC + 1) + cell], hi = start[grp * (NC + 1) + cell + 1];
     if (lo == hi) return;
 
     const int g = lane % G, slot = lane / G, lane_elem = g * DC;
-    const int y0 = cell / (dm.Wimg + 1) - 1, x0 = cell % (dm.Wimg + 1) - 1;
+    const int y0 = cy - 1, x0 = cx - 1;
     const bool vy0 = y0 >= 0, vy1 = y0 + 1 < dm.Himg, vx0 = x0 >= 0, vx1 = x0 + 1 < dm.Wimg;
     const bool tv[4] = { vy0 && vx0, vy0 && vx1, vy1 && vx0, vy1 && vx1 };
     const int tpix[4] = { y0 * dm.Wimg + x0, y0 * dm.Wimg + x0 + 1, (y0 + 1) * dm.Wimg + x0,

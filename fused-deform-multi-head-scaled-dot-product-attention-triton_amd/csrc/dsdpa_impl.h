@@ -356,15 +356,25 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
     ScopedKernelTimer timer(1, st);
     for (int colour = deterministic ? 0 : -1; colour < (deterministic ? 4 : 0); ++colour) {
         const int cw = dm.Wimg + 1, ch = dm.Himg + 1;
-        const int oy = colour < 0 ? 0 : colour >> 1, ox = colour < 0 ? 0 : colour & 1, step = colour < 0 ? 1 : 2;
-        const long long ncells = (long long)((cw - ox + step - 1) / step) * ((ch - oy + step - 1) / step);
-        const long long nwork = (long long)dm.B * dm.H * dm.V * ncells;
-        const long long blocks = (nwork + kCellWaves - 1) / kCellWaves;
-        if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+        CellGrid cg;
+        cg.colour = colour;
+        cg.oy = colour < 0 ? 0 : colour >> 1;
+        cg.ox = colour < 0 ? 0 : colour & 1;
+        cg.step = colour < 0 ? 1 : 2;
+        cg.ncx = (cw - cg.ox + cg.step - 1) / cg.step;
+        cg.ncells = cg.ncx * ((ch - cg.oy + cg.step - 1) / cg.step);
+        const long long nwork = (long long)dm.B * dm.H * dm.V * cg.ncells;
+        if (nwork >= 0x7fffffffll - kCellWaves) return DSDPA_ERR_TOO_LARGE;
+        cg.nwork = (unsigned)nwork;
+        cg.div_cells = FastDiv::make((unsigned)cg.ncells);
+        cg.div_ncx = FastDiv::make((unsigned)cg.ncx);
+        cg.div_v = FastDiv::make((unsigned)dm.V);
+        cg.div_h = FastDiv::make((unsigned)dm.H);
+        const unsigned blocks = (unsigned)((nwork + kCellWaves - 1) / kCellWaves);
         const bool first = colour <= 0, last = colour < 0 || colour == 3;
-        hipExtLaunchKernelGGL((bwd_dkdv_cell_kernel<S, D, DC>), dim3((unsigned)blocks), dim3(kCellWaves * kWave), 0, st,
+        hipExtLaunchKernelGGL((bwd_dkdv_cell_kernel<S, D, DC>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
                               first ? timer.start() : nullptr, last ? timer.stop() : nullptr, 0, q, k, v, coords,
-                              lse, delta, dout, start, sorted, dk_acc, dv_acc, dm, NC, colour);
+                              lse, delta, dout, start, sorted, dk_acc, dv_acc, dm, NC, cg);
     }
     return check_launch();
 }
