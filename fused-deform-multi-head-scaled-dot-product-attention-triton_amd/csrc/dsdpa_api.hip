@@ -1,6 +1,6 @@
 // C ABI of libdsdpa.so (declared in include/dsdpa.h): the extern "C" entry points and the shared
 // host-side state. The kernels and their launchers are compiled per storage type (dsdpa_f32.hip,
-// dsdpa_bf16.hip, dsdpa_f16.hip).
+// dsdpa_bf16.hip, dsdpa_f16.hip); the list sort of the deterministic backward lives in dsdpa_sort.hip.
 #include "dsdpa_host.h"
 #include "dsdpa_common.h"
 

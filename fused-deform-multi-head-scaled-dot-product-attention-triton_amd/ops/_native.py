@@ -85,12 +85,13 @@ def set_path(path):
 
 
 def timer_enable(on):
-    """Bracket every main fwd/bwd kernel launch (process-wide) with HIP events; returns the previous state."""
+    """Attach HIP events to every main fwd/bwd kernel launch (process-wide); returns the previous state."""
     return load().dsdpa_timer_enable(1 if on else 0)
 
 
 def timer_collect(which):
-    """(total kernel ms, launches) of the events recorded since the last collect; which: 0 fwd, 1 bwd."""
+    """(total kernel ms, launches) since the last collect; which: 0 forward, 1 backward dk/dv, 2 backward dq,
+    3 cell binning (its launches together), 4 tap table fill."""
     ms, n = ctypes.c_double(0.0), ctypes.c_int(0)
     check(load().dsdpa_timer_collect(int(which), ctypes.byref(ms), ctypes.byref(n)))
     return ms.value, n.value

@@ -11,7 +11,8 @@
  *
  * Conventions
  *   - plain pointers and sizes only; every pointer is DEVICE memory owned by
- *     the caller; nothing is allocated or freed by the library;
+ *     the caller; nothing is allocated or freed by the library (scratch
+ *     memory comes in as the `workspace` arguments);
  *   - tensors are contiguous, row-major:
  *         q, k, v, out, dout, dq, dk, dv : [B][V][H][L][D],  L = Himg*Wimg
  *         coords : [B][V][L][V][P][2] float32, (x, y) normalised to [0, 1],
@@ -160,12 +161,14 @@ int dsdpa_set_path(int path);
 /*
  * Kernel timer, for measurement (the reference times whole calls with
  * triton.testing.do_bench, benchmark.py:90). While enabled (process-wide),
- * every main forward / backward kernel launch is bracketed by a pair of
- * HIP events recorded on the launch stream. dsdpa_timer_collect waits for the
- * recorded events, returns the summed kernel time and the number of launches
- * for `which` (0 = forward kernel, 1 = backward dk/dv kernel, 2 = backward dq
- * kernel, 3 = the three cell-binning launches taken together, 4 = the launches
- * that fill the per-coordinate table, one per forward and one per backward call) and releases them.
+ * every main forward / backward kernel launch carries a pair of HIP events on
+ * the launch stream (attached to the kernel's own dispatch: its start and end
+ * timestamps; a timed launch costs a few microseconds of GPU idle time).
+ * dsdpa_timer_collect waits for the events, returns the summed kernel time and
+ * the number of launches for `which` (0 = forward kernel, 1 = backward dk/dv
+ * kernel, 2 = backward dq kernel, 3 = the three cell-binning launches taken
+ * together, 4 = the launches that fill the per-coordinate table, one per
+ * forward and one per backward call) and releases them.
  * dsdpa_timer_enable returns the previous state.
  */
 int dsdpa_timer_enable(int on);
