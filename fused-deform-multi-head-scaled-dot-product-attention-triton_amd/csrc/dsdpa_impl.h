@@ -204,20 +204,15 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float4 *
 {
     constexpr int DC = Chunk<S, D>::value;
     const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes;
-    constexpr int QW = PlaneRows<DC>::value;
-    const int rows_per_block = kPlaneWaves * QW;
+    const int rows_per_block = kPlaneWaves * (kWave / (D / DC));
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
-    constexpr bool kCanPair = QW % 2 == 0;
-    // (a P == 32 compile-time instantiation was tried: the unrolled chunk spills 432 bytes per lane)
-    auto kern = (kCanPair && dm.P <= 32) ? fwd_plane_kernel<S, D, DC, QW, kCanPair, 0>
-                                         : fwd_plane_kernel<S, D, DC, QW, false, 0>;
+    auto kern = fwd_slot_kernel<S, D, DC>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(0, st);
     hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
-                          timer.start(), timer.stop(), 0,
-                       q, k, v, desc_w, desc_e, out, lse, dm);
+                          timer.start(), timer.stop(), 0, q, k, v, desc_w, desc_e, out, lse, dm);
     return check_launch();
 }
 
@@ -229,19 +224,15 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
 {
     constexpr int DC = Chunk<S, D>::value;
     const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes;
-    constexpr int QW = PlaneRows<DC>::value;
-    const int rows_per_block = kPlaneWaves * QW;
+    const int rows_per_block = kPlaneWaves * (kWave / (D / DC));
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
-    constexpr bool kCanPair = QW % 2 == 0;
-    auto kern = (kCanPair && dm.P <= 32) ? bwd_dq_plane_kernel<S, D, DC, QW, kCanPair, 0>
-                                         : bwd_dq_plane_kernel<S, D, DC, QW, false, 0>;
+    auto kern = bwd_dq_slot_kernel<S, D, DC>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(2, st);
     hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
-                          timer.start(), timer.stop(), 0,
-                       q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, dm);
+                          timer.start(), timer.stop(), 0, q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, dm);
     return check_launch();
 }
 

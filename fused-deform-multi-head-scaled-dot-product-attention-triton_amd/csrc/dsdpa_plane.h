@@ -536,4 +536,268 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
     }
 }
 
+// ====================================================================== one query row per slot
+// The same staged planes and tap table, with the rows dealt differently: slot s of a wave (its G
+// lanes) owns query row s of the wave's NS = 64/G rows for the whole kernel, and in every trip the NS
+// slots consume one sample each -- of NS different rows. A lane then carries the state of ONE row (q,
+// accumulator, running max and sum: ~10 registers instead of ~40 for four rows), there is nothing to
+// merge across slots at the end, every trip is full whatever P is (the kernels above leave slots idle
+// when P is not a multiple of NS), and a workgroup covers 16*NS rows, so each staged plane serves
+// twice as many rows.
+//
+// Per key view and pass, lane (slot, g) fetches the table entry of sample c0+g of its own row: G samples
+// per row and pass, parked sample-major (entry of trip t and slot s at t*NS + s, so the NS slots of a
+// trip read one contiguous stretch). Odd slots swap the two samples of every pair of trips: with the
+// table's alternating bank-half order, neighbouring slots then gather from opposite halves in every trip.
+template <typename S, int D>
+__device__ __forceinline__ void stage_slot_descriptors(const float4 *__restrict__ desc_w,
+                                                       const uint32_t *__restrict__ desc_e, size_t d_row, int P,
+                                                       int c0, int g, int slot, int G_, int NS_, float4 *s_w,
+                                                       int2 *s_e)
+{
+    constexpr int kRow = D * S::kBytes;
+    const int n = c0 + g;
+    const bool valid = n < P;
+    const size_t i = d_row + (valid ? n : 0);
+    float4 w = desc_w[i];
+    const uint32_t c = desc_e[i];
+    if (!valid) w = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int cnt = min(G_, P - c0);                       // samples of this pass (same for every row)
+    const int trip = (cnt & 1) == 0 ? g ^ (slot & 1) : g;    // pair swap only when no pair straddles the end
+    wave_lds_sync();
+    s_w[trip * NS_ + slot] = w;
+    s_e[trip * NS_ + slot] = make_int2((int)(c & 0xffffu) * kRow, (int)(c >> 16) * kRow);
+    wave_lds_sync();
+}
+
+template <typename S, int D, int DC>
+__global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
+    const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
+    const float4 *__restrict__ desc_w, const uint32_t *__restrict__ desc_e, void *__restrict__ out_,
+    float *__restrict__ lse_, Dims dm)
+{
+    constexpr int G = D / DC, NS = kWave / G;
+    constexpr int kRow = D * S::kBytes;
+    constexpr bool kPacked = S::kBytes == 2;
+    static_assert(G >= 2 && G <= 16 && G * DC == D, "lane split");
+    extern __shared__ __attribute__((aligned(kPlaneLdsAlign))) unsigned char smem[];
+    const int img_bytes = plane_lds_bytes<S, D>(dm.L);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
+    int2 *s_e = reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
+
+    const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * NS);
+    const int nq = dm.V * dm.L;
+    const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
+    const float qscale = dm.sm_scale * kLog2e;
+    const uint32_t lbase = lds_offset(smem) + lane_byte;
+
+    zero_plane_pads<S, D>(smem, dm.L);
+
+    const int qidx = pb.qbase + wave * NS + slot;
+    const bool have = qidx < nq;
+    const unsigned qc = (unsigned)(have ? qidx : nq - 1);
+    const unsigned s1 = dm.divL.div(qc), l = qc - s1 * (unsigned)dm.L;
+    const size_t row = (((size_t)pb.b * dm.V + s1) * dm.H + pb.h) * dm.L + l;
+    const size_t crow = (((size_t)pb.b * dm.V + s1) * dm.L + l) * (size_t)dm.N;
+    float qf[DC], acc[DC];
+    uint32_t qp[kPacked ? DC / 2 : 1];
+    if constexpr (kPacked) {
+        load_packed<S, DC>((const char *)q_ + (row * D + lane_elem) * S::kBytes, qp);
+    } else {
+        load_chunk<S, DC>((const char *)q_ + (row * D + lane_elem) * S::kBytes, qf);
+#pragma unroll
+        for (int d = 0; d < DC; ++d) qf[d] *= qscale;
+    }
+    float m = kNegBig, lsum = 0.f;
+#pragma unroll
+    for (int d = 0; d < DC; ++d) acc[d] = 0.f;
+
+    for (int s2 = 0; s2 < dm.V; ++s2) {
+        const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;
+        __syncthreads();                                       // the previous view's readers are done
+        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, 0);
+        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
+        __syncthreads();
+        for (int c0 = 0; c0 < dm.P; c0 += G) {
+            stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g, slot, G, NS, s_w,
+                                         s_e);
+            const int cnt = min(G, dm.P - c0);
+            float sv[G];
+            float mc = kNegBig;
+#pragma unroll
+            for (int t = 0; t < G; ++t) {
+                sv[t] = kNegBig;
+                if (t < cnt) {
+                    const float4 w = s_w[t * NS + slot];
+                    const int2 e = s_e[t * NS + slot];
+                    const uint32_t at = e.x + lbase, ab = e.y + lbase;
+                    const unsigned char *top = lds_at(at), *bot = lds_at(ab);
+                    const unsigned char *topr = lds_at((at ^ kRow) + 2 * kRow), *botr = lds_at((ab ^ kRow) + 2 * kRow);
+                    float dot = 0.f;
+                    if constexpr (kPacked) {
+                        dot = qscale * tap_dot16<S, DC>(top, topr, bot, botr, w, qp);
+                    } else {
+                        float t0[DC], t1[DC], t2[DC], t3[DC];
+                        load_chunk<S, DC>(top, t0);
+                        load_chunk<S, DC>(topr, t1);
+                        load_chunk<S, DC>(bot, t2);
+                        load_chunk<S, DC>(botr, t3);
+#pragma unroll
+                        for (int d = 0; d < DC; ++d) {
+                            const float kk = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
+                            dot = fmaf(qf[d], kk, dot);
+                        }
+                    }
+                    sv[t] = group_sum<G>(dot);
+                    mc = fmaxf(mc, sv[t]);
+                }
+            }
+            const float m_new = fmaxf(m, mc);
+            const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+            m = m_new;
+            lsum *= alpha;
+#pragma unroll
+            for (int d = 0; d < DC; ++d) acc[d] *= alpha;
+#pragma unroll
+            for (int t = 0; t < G; ++t) {
+                if (t < cnt) {
+                    const float p = __builtin_amdgcn_exp2f(sv[t] - m_new);
+                    lsum += p;
+                    const float4 w = s_w[t * NS + slot];
+                    const int2 e = s_e[t * NS + slot];
+                    const uint32_t at = e.x + lbase, ab = e.y + lbase;
+                    float t0[DC], t1[DC], t2[DC], t3[DC];
+                    load_chunk<S, DC>(lds_at(at ^ kRow), t0);                  // V, left taps
+                    load_chunk<S, DC>(lds_at(at + 2 * kRow), t1);              // V, right taps
+                    load_chunk<S, DC>(lds_at(ab ^ kRow), t2);
+                    load_chunk<S, DC>(lds_at(ab + 2 * kRow), t3);
+                    const float c0w = p * w.x, c1w = p * w.y, c2w = p * w.z, c3w = p * w.w;
+#pragma unroll
+                    for (int d = 0; d < DC; ++d)
+                        acc[d] = fmaf(c0w, t0[d], fmaf(c1w, t1[d], fmaf(c2w, t2[d], fmaf(c3w, t3[d], acc[d]))));
+                }
+            }
+        }
+    }
+
+    if (have) {
+        const float inv = 1.0f / lsum;
+#pragma unroll
+        for (int d = 0; d < DC; ++d) acc[d] *= inv;
+        store_chunk<S, DC>((char *)out_ + (row * D + lane_elem) * S::kBytes, acc);
+        if (g == 0) lse_[row] = m + __log2f(lsum);
+    }
+}
+
+template <typename S, int D, int DC>
+__global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
+    const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
+    const float4 *__restrict__ desc_w, const uint32_t *__restrict__ desc_e, const void *__restrict__ out_,
+    const float *__restrict__ lse_, const void *__restrict__ dout_, void *__restrict__ dq_,
+    float *__restrict__ delta_, Dims dm)
+{
+    constexpr int G = D / DC, NS = kWave / G;
+    constexpr int kRow = D * S::kBytes;
+    constexpr bool kPacked = S::kBytes == 2;
+    static_assert(G >= 2 && G <= 16 && G * DC == D, "lane split");
+    extern __shared__ __attribute__((aligned(kPlaneLdsAlign))) unsigned char smem[];
+    const int img_bytes = plane_lds_bytes<S, D>(dm.L);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
+    int2 *s_e = reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
+
+    const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * NS);
+    const int nq = dm.V * dm.L;
+    const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
+    const float qscale = dm.sm_scale * kLog2e;
+    const uint32_t lbase = lds_offset(smem) + lane_byte;
+
+    zero_plane_pads<S, D>(smem, dm.L);
+
+    const int qidx = pb.qbase + wave * NS + slot;
+    const bool have = qidx < nq;
+    const unsigned qc = (unsigned)(have ? qidx : nq - 1);
+    const unsigned s1 = dm.divL.div(qc), l = qc - s1 * (unsigned)dm.L;
+    const size_t row = (((size_t)pb.b * dm.V + s1) * dm.H + pb.h) * dm.L + l;
+    const size_t crow = (((size_t)pb.b * dm.V + s1) * dm.L + l) * (size_t)dm.N;
+    const size_t roff = (row * D + lane_elem) * S::kBytes;
+    float qf[DC], dof[DC], dqa[DC];
+    uint32_t dop[kPacked ? DC / 2 : 1];
+    float delta;
+    {
+        float of[DC];
+        load_chunk<S, DC>((const char *)q_ + roff, qf);
+        load_chunk<S, DC>((const char *)dout_ + roff, dof);
+        if constexpr (kPacked) load_packed<S, DC>((const char *)dout_ + roff, dop);
+        load_chunk<S, DC>((const char *)out_ + roff, of);
+        float dl = 0.f;
+#pragma unroll
+        for (int d = 0; d < DC; ++d) { dl = fmaf(dof[d], of[d], dl); dqa[d] = 0.f; }
+        delta = group_sum<G>(dl);              // the reference's _bwd_preprocess, fused
+    }
+    const float lse = lse_[row];
+    if (have && g == 0) delta_[row] = delta;
+
+    for (int s2 = 0; s2 < dm.V; ++s2) {
+        const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;
+        __syncthreads();
+        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, 0);
+        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
+        __syncthreads();
+        for (int c0 = 0; c0 < dm.P; c0 += G) {
+            stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g, slot, G, NS, s_w,
+                                         s_e);
+            const int cnt = min(G, dm.P - c0);
+            for (int t = 0; t < cnt; ++t) {
+                const float4 w = s_w[t * NS + slot];
+                const int2 e = s_e[t * NS + slot];
+                const uint32_t at = e.x + lbase, ab = e.y + lbase;
+                const unsigned char *top = lds_at(at), *bot = lds_at(ab);                      // K left; V right at +2*ROW
+                const unsigned char *topx = lds_at(at ^ kRow), *botx = lds_at(ab ^ kRow);      // V left; K right at +2*ROW
+                float kk[DC];
+                float dot = 0.f, dp = 0.f;
+                {
+                    float t0[DC], t1[DC], t2[DC], t3[DC];
+                    load_chunk<S, DC>(top, t0);
+                    load_chunk<S, DC>(topx + 2 * kRow, t1);
+                    load_chunk<S, DC>(bot, t2);
+                    load_chunk<S, DC>(botx + 2 * kRow, t3);
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) {
+                        kk[d] = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
+                        dot = fmaf(qf[d], kk[d], dot);
+                    }
+                }
+                if constexpr (kPacked) {
+                    dp = tap_dot16<S, DC>(topx, top + 2 * kRow, botx, bot + 2 * kRow, w, dop);
+                } else {
+                    float u0[DC], u1[DC], u2[DC], u3[DC];
+                    load_chunk<S, DC>(topx, u0);
+                    load_chunk<S, DC>(top + 2 * kRow, u1);
+                    load_chunk<S, DC>(botx, u2);
+                    load_chunk<S, DC>(bot + 2 * kRow, u3);
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) {
+                        const float vv = fmaf(w.x, u0[d], fmaf(w.y, u1[d], fmaf(w.z, u2[d], w.w * u3[d])));
+                        dp = fmaf(dof[d], vv, dp);
+                    }
+                }
+                dot = group_sum<G>(dot);
+                dp = group_sum<G>(dp);
+                const float p = __builtin_amdgcn_exp2f(dot * qscale - lse);
+                const float ds = p * (dp - delta);
+#pragma unroll
+                for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
+            }
+        }
+    }
+
+    if (have) {
+#pragma unroll
+        for (int d = 0; d < DC; ++d) dqa[d] *= dm.sm_scale;
+        store_chunk<S, DC>((char *)dq_ + roff, dqa);
+    }
+}
+
 }  // namespace dsdpa
