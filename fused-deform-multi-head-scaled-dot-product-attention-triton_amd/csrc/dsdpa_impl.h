@@ -11,8 +11,6 @@
 namespace dsdpa {
 
 static_assert(kPlaneDescLdsBytes == (size_t)kPlaneDescBytes, "host and device agree on the descriptor block");
-// query rows per wave in the plane kernels: rows * elements-per-lane = 16 keeps them at 128 VGPRs
-template <int DC> struct PlaneRows { static constexpr int value = 16 / DC >= 1 ? 16 / DC : 1; };
 
 // ------------------------------------------------------------------ small kernels
 // Zero up to four 16-byte aligned float buffers in one launch (sizes in floats; unused slots have size 0).

@@ -2,12 +2,13 @@
 // K and V planes staged in LDS, for shapes where one (b, s2, h) plane pair
 // fits next to the per-wave tap descriptors.
 //
-// A workgroup of 16 waves owns 16*QW consecutive query rows of one (b, h) (rows
-// are counted over (s1, l), so a workgroup may straddle two query views) and
-// walks the V key views: stage K_s2 and V_s2 (coalesced 16-byte loads, kept in
-// the storage type), barrier, every wave runs its QW rows against the staged
-// planes, barrier, next view. The online-softmax state (forward) or the dq
-// accumulator (backward) of each row stays in registers across the views.
+// A workgroup of 16 waves owns 16*NS consecutive query rows of one (b, h) (NS = 64/G
+// rows per wave, one per slot of G lanes; rows are counted over (s1, l), so a
+// workgroup may straddle two query views) and walks the V key views: stage K_s2 and
+// V_s2 (coalesced 16-byte loads, kept in the storage type), barrier, every wave runs
+// its rows against the staged planes, barrier, next view. The online-softmax state
+// (forward) or the dq accumulator (backward) of a row stays in the registers of its
+// slot across the views.
 //
 // LDS image of a view: pixel p of the plane owns the 2*ROW bytes at (p + 1) * 2*ROW
 // (ROW = D * element size), with one zeroed pad pixel before pixel 0 and one after
@@ -149,401 +150,13 @@ static __global__ __launch_bounds__(kDescThreads) void plane_descriptor_kernel(
     }
 }
 
-// Descriptors for two rows of a wave and one key view in one 64-lane pass (the PAIR instantiations,
-// launched when P <= 32 and QW is even): lanes 0-31 take the even row, 32-63 the odd one, parked at
-// descriptor slots 0.. and 32..   d_even / d_odd: index of the rows' first table entry for this view.
-template <typename S, int D>
-__device__ __forceinline__ void stage_pair_descriptors(const float4 *__restrict__ desc_w,
-                                                       const uint32_t *__restrict__ desc_e, size_t d_even,
-                                                       size_t d_odd, int P, int lane, float4 *s_w, int2 *s_e)
-{
-    constexpr int kRow = D * S::kBytes;
-    const int n = lane & 31;
-    const bool valid = n < P;
-    const size_t i = ((lane < 32) ? d_even : d_odd) + (valid ? n : 0);
-    float4 w = desc_w[i];
-    const uint32_t c = desc_e[i];
-    if (!valid) w = make_float4(0.f, 0.f, 0.f, 0.f);
-    wave_lds_sync();
-    s_w[lane] = w;
-    s_e[lane] = make_int2((int)(c & 0xffffu) * kRow, (int)(c >> 16) * kRow);
-    wave_lds_sync();
-}
-
-// One row, samples c0 .. c0+63.
-template <typename S, int D>
-__device__ __forceinline__ void stage_row_descriptors(const float4 *__restrict__ desc_w,
-                                                      const uint32_t *__restrict__ desc_e, size_t d_row, int P,
-                                                      int c0, int lane, float4 *s_w, int2 *s_e)
-{
-    constexpr int kRow = D * S::kBytes;
-    const int n = c0 + lane;
-    const bool valid = n < P;
-    const size_t i = d_row + (valid ? n : 0);
-    float4 w = desc_w[i];
-    const uint32_t c = desc_e[i];
-    if (!valid) w = make_float4(0.f, 0.f, 0.f, 0.f);
-    wave_lds_sync();
-    s_w[lane] = w;
-    s_e[lane] = make_int2((int)(c & 0xffffu) * kRow, (int)(c >> 16) * kRow);
-    wave_lds_sync();
-}
-
-// ------------------------------------------------------------------ forward
-// One chunk (cnt <= 64 samples, descriptors at s_w/s_e[dbase ...]) of one row.
-// (Requesting the taps of slot-iteration it+1 before the arithmetic of iteration it -- a hand-made
-// software pipeline -- was measured: no gain for the forward, register spills for dq. The four waves
-// per SIMD already overlap the LDS pipe and the VALU.)
-// CNT > 0 fixes the sample count at compile time (branch-free, fully unrolled chunk).
-template <typename S, int D, int DC, int CNT>
-__device__ __forceinline__ void fwd_plane_chunk(uint32_t lbase, const float4 *s_w, const int2 *s_e,
-                                                int dbase, int cnt_rt, int slot,
-                                                const float (&qf)[DC], const uint32_t *qp, float qscale,
-                                                float &m, float &lsum, float (&acc)[DC])
-{
-    constexpr bool kPacked = S::kBytes == 2;
-    constexpr int G = D / DC, NS = kWave / G;
-    constexpr int ITS = CNT > 0 ? (CNT + NS - 1) / NS : G;
-    const int cnt = CNT > 0 ? CNT : cnt_rt;
-    constexpr int kRow = D * S::kBytes;
-    float sv[ITS];
-    float mc = kNegBig;
-#pragma unroll
-    for (int it = 0; it < ITS; ++it) {
-        sv[it] = kNegBig;
-        if (it * NS < cnt) {
-            const int j = it * NS + slot;
-            const float4 w = s_w[dbase + j];
-            const int2 e = s_e[dbase + j];
-            const uint32_t at = e.x + lbase, ab = e.y + lbase;     // lbase: LDS address of the image + this lane's byte
-            const unsigned char *top = lds_at(at), *bot = lds_at(ab);                                          // K, left taps
-            const unsigned char *topr = lds_at((at ^ kRow) + 2 * kRow), *botr = lds_at((ab ^ kRow) + 2 * kRow);   // K, right taps
-            float dot = 0.f;
-            if constexpr (kPacked) {
-                uint32_t qq[DC / 2];
-#pragma unroll
-                for (int i = 0; i < DC / 2; ++i) qq[i] = qp[i];
-                dot = qscale * tap_dot16<S, DC>(top, topr, bot, botr, w, qq);
-            } else {
-                float t0[DC], t1[DC], t2[DC], t3[DC];
-                load_chunk<S, DC>(top, t0);
-                load_chunk<S, DC>(topr, t1);
-                load_chunk<S, DC>(bot, t2);
-                load_chunk<S, DC>(botr, t3);
-#pragma unroll
-                for (int d = 0; d < DC; ++d) {
-                    const float kk = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
-                    dot = fmaf(qf[d], kk, dot);
-                }
-            }
-            dot = group_sum<G>(dot);
-            sv[it] = (j < cnt) ? dot : kNegBig;
-            mc = fmaxf(mc, sv[it]);
-        }
-    }
-    const float m_new = fmaxf(m, mc);
-    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
-    m = m_new;
-    lsum *= alpha;
-#pragma unroll
-    for (int d = 0; d < DC; ++d) acc[d] *= alpha;
-#pragma unroll
-    for (int it = 0; it < ITS; ++it) {
-        if (it * NS < cnt) {
-            const int j = it * NS + slot;
-            const float p = (j < cnt) ? __builtin_amdgcn_exp2f(sv[it] - m_new) : 0.f;
-            lsum += p;
-            const float4 w = s_w[dbase + j];
-            const int2 e = s_e[dbase + j];
-            const uint32_t at = e.x + lbase, ab = e.y + lbase;
-            float t0[DC], t1[DC], t2[DC], t3[DC];
-            load_chunk<S, DC>(lds_at(at ^ kRow), t0);                  // V, left taps
-            load_chunk<S, DC>(lds_at(at + 2 * kRow), t1);              // V, right taps
-            load_chunk<S, DC>(lds_at(ab ^ kRow), t2);
-            load_chunk<S, DC>(lds_at(ab + 2 * kRow), t3);
-            const float c0 = p * w.x, c1 = p * w.y, c2 = p * w.z, c3 = p * w.w;
-#pragma unroll
-            for (int d = 0; d < DC; ++d)
-                acc[d] = fmaf(c0, t0[d], fmaf(c1, t1[d], fmaf(c2, t2[d], fmaf(c3, t3[d], acc[d]))));
-        }
-    }
-}
-
-// PAIR: two rows per descriptor pass (P <= 32); PCNT > 0: P is exactly PCNT, known at compile time.
-template <typename S, int D, int DC, int QW, bool PAIR, int PCNT>
-__global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_plane_kernel(
-    const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
-    const float4 *__restrict__ desc_w, const uint32_t *__restrict__ desc_e, void *__restrict__ out_,
-    float *__restrict__ lse_, Dims dm)
-{
-    constexpr int G = D / DC;
-    static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
-    extern __shared__ __attribute__((aligned(kPlaneLdsAlign))) unsigned char smem[];
-    const int img_bytes = plane_lds_bytes<S, D>(dm.L);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
-    float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
-    int2 *s_e = reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
-
-    const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * QW);
-    const int nq = dm.V * dm.L;
-    const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
-    const float qscale = dm.sm_scale * kLog2e;
-    const uint32_t lbase = lds_offset(smem) + lane_byte;
-
-    zero_plane_pads<S, D>(smem, dm.L);
-
-    // fp32 storage: q widened and pre-scaled (qf); 16-bit storage: q as packed pairs (qp), scale on the logit
-    constexpr bool kPacked = S::kBytes == 2;
-    float qf[QW][DC], acc[QW][DC], m[QW], lsum[QW];
-    uint32_t qp[QW][kPacked ? DC / 2 : 1];
-    size_t row[QW], crow[QW];
-    bool have[QW];
-#pragma unroll
-    for (int qi = 0; qi < QW; ++qi) {
-        const int qidx = pb.qbase + wave * QW + qi;
-        have[qi] = qidx < nq;
-        const int qc = have[qi] ? qidx : nq - 1;
-        const int s1 = qc / dm.L, l = qc % dm.L;
-        row[qi] = (((size_t)pb.b * dm.V + s1) * dm.H + pb.h) * dm.L + l;
-        crow[qi] = (((size_t)pb.b * dm.V + s1) * dm.L + l) * (size_t)dm.N;
-        if constexpr (kPacked) {
-            load_packed<S, DC>((const char *)q_ + (row[qi] * D + lane_elem) * S::kBytes, qp[qi]);
-        } else {
-            load_chunk<S, DC>((const char *)q_ + (row[qi] * D + lane_elem) * S::kBytes, qf[qi]);
-#pragma unroll
-            for (int d = 0; d < DC; ++d) qf[qi][d] *= qscale;
-        }
-        m[qi] = kNegBig;
-        lsum[qi] = 0.f;
-#pragma unroll
-        for (int d = 0; d < DC; ++d) acc[qi][d] = 0.f;
-    }
-
-    for (int s2 = 0; s2 < dm.V; ++s2) {
-        const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;
-        __syncthreads();                                       // the previous view's readers are done
-        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, 0);
-        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
-        __syncthreads();
-        if constexpr (PAIR) {
-#pragma unroll
-            for (int qr = 0; qr + 1 < QW; qr += 2) {
-                if (!have[qr]) continue;                       // wave-uniform; rows are consecutive
-                stage_pair_descriptors<S, D>(desc_w, desc_e, crow[qr] + (size_t)s2 * dm.P,
-                                             crow[qr + 1] + (size_t)s2 * dm.P, dm.P, lane, s_w, s_e);
-                fwd_plane_chunk<S, D, DC, PCNT>(lbase, s_w, s_e, 0, dm.P, slot, qf[qr], qp[qr], qscale,
-                                                m[qr], lsum[qr], acc[qr]);
-                if (have[qr + 1])
-                    fwd_plane_chunk<S, D, DC, PCNT>(lbase, s_w, s_e, 32, dm.P, slot, qf[qr + 1], qp[qr + 1],
-                                                    qscale, m[qr + 1], lsum[qr + 1], acc[qr + 1]);
-            }
-        } else {
-#pragma unroll
-            for (int qi = 0; qi < QW; ++qi) {
-                if (!have[qi]) continue;
-                const size_t cq = crow[qi] + (size_t)s2 * dm.P;
-                for (int c0 = 0; c0 < dm.P; c0 += kWave) {
-                    stage_row_descriptors<S, D>(desc_w, desc_e, cq, dm.P, c0, lane, s_w, s_e);
-                    fwd_plane_chunk<S, D, DC, 0>(lbase, s_w, s_e, 0, min(kWave, dm.P - c0), slot, qf[qi],
-                                                 qp[qi], qscale, m[qi], lsum[qi], acc[qi]);
-                }
-            }
-        }
-    }
-
-#pragma unroll
-    for (int qi = 0; qi < QW; ++qi) {
-        if (!have[qi]) continue;
-        float mm = m[qi], ll = lsum[qi];
-#pragma unroll
-        for (int off = G; off < kWave; off <<= 1) {
-            const float mo = __shfl_xor(mm, off, kWave);
-            const float lo = __shfl_xor(ll, off, kWave);
-            const float mn = fmaxf(mm, mo);
-            const float a = __builtin_amdgcn_exp2f(mm - mn), bsc = __builtin_amdgcn_exp2f(mo - mn);
-            ll = ll * a + lo * bsc;
-#pragma unroll
-            for (int d = 0; d < DC; ++d) {
-                const float ao = __shfl_xor(acc[qi][d], off, kWave);
-                acc[qi][d] = acc[qi][d] * a + ao * bsc;
-            }
-            mm = mn;
-        }
-        if (slot == 0) {
-            const float inv = 1.0f / ll;
-#pragma unroll
-            for (int d = 0; d < DC; ++d) acc[qi][d] *= inv;
-            store_chunk<S, DC>((char *)out_ + (row[qi] * D + lane_elem) * S::kBytes, acc[qi]);
-            if (g == 0) lse_[row[qi]] = mm + __log2f(ll);
-        }
-    }
-}
-
-// ------------------------------------------------------------------ backward: dq and delta
-template <typename S, int D, int DC, int CNT>
-__device__ __forceinline__ void dq_plane_chunk(uint32_t lbase, const float4 *s_w, const int2 *s_e,
-                                               int dbase, int cnt_rt, int slot, float qscale,
-                                               const float (&qf)[DC], const float (&dof)[DC], const uint32_t *dop,
-                                               float lse, float delta, float (&dqa)[DC])
-{
-    constexpr int G = D / DC, NS = kWave / G;
-    constexpr int kRow = D * S::kBytes;
-    constexpr bool kPacked = S::kBytes == 2;
-    const int cnt = CNT > 0 ? CNT : cnt_rt;
-    for (int j0 = 0; j0 < cnt; j0 += NS) {
-        const int j = j0 + slot;
-        const float4 w = s_w[dbase + j];
-        const int2 e = s_e[dbase + j];
-        const uint32_t at = e.x + lbase, ab = e.y + lbase;
-        const unsigned char *top = lds_at(at), *bot = lds_at(ab);                      // K left taps; V right taps at +2*ROW
-        const unsigned char *topx = lds_at(at ^ kRow), *botx = lds_at(ab ^ kRow);      // V left taps; K right taps at +2*ROW
-        float kk[DC];
-        float dot = 0.f, dp = 0.f;
-        {
-            float t0[DC], t1[DC], t2[DC], t3[DC];
-            load_chunk<S, DC>(top, t0);
-            load_chunk<S, DC>(topx + 2 * kRow, t1);
-            load_chunk<S, DC>(bot, t2);
-            load_chunk<S, DC>(botx + 2 * kRow, t3);
-#pragma unroll
-            for (int d = 0; d < DC; ++d) {
-                kk[d] = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
-                dot = fmaf(qf[d], kk[d], dot);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);     // keep the V taps out of the K taps' live range (register budget)
-        if constexpr (kPacked) {
-            uint32_t dd[DC / 2];
-#pragma unroll
-            for (int i = 0; i < DC / 2; ++i) dd[i] = dop[i];
-            dp = tap_dot16<S, DC>(topx, top + 2 * kRow, botx, bot + 2 * kRow, w, dd);
-        } else {
-            float u0[DC], u1[DC], u2[DC], u3[DC];
-            load_chunk<S, DC>(topx, u0);
-            load_chunk<S, DC>(top + 2 * kRow, u1);
-            load_chunk<S, DC>(botx, u2);
-            load_chunk<S, DC>(bot + 2 * kRow, u3);
-#pragma unroll
-            for (int d = 0; d < DC; ++d) {
-                const float vv = fmaf(w.x, u0[d], fmaf(w.y, u1[d], fmaf(w.z, u2[d], w.w * u3[d])));
-                dp = fmaf(dof[d], vv, dp);
-            }
-        }
-        dot = group_sum<G>(dot);
-        dp = group_sum<G>(dp);
-        const float p = (j < cnt) ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
-        const float ds = p * (dp - delta);
-#pragma unroll
-        for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
-    }
-}
-
-template <typename S, int D, int DC, int QW, bool PAIR, int PCNT>
-__global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_plane_kernel(
-    const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
-    const float4 *__restrict__ desc_w, const uint32_t *__restrict__ desc_e, const void *__restrict__ out_,
-    const float *__restrict__ lse_, const void *__restrict__ dout_, void *__restrict__ dq_,
-    float *__restrict__ delta_, Dims dm)
-{
-    constexpr int G = D / DC;
-    static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
-    extern __shared__ __attribute__((aligned(kPlaneLdsAlign))) unsigned char smem[];
-    const int img_bytes = plane_lds_bytes<S, D>(dm.L);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
-    float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
-    int2 *s_e = reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
-
-    const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * QW);
-    const int nq = dm.V * dm.L;
-    const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
-    const float qscale = dm.sm_scale * kLog2e;
-    const uint32_t lbase = lds_offset(smem) + lane_byte;
-
-    zero_plane_pads<S, D>(smem, dm.L);
-
-    constexpr bool kPacked = S::kBytes == 2;
-    float qf[QW][DC], dof[QW][DC], dqa[QW][DC], lse[QW], delta[QW];
-    uint32_t dop[QW][kPacked ? DC / 2 : 1];      // 16-bit storage: dout as packed pairs for the dp dot products
-    size_t row[QW], crow[QW];
-    bool have[QW];
-#pragma unroll
-    for (int qi = 0; qi < QW; ++qi) {
-        const int qidx = pb.qbase + wave * QW + qi;
-        have[qi] = qidx < nq;
-        const int qc = have[qi] ? qidx : nq - 1;
-        const int s1 = qc / dm.L, l = qc % dm.L;
-        row[qi] = (((size_t)pb.b * dm.V + s1) * dm.H + pb.h) * dm.L + l;
-        crow[qi] = (((size_t)pb.b * dm.V + s1) * dm.L + l) * (size_t)dm.N;
-        const size_t roff = (row[qi] * D + lane_elem) * S::kBytes;
-        float of[DC];
-        load_chunk<S, DC>((const char *)q_ + roff, qf[qi]);
-        load_chunk<S, DC>((const char *)dout_ + roff, dof[qi]);
-        if constexpr (kPacked) load_packed<S, DC>((const char *)dout_ + roff, dop[qi]);
-        load_chunk<S, DC>((const char *)out_ + roff, of);
-        float dl = 0.f;
-#pragma unroll
-        for (int d = 0; d < DC; ++d) { dl = fmaf(dof[qi][d], of[d], dl); dqa[qi][d] = 0.f; }
-        delta[qi] = group_sum<G>(dl);          // the reference's _bwd_preprocess, fused
-        lse[qi] = lse_[row[qi]];
-        if (have[qi] && lane == 0) delta_[row[qi]] = delta[qi];
-    }
-
-    for (int s2 = 0; s2 < dm.V; ++s2) {
-        const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;
-        __syncthreads();
-        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, 0);
-        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
-        __syncthreads();
-        if constexpr (PAIR) {
-#pragma unroll
-            for (int qp = 0; qp + 1 < QW; qp += 2) {
-                if (!have[qp]) continue;
-                stage_pair_descriptors<S, D>(desc_w, desc_e, crow[qp] + (size_t)s2 * dm.P,
-                                             crow[qp + 1] + (size_t)s2 * dm.P, dm.P, lane, s_w, s_e);
-                dq_plane_chunk<S, D, DC, PCNT>(lbase, s_w, s_e, 0, dm.P, slot, qscale, qf[qp], dof[qp],
-                                               dop[qp], lse[qp], delta[qp], dqa[qp]);
-                if (have[qp + 1])
-                    dq_plane_chunk<S, D, DC, PCNT>(lbase, s_w, s_e, 32, dm.P, slot, qscale, qf[qp + 1],
-                                                   dof[qp + 1], dop[qp + 1], lse[qp + 1], delta[qp + 1], dqa[qp + 1]);
-            }
-        } else {
-#pragma unroll
-            for (int qi = 0; qi < QW; ++qi) {
-                if (!have[qi]) continue;
-                const size_t cq = crow[qi] + (size_t)s2 * dm.P;
-                for (int c0 = 0; c0 < dm.P; c0 += kWave) {
-                    stage_row_descriptors<S, D>(desc_w, desc_e, cq, dm.P, c0, lane, s_w, s_e);
-                    dq_plane_chunk<S, D, DC, 0>(lbase, s_w, s_e, 0, min(kWave, dm.P - c0), slot, qscale,
-                                                qf[qi], dof[qi], dop[qi], lse[qi], delta[qi], dqa[qi]);
-                }
-            }
-        }
-    }
-
-#pragma unroll
-    for (int qi = 0; qi < QW; ++qi) {
-        if (!have[qi]) continue;
-#pragma unroll
-        for (int off = G; off < kWave; off <<= 1) {
-#pragma unroll
-            for (int d = 0; d < DC; ++d) dqa[qi][d] += __shfl_xor(dqa[qi][d], off, kWave);
-        }
-        if (slot == 0) {
-#pragma unroll
-            for (int d = 0; d < DC; ++d) dqa[qi][d] *= dm.sm_scale;
-            store_chunk<S, DC>((char *)dq_ + (row[qi] * D + lane_elem) * S::kBytes, dqa[qi]);
-        }
-    }
-}
-
-// ====================================================================== one query row per slot
-// The same staged planes and tap table, with the rows dealt differently: slot s of a wave (its G
-// lanes) owns query row s of the wave's NS = 64/G rows for the whole kernel, and in every trip the NS
-// slots consume one sample each -- of NS different rows. A lane then carries the state of ONE row (q,
-// accumulator, running max and sum: ~10 registers instead of ~40 for four rows), there is nothing to
-// merge across slots at the end, every trip is full whatever P is (the kernels above leave slots idle
-// when P is not a multiple of NS), and a workgroup covers 16*NS rows, so each staged plane serves
-// twice as many rows.
+// ------------------------------------------------------------------ one query row per slot
+// Slot s of a wave (its G lanes) owns query row s of the wave's NS = 64/G rows for the whole kernel, and in
+// every trip the NS slots consume one sample each -- of NS different rows. A lane carries the state of
+// ONE row (q, accumulator, running max and sum: about 10 registers), nothing is merged across slots at
+// the end, and every trip is full whatever P is. (An earlier layout gave a wave 16/DC rows and spread
+// the samples of one row over the slots: four rows of state per lane, idle slots when P is not a
+// multiple of NS, half as many rows per staged plane; 8 % slower forward at P = 32, more at small P.)
 //
 // Per key view and pass, lane (slot, g) fetches the table entry of sample c0+g of its own row: G samples
 // per row and pass, parked sample-major (entry of trip t and slot s at t*NS + s, so the NS slots of a
@@ -623,7 +236,12 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
             stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g, slot, G, NS, s_w,
                                          s_e);
             const int cnt = min(G, dm.P - c0);
+            // up to 8 trips per pass the descriptors stay in registers from the K pass to the V pass (a lane
+            // holds one row: there is room); with 16 they are read again
+            constexpr bool kKeep = G <= 8;
             float sv[G];
+            float4 wt[kKeep ? G : 1];
+            uint32_t att[kKeep ? G : 1], abt[kKeep ? G : 1];
             float mc = kNegBig;
 #pragma unroll
             for (int t = 0; t < G; ++t) {
@@ -632,6 +250,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
                     const float4 w = s_w[t * NS + slot];
                     const int2 e = s_e[t * NS + slot];
                     const uint32_t at = e.x + lbase, ab = e.y + lbase;
+                    if constexpr (kKeep) { wt[t] = w; att[t] = at; abt[t] = ab; }
                     const unsigned char *top = lds_at(at), *bot = lds_at(ab);
                     const unsigned char *topr = lds_at((at ^ kRow) + 2 * kRow), *botr = lds_at((ab ^ kRow) + 2 * kRow);
                     float dot = 0.f;
@@ -664,9 +283,15 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
                 if (t < cnt) {
                     const float p = __builtin_amdgcn_exp2f(sv[t] - m_new);
                     lsum += p;
-                    const float4 w = s_w[t * NS + slot];
-                    const int2 e = s_e[t * NS + slot];
-                    const uint32_t at = e.x + lbase, ab = e.y + lbase;
+                    float4 w;
+                    uint32_t at, ab;
+                    if constexpr (kKeep) {
+                        w = wt[t]; at = att[t]; ab = abt[t];
+                    } else {
+                        w = s_w[t * NS + slot];
+                        const int2 e = s_e[t * NS + slot];
+                        at = e.x + lbase; ab = e.y + lbase;
+                    }
                     float t0[DC], t1[DC], t2[DC], t3[DC];
                     load_chunk<S, DC>(lds_at(at ^ kRow), t0);                  // V, left taps
                     load_chunk<S, DC>(lds_at(at + 2 * kRow), t1);              // V, right taps
