@@ -68,7 +68,7 @@ inline int check_launch()
 // The plane kernels (forward, dq) keep one K and one V plane of a (b, s2, h) in LDS next to their
 // per-wave descriptors; they serve every shape for which that fits in the 160 KB of a gfx950 workgroup.
 constexpr size_t kLdsBytes = 160 * 1024;
-constexpr size_t kPlaneDescLdsBytes = 16 * 64 * (16 + 8);   // 16 waves x 64 samples x (4 weights + 2 offsets)
+constexpr size_t kPlaneDescLdsBytes = 16 * 96 * (16 + 8);   // 16 waves x 96 places x (4 weights + 2 offsets)
 inline bool plane_path_fits(size_t L, size_t D, size_t esize)
 {
     return (L + 2) * 2 * D * esize + kPlaneDescLdsBytes <= kLdsBytes;

@@ -44,7 +44,10 @@ using lds_bytes = __attribute__((address_space(3))) const unsigned char *;
 __device__ __forceinline__ uint32_t lds_offset(const void *p) { return (uint32_t)(size_t)(lds_bytes)p; }
 __device__ __forceinline__ const unsigned char *lds_at(uint32_t off) { return (const unsigned char *)(lds_bytes)(size_t)off; }
 constexpr int kPlaneLdsAlign = 2048;   // 2*ROW for the widest row (D = 256, fp32)
-constexpr int kPlaneDescBytes = kPlaneWaves * kWave * (16 + 8);   // float4 weights + int2 base offsets
+// per wave: NS rows x (G + 1) descriptor places (one pad place per row, see stage_slot_descriptors);
+// NS*(G+1) = 64 + NS <= 96 for every lane split
+constexpr int kPlaneDescPlaces = 96;
+constexpr int kPlaneDescBytes = kPlaneWaves * kPlaneDescPlaces * (16 + 8);   // float4 weights + int2 base offsets
 
 template <typename S, int D>
 __host__ __device__ constexpr int plane_lds_bytes(int L) { return (L + 2) * 2 * D * S::kBytes; }
@@ -159,13 +162,15 @@ static __global__ __launch_bounds__(kDescThreads) void plane_descriptor_kernel(
 // multiple of NS, half as many rows per staged plane; 8 % slower forward at P = 32, more at small P.)
 //
 // Per key view and pass, lane (slot, g) fetches the table entry of sample c0+g of its own row: G samples
-// per row and pass, parked sample-major (entry of trip t and slot s at t*NS + s, so the NS slots of a
-// trip read one contiguous stretch). Odd slots swap the two samples of every pair of trips: with the
-// table's alternating bank-half order, neighbouring slots then gather from opposite halves in every trip.
+// per row and pass, parked at place slot*(G+1) + trip. The pad place per row keeps both sides free of
+// bank conflicts: the lanes of a slot write G consecutive places, and the NS slots of a trip read places
+// (G+1)*16 bytes apart, which fall in different 16-byte bank groups. Odd slots swap the two samples of
+// every pair of trips: with the table's alternating bank-half order, neighbouring slots then gather from
+// opposite halves of the bank line in every trip.
 template <typename S, int D>
 __device__ __forceinline__ void stage_slot_descriptors(const float4 *__restrict__ desc_w,
                                                        const uint32_t *__restrict__ desc_e, size_t d_row, int P,
-                                                       int c0, int g, int slot, int G_, int NS_, float4 *s_w,
+                                                       int c0, int g, int slot, int G_, float4 *s_w,
                                                        int2 *s_e)
 {
     constexpr int kRow = D * S::kBytes;
@@ -178,8 +183,8 @@ __device__ __forceinline__ void stage_slot_descriptors(const float4 *__restrict_
     const int cnt = min(G_, P - c0);                       // samples of this pass (same for every row)
     const int trip = (cnt & 1) == 0 ? g ^ (slot & 1) : g;    // pair swap only when no pair straddles the end
     wave_lds_sync();
-    s_w[trip * NS_ + slot] = w;
-    s_e[trip * NS_ + slot] = make_int2((int)(c & 0xffffu) * kRow, (int)(c >> 16) * kRow);
+    s_w[slot * (G_ + 1) + trip] = w;
+    s_e[slot * (G_ + 1) + trip] = make_int2((int)(c & 0xffffu) * kRow, (int)(c >> 16) * kRow);
     wave_lds_sync();
 }
 
@@ -196,8 +201,9 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
     extern __shared__ __attribute__((aligned(kPlaneLdsAlign))) unsigned char smem[];
     const int img_bytes = plane_lds_bytes<S, D>(dm.L);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
-    int2 *s_e = reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
+    float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kPlaneDescPlaces;
+    int2 *s_e =
+        reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kPlaneDescPlaces * 16) + wave * kPlaneDescPlaces;
 
     const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * NS);
     const int nq = dm.V * dm.L;
@@ -233,7 +239,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
         stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
         __syncthreads();
         for (int c0 = 0; c0 < dm.P; c0 += G) {
-            stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g, slot, G, NS, s_w,
+            stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g, slot, G, s_w,
                                          s_e);
             const int cnt = min(G, dm.P - c0);
             // up to 8 trips per pass the descriptors stay in registers from the K pass to the V pass (a lane
@@ -247,8 +253,8 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
             for (int t = 0; t < G; ++t) {
                 sv[t] = kNegBig;
                 if (t < cnt) {
-                    const float4 w = s_w[t * NS + slot];
-                    const int2 e = s_e[t * NS + slot];
+                    const float4 w = s_w[slot * (G + 1) + t];
+                    const int2 e = s_e[slot * (G + 1) + t];
                     const uint32_t at = e.x + lbase, ab = e.y + lbase;
                     if constexpr (kKeep) { wt[t] = w; att[t] = at; abt[t] = ab; }
                     const unsigned char *top = lds_at(at), *bot = lds_at(ab);
@@ -288,8 +294,8 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
                     if constexpr (kKeep) {
                         w = wt[t]; at = att[t]; ab = abt[t];
                     } else {
-                        w = s_w[t * NS + slot];
-                        const int2 e = s_e[t * NS + slot];
+                        w = s_w[slot * (G + 1) + t];
+                        const int2 e = s_e[slot * (G + 1) + t];
                         at = e.x + lbase; ab = e.y + lbase;
                     }
                     float t0[DC], t1[DC], t2[DC], t3[DC];
@@ -329,8 +335,9 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
     extern __shared__ __attribute__((aligned(kPlaneLdsAlign))) unsigned char smem[];
     const int img_bytes = plane_lds_bytes<S, D>(dm.L);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kWave;
-    int2 *s_e = reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kWave * 16) + wave * kWave;
+    float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kPlaneDescPlaces;
+    int2 *s_e =
+        reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kPlaneDescPlaces * 16) + wave * kPlaneDescPlaces;
 
     const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * NS);
     const int nq = dm.V * dm.L;
@@ -371,12 +378,12 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
         stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
         __syncthreads();
         for (int c0 = 0; c0 < dm.P; c0 += G) {
-            stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g, slot, G, NS, s_w,
+            stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g, slot, G, s_w,
                                          s_e);
             const int cnt = min(G, dm.P - c0);
             for (int t = 0; t < cnt; ++t) {
-                const float4 w = s_w[t * NS + slot];
-                const int2 e = s_e[t * NS + slot];
+                const float4 w = s_w[slot * (G + 1) + t];
+                const int2 e = s_e[slot * (G + 1) + t];
                 const uint32_t at = e.x + lbase, ab = e.y + lbase;
                 const unsigned char *top = lds_at(at), *bot = lds_at(ab);                      // K left; V right at +2*ROW
                 const unsigned char *topx = lds_at(at ^ kRow), *botx = lds_at(ab ^ kRow);      // V left; K right at +2*ROW

@@ -43,7 +43,7 @@ def test_workspace_bytes():
     def table(B, V, Himg, Wimg, D, P, storage16):
         """per-coordinate table of the staged kernels: only when one K and one V plane fit in LDS"""
         L, e = Himg * Wimg, 2 if storage16 else 4
-        if (L + 2) * 2 * D * e + 16 * 64 * 24 > 160 * 1024:
+        if (L + 2) * 2 * D * e + 16 * 96 * 24 > 160 * 1024:
             return 0
         m = B * V * L * V * P
         return r256(m * 16) + r256(m * 4)
