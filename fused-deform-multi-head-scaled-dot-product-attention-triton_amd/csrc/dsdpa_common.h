@@ -285,6 +285,24 @@ __device__ __forceinline__ TapGrads make_tap_grads(float cx, float cy, int Wimg,
     return t;
 }
 
+// ------------------------------------------------------------------ clearing buffers
+// Up to four 16-byte aligned float buffers cleared by all threads of a launch (sizes in floats; unused
+// slots have size 0).
+struct ZeroJob { float *p[4]; size_t n[4]; };
+
+__device__ __forceinline__ void zero_buffers(const ZeroJob &job)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const size_t n4 = job.n[k] / 4;
+        float4 *p4 = reinterpret_cast<float4 *>(job.p[k]);
+        for (size_t i = first; i < n4; i += stride) p4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (size_t i = 4 * n4 + first; i < job.n[k]; i += stride) job.p[k][i] = 0.f;
+    }
+}
+
 // ------------------------------------------------------------------ wave-level helpers
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float x)

@@ -13,20 +13,7 @@ namespace dsdpa {
 static_assert(kPlaneDescLdsBytes == (size_t)kPlaneDescBytes, "host and device agree on the descriptor block");
 
 // ------------------------------------------------------------------ small kernels
-// Zero up to four 16-byte aligned float buffers in one launch (sizes in floats; unused slots have size 0).
-struct ZeroJob { float *p[4]; size_t n[4]; };
-static __global__ void fill_zero_kernel(ZeroJob job)
-{
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        const size_t n4 = job.n[k] / 4;
-        float4 *p4 = reinterpret_cast<float4 *>(job.p[k]);
-        for (size_t i = first; i < n4; i += stride) p4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (size_t i = 4 * n4 + first; i < job.n[k]; i += stride) job.p[k][i] = 0.f;
-    }
-}
+static __global__ void fill_zero_kernel(ZeroJob job) { zero_buffers(job); }
 
 // fp32 accumulators -> 16-bit storage, 8 elements per thread
 template <typename S>
@@ -182,8 +169,9 @@ bool plane_fits(const Dims &dm, int D)
 }
 
 // Fill the descriptor table of the plane kernels (one thread per coordinate pair, padded to whole waves).
+// `zero`: buffers the same launch clears on the side (the backward's accumulators and counters).
 static inline int launch_plane_descriptors(const float *coords, const Dims &dm, char *table, const DescLayout &dl,
-                                           int timer_slot, hipStream_t st)
+                                           const ZeroJob &zero, int timer_slot, hipStream_t st)
 {
     const long long nblk = (long long)dm.B * dm.V * dm.L * dm.V;
     const long long waves = dm.P <= 32 ? (nblk + 1) / 2 : nblk * ((dm.P + 63) / 64);
@@ -192,7 +180,7 @@ static inline int launch_plane_descriptors(const float *coords, const Dims &dm, 
     ScopedKernelTimer timer(timer_slot, st);
     hipExtLaunchKernelGGL(plane_descriptor_kernel, dim3((unsigned)blocks), dim3(kDescThreads), 0, st,
                           timer.start(), timer.stop(), 0, coords, dm,
-                       (float4 *)(table + dl.w), (uint32_t *)(table + dl.e));
+                       (float4 *)(table + dl.w), (uint32_t *)(table + dl.e), zero);
     return check_launch();
 }
 
@@ -247,7 +235,7 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
     if (dl.bytes && !workspace) return DSDPA_ERR_NULL_POINTER;
     const bool staged = g_path.load() != DSDPA_PATH_GATHER && dl.bytes != 0;
     char *ws = (char *)workspace;
-    if (staged && (rc = launch_plane_descriptors(coords, dm, ws, dl, 4, st)) != DSDPA_OK) return rc;
+    if (staged && (rc = launch_plane_descriptors(coords, dm, ws, dl, ZeroJob{}, 4, st)) != DSDPA_OK) return rc;
     const float4 *desc_w = (const float4 *)(ws + dl.w);
     const uint32_t *desc_e = (const uint32_t *)(ws + dl.e);
 #define DSDPA_FWD_CASE(DD)                                                                        \
@@ -265,10 +253,8 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
     return DSDPA_ERR_HEAD_DIM;
 }
 
-static inline int zero_fill(float *a, size_t na, float *b, size_t nb, float *c, size_t nc, float *d, size_t nd,
-                            hipStream_t st)
+static inline int zero_fill(const ZeroJob &job, hipStream_t st)
 {
-    ZeroJob job{{a, b, c, d}, {na, nb, nc, d ? nd : 0}};
     size_t big = 0;
     for (int i = 0; i < 4; ++i) big = job.n[i] / 4 > big ? job.n[i] / 4 : big;
     const int threads = 256;
@@ -418,10 +404,12 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     // one launch zeroes the dk/dv accumulators and, for the cell-binned path, the cell counters
     float *dk_acc = S::kBytes == 4 ? (float *)dk : (float *)(ws + wl.acc);
     float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
-    rc = zero_fill(dk_acc, n, dv_acc, n, (float *)(ws + wl.counters), cell_binned ? wl.counters_bytes / 4 : 0,
-                   dcoords, (size_t)dm.B * dm.V * dm.L * dm.N * 2, st);
+    const ZeroJob zero{{dk_acc, dv_acc, (float *)(ws + wl.counters), dcoords},
+                       {n, n, cell_binned ? wl.counters_bytes / 4 : 0,
+                        dcoords ? (size_t)dm.B * dm.V * dm.L * dm.N * 2 : 0}};
+    // the tap-table launch, when there is one, clears them on the side; else a launch of its own
+    rc = staged ? launch_plane_descriptors(coords, dm, ws + wl.desc, wl.dl, zero, 4, st) : zero_fill(zero, st);
     if (rc != DSDPA_OK) return rc;
-    if (staged && (rc = launch_plane_descriptors(coords, dm, ws + wl.desc, wl.dl, 4, st)) != DSDPA_OK) return rc;
     if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
     if (deterministic && (rc = launch_list_ordering(dm, wl, ws, st)) != DSDPA_OK) return rc;
 #define DSDPA_BWD_CASE(DD)                                                                                      \

@@ -120,8 +120,10 @@ __device__ __forceinline__ PlaneBlock decode_plane_block(const Dims &dm, int row
 constexpr int kDescThreads = 256;
 
 static __global__ __launch_bounds__(kDescThreads) void plane_descriptor_kernel(
-    const float *__restrict__ coords_, Dims dm, float4 *__restrict__ desc_w, uint32_t *__restrict__ desc_e)
+    const float *__restrict__ coords_, Dims dm, float4 *__restrict__ desc_w, uint32_t *__restrict__ desc_e,
+    ZeroJob zero)
 {
+    zero_buffers(zero);        // the backward's accumulators and counters ride along (empty in the forward)
     const int lane = threadIdx.x & 63;
     const long long wave = ((long long)blockIdx.x * kDescThreads + threadIdx.x) >> 6;
     const long long nblk = (long long)dm.B * dm.V * dm.L * dm.V;        // (b, s1, l, s2) runs of P samples
