@@ -68,7 +68,7 @@ size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int W
     if (dtype != DSDPA_F32 && dtype != DSDPA_BF16 && dtype != DSDPA_F16) return 0;
     if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || D < 1 || P < 1) return 0;
     return workspace_layout(B, V, H, Himg, Wimg, D, P, dtype != DSDPA_F32,
-                            (flags & DSDPA_FLAG_DETERMINISTIC) != 0).total;
+                            (flags & DSDPA_FLAG_DETERMINISTIC) != 0, (flags & DSDPA_FLAG_COORDS_GRAD) != 0).total;
 }
 
 const char *dsdpa_error_string(int code)

@@ -69,24 +69,28 @@ inline int check_launch()
 // per-wave descriptors; they serve every shape for which that fits in the 160 KB of a gfx950 workgroup.
 constexpr size_t kLdsBytes = 160 * 1024;
 constexpr size_t kPlaneDescLdsBytes = 16 * 96 * (16 + 8);   // 16 waves x 96 places x (4 weights + 2 offsets)
-inline bool plane_path_fits(size_t L, size_t D, size_t esize)
+constexpr size_t kPlaneGradLdsBytes = 16 * 96 * 8;         // + fx, fy per place (coordinate gradient)
+inline bool plane_path_fits(size_t L, size_t D, size_t esize, bool coords_grad = false)
 {
-    return (L + 2) * 2 * D * esize + kPlaneDescLdsBytes <= kLdsBytes;
+    return (L + 2) * 2 * D * esize + kPlaneDescLdsBytes + (coords_grad ? kPlaneGradLdsBytes : 0) <= kLdsBytes;
 }
 
 // Descriptor table of the plane kernels: per coordinate pair 16 bytes of weights and 4 of packed slot
-// codes, computed once per call by plane_descriptor_kernel. Empty when the plane kernels do not apply.
-struct DescLayout { size_t w, e, bytes; };
+// codes (plus, for the coordinate gradient, 16 bytes of derivative weights), computed once per call by
+// plane_descriptor_kernel. Empty when the plane kernels do not apply.
+struct DescLayout { size_t w, e, g, bytes; };
 inline size_t round256(size_t b) { return (b + 255) / 256 * 256; }
-inline DescLayout desc_layout(size_t B, size_t V, size_t Himg, size_t Wimg, size_t D, size_t P, size_t esize)
+inline DescLayout desc_layout(size_t B, size_t V, size_t Himg, size_t Wimg, size_t D, size_t P, size_t esize,
+                              bool coords_grad = false)
 {
-    DescLayout d{0, 0, 0};
+    DescLayout d{0, 0, 0, 0};
     const size_t L = Himg * Wimg;
-    if (!plane_path_fits(L, D, esize)) return d;
+    if (!plane_path_fits(L, D, esize, coords_grad)) return d;
     const size_t m = B * V * L * V * P;
     d.w = 0;
     d.e = round256(m * 16);
-    d.bytes = d.e + round256(m * 4);
+    d.g = d.e + round256(m * 4);
+    d.bytes = d.g + (coords_grad ? round256(m * 16) : 0);
     return d;
 }
 
@@ -97,7 +101,8 @@ inline DescLayout desc_layout(size_t B, size_t V, size_t Himg, size_t Wimg, size
 //   start    B*V*(NC+1) u32                  exclusive scan of the counts
 //   sorted   B*V*(V*L*P) u32                 sample ids ordered by cell
 //   acc      2*n floats                      fp32 dk/dv accumulators (16-bit storage only)
-//   desc     20 bytes per coordinate pair    descriptor table (only when the plane kernels apply)
+//   desc     20 bytes per coordinate pair    descriptor table (only when the plane kernels apply); 36 with
+//                                            the coordinate gradient
 // deterministic backward only (DSDPA_FLAG_DETERMINISTIC):
 //   sorted2  as sorted                       the lists with every cell's ids in ascending order
 //   seg      2*B*V*NC u32                    begin / end of every list in the flat id array
@@ -115,7 +120,7 @@ struct WorkspaceLayout {
     int NC;
 };
 inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Himg, size_t Wimg, size_t D, size_t P,
-                                        bool storage16, bool deterministic)
+                                        bool storage16, bool deterministic, bool coords_grad)
 {
     WorkspaceLayout w;
     const size_t rows = B * V * H * Himg * Wimg;
@@ -126,7 +131,9 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     w.start = off; off += round256(B * V * ((size_t)w.NC + 1) * 4);
     w.sorted = off; off += round256(B * V * (V * Himg * Wimg * P) * 4);
     w.acc = off; if (storage16) off += round256(2 * rows * D * 4);
-    w.dl = desc_layout(B, V, Himg, Wimg, D, P, storage16 ? 2 : 4);
+    // with the coordinate gradient the staged dq kernel needs more LDS; where it no longer fits, dq takes the
+    // gather kernel and no table is needed
+    w.dl = desc_layout(B, V, Himg, Wimg, D, P, storage16 ? 2 : 4, coords_grad);
     w.desc = off; off += w.dl.bytes;
     w.sorted2 = w.seg = w.sorttmp = off;
     w.sorttmp_bytes = 0;

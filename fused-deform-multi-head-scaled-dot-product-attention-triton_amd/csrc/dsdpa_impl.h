@@ -10,7 +10,8 @@
 
 namespace dsdpa {
 
-static_assert(kPlaneDescLdsBytes == (size_t)kPlaneDescBytes, "host and device agree on the descriptor block");
+static_assert(kPlaneDescLdsBytes == (size_t)kPlaneDescBytes && kPlaneGradLdsBytes == (size_t)kPlaneGradBytes,
+              "host and device agree on the descriptor block");
 
 // ------------------------------------------------------------------ small kernels
 static __global__ void fill_zero_kernel(ZeroJob job) { zero_buffers(job); }
@@ -171,7 +172,7 @@ bool plane_fits(const Dims &dm, int D)
 // Fill the descriptor table of the plane kernels (one thread per coordinate pair, padded to whole waves).
 // `zero`: buffers the same launch clears on the side (the backward's accumulators and counters).
 static inline int launch_plane_descriptors(const float *coords, const Dims &dm, char *table, const DescLayout &dl,
-                                           const ZeroJob &zero, int timer_slot, hipStream_t st)
+                                           bool coords_grad, const ZeroJob &zero, int timer_slot, hipStream_t st)
 {
     const long long nblk = (long long)dm.B * dm.V * dm.L * dm.V;
     const long long waves = dm.P <= 32 ? (nblk + 1) / 2 : nblk * ((dm.P + 63) / 64);
@@ -180,7 +181,8 @@ static inline int launch_plane_descriptors(const float *coords, const Dims &dm, 
     ScopedKernelTimer timer(timer_slot, st);
     hipExtLaunchKernelGGL(plane_descriptor_kernel, dim3((unsigned)blocks), dim3(kDescThreads), 0, st,
                           timer.start(), timer.stop(), 0, coords, dm,
-                       (float4 *)(table + dl.w), (uint32_t *)(table + dl.e), zero);
+                       (float4 *)(table + dl.w), (uint32_t *)(table + dl.e),
+                       coords_grad ? (float4 *)(table + dl.g) : (float4 *)nullptr, zero);
     return check_launch();
 }
 
@@ -205,20 +207,21 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float4 *
 template <typename S, int D>
 int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float4 *desc_w,
                         const uint32_t *desc_e, const void *out,
-                        const float *lse, const void *dout, void *dq, float *delta, const Dims &dm,
-                        hipStream_t st)
+                        const float *lse, const void *dout, void *dq, float *delta, const float4 *desc_g,
+                        float *dcoords, const Dims &dm, hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
-    const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes;
+    const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes + (dcoords ? kPlaneGradBytes : 0);
     const int rows_per_block = kPlaneWaves * (kWave / (D / DC));
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
-    auto kern = bwd_dq_slot_kernel<S, D, DC>;
+    auto kern = dcoords ? bwd_dq_slot_kernel<S, D, DC, true> : bwd_dq_slot_kernel<S, D, DC, false>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(2, st);
     hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
-                          timer.start(), timer.stop(), 0, q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, dm);
+                          timer.start(), timer.stop(), 0, q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, desc_g,
+                          dcoords, dm);
     return check_launch();
 }
 
@@ -235,7 +238,7 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
     if (dl.bytes && !workspace) return DSDPA_ERR_NULL_POINTER;
     const bool staged = g_path.load() != DSDPA_PATH_GATHER && dl.bytes != 0;
     char *ws = (char *)workspace;
-    if (staged && (rc = launch_plane_descriptors(coords, dm, ws, dl, ZeroJob{}, 4, st)) != DSDPA_OK) return rc;
+    if (staged && (rc = launch_plane_descriptors(coords, dm, ws, dl, false, ZeroJob{}, 4, st)) != DSDPA_OK) return rc;
     const float4 *desc_w = (const float4 *)(ws + dl.w);
     const uint32_t *desc_e = (const uint32_t *)(ws + dl.e);
 #define DSDPA_FWD_CASE(DD)                                                                        \
@@ -380,7 +383,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
 {
     if (!q || !k || !v || !coords || !out || !lse || !dout || !dq || !dk || !dv || !workspace)
         return DSDPA_ERR_NULL_POINTER;
-    if (flags & ~(unsigned)DSDPA_FLAG_DETERMINISTIC) return DSDPA_ERR_UNSUPPORTED;
+    if (flags & ~(unsigned)(DSDPA_FLAG_DETERMINISTIC | DSDPA_FLAG_COORDS_GRAD)) return DSDPA_ERR_UNSUPPORTED;
     const bool deterministic = (flags & DSDPA_FLAG_DETERMINISTIC) != 0;
     if (deterministic && dcoords) return DSDPA_ERR_UNSUPPORTED;   // dcoords sums over heads with float atomics
     Dims dm;
@@ -389,16 +392,19 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     if ((long long)dm.L * dm.N > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;   // sample ids are 32-bit
     hipStream_t st = (hipStream_t)stream;
     const size_t n = (size_t)dm.rows * D;
-    const WorkspaceLayout wl = workspace_layout(B, V, H, Himg, Wimg, D, P, S::kBytes != 4, deterministic);
+    // the staged dq kernel computes dcoords only when the caller sized the workspace for it (same flags)
+    const bool cg_table = dcoords && (flags & DSDPA_FLAG_COORDS_GRAD) != 0;
+    const WorkspaceLayout wl = workspace_layout(B, V, H, Himg, Wimg, D, P, S::kBytes != 4, deterministic, cg_table);
     char *ws = (char *)workspace;
     float *delta = (float *)(ws + wl.delta);
     const int path = deterministic ? (int)DSDPA_PATH_AUTO : g_path.load();   // only the cell-binned path has a fixed order
     const bool fused_atomics = path == DSDPA_PATH_GATHER;
     const bool cell_binned = path == DSDPA_PATH_AUTO;
-    // the coordinate gradient lives in the gather dq kernel only: dq leaves the staged kernels when it is asked for
-    const bool staged = !fused_atomics && wl.dl.bytes != 0 && !dcoords;
+    // (with the coordinate gradient the layout holds a table only where the larger LDS block still fits)
+    const bool staged = !fused_atomics && wl.dl.bytes != 0 && (!dcoords || cg_table);
     const float4 *desc_w = (const float4 *)(ws + wl.desc + wl.dl.w);
     const uint32_t *desc_e = (const uint32_t *)(ws + wl.desc + wl.dl.e);
+    const float4 *desc_g = (const float4 *)(ws + wl.desc + wl.dl.g);
     const unsigned *start = (const unsigned *)(ws + wl.start);
     const unsigned *sorted = (const unsigned *)(ws + (deterministic ? wl.sorted2 : wl.sorted));
     // one launch zeroes the dk/dv accumulators and, for the cell-binned path, the cell counters
@@ -408,7 +414,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
                        {n, n, cell_binned ? wl.counters_bytes / 4 : 0,
                         dcoords ? (size_t)dm.B * dm.V * dm.L * dm.N * 2 : 0}};
     // the tap-table launch, when there is one, clears them on the side; else a launch of its own
-    rc = staged ? launch_plane_descriptors(coords, dm, ws + wl.desc, wl.dl, zero, 4, st) : zero_fill(zero, st);
+    rc = staged ? launch_plane_descriptors(coords, dm, ws + wl.desc, wl.dl, cg_table, zero, 4, st) : zero_fill(zero, st);
     if (rc != DSDPA_OK) return rc;
     if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
     if (deterministic && (rc = launch_list_ordering(dm, wl, ws, st)) != DSDPA_OK) return rc;
@@ -417,7 +423,8 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
         if (fused_atomics && !dcoords) {                                                                        \
             rc = launch_bwd_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st);         \
         } else {                                                                                                \
-            rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, dm, st) \
+            rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, desc_g, \
+                                                     dcoords, dm, st)                                           \
                         : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm,  \
                                                       st);                                                      \
             if (rc == DSDPA_OK && cell_binned)                                                                  \

@@ -48,6 +48,7 @@ constexpr int kPlaneLdsAlign = 2048;   // 2*ROW for the widest row (D = 256, fp3
 // NS*(G+1) = 64 + NS <= 96 for every lane split
 constexpr int kPlaneDescPlaces = 96;
 constexpr int kPlaneDescBytes = kPlaneWaves * kPlaneDescPlaces * (16 + 8);   // float4 weights + int2 base offsets
+constexpr int kPlaneGradBytes = kPlaneWaves * kPlaneDescPlaces * 8;         // fx, fy per place (coordinate-gradient kernel)
 
 template <typename S, int D>
 __host__ __device__ constexpr int plane_lds_bytes(int L) { return (L + 2) * 2 * D * S::kBytes; }
@@ -115,13 +116,18 @@ __device__ __forceinline__ PlaneBlock decode_plane_block(const Dims &dm, int row
 // call -- one thread per coordinate pair, same order (b, s1, l, s2, p) as the coordinates -- and the
 // plane kernels of all H heads read them back: 16 bytes of weights and the two K slot codes
 // 2*q + (q & 1) (byte offset / ROW, so the table does not depend on the head width or storage type)
-// packed into one 32-bit word. Within every run of up to 64 samples of one (b, s1, l, s2) the entries
-// are stored in paired_position order.
+// packed into one 32-bit word (13 bits each: a plane that fits in LDS has fewer than 2200 slots). Within
+// every run of up to 64 samples of one (b, s1, l, s2) the entries are stored in paired_position order.
+// For the coordinate gradient (desc_g not null) the word also carries which taps lie inside the image
+// -- bits 13, 14: columns x0, x0+1; bits 29, 30: rows y0, y0+1 -- and desc_g holds (fx, fy, the sample's
+// index n inside its run as an integer, unused): the entries are stored in a permuted order, and the
+// gradient has to go back to the sample it belongs to.
 constexpr int kDescThreads = 256;
+constexpr uint32_t kDescCodeMask = 0x1fffu;
 
 static __global__ __launch_bounds__(kDescThreads) void plane_descriptor_kernel(
     const float *__restrict__ coords_, Dims dm, float4 *__restrict__ desc_w, uint32_t *__restrict__ desc_e,
-    ZeroJob zero)
+    float4 *__restrict__ desc_g, ZeroJob zero)
 {
     zero_buffers(zero);        // the backward's accumulators and counters ride along (empty in the forward)
     const int lane = threadIdx.x & 63;
@@ -151,7 +157,20 @@ static __global__ __launch_bounds__(kDescThreads) void plane_descriptor_kernel(
     if (valid) {
         const long long dst = blk * dm.P + pos;
         desc_w[dst] = make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]);
-        desc_e[dst] = (uint32_t)(2 * qt + (qt & 1)) | ((uint32_t)(2 * qb + (qb & 1)) << 16);
+        uint32_t word = (uint32_t)(2 * qt + (qt & 1)) | ((uint32_t)(2 * qb + (qb & 1)) << 16);
+        if (desc_g) {
+            // same arithmetic as make_taps, so that fx, fy and the inside tests agree with the weights
+            const float x = ((xy.x * 2.0f - 1.0f) + 1.0f) * ((float)(dm.Wimg - 1) * 0.5f);
+            const float y = ((xy.y * 2.0f - 1.0f) + 1.0f) * ((float)(dm.Himg - 1) * 0.5f);
+            const float fx = x - floorf(x), fy = y - floorf(y);
+            const bool fin = (x == x) && (y == y);
+            const int x0 = tp.x0, y0 = tp.y0;
+            const bool vx0 = fin && x0 >= 0 && x0 < dm.Wimg, vx1 = fin && x0 + 1 >= 0 && x0 + 1 < dm.Wimg;
+            const bool vy0 = fin && y0 >= 0 && y0 < dm.Himg, vy1 = fin && y0 + 1 >= 0 && y0 + 1 < dm.Himg;
+            word |= (vx0 ? 1u << 13 : 0u) | (vx1 ? 1u << 14 : 0u) | (vy0 ? 1u << 29 : 0u) | (vy1 ? 1u << 30 : 0u);
+            desc_g[dst] = make_float4(fin ? fx : 0.f, fin ? fy : 0.f, __int_as_float(n), 0.f);
+        }
+        desc_e[dst] = word;
     }
 }
 
@@ -169,11 +188,15 @@ static __global__ __launch_bounds__(kDescThreads) void plane_descriptor_kernel(
 // (G+1)*16 bytes apart, which fall in different 16-byte bank groups. Odd slots swap the two samples of
 // every pair of trips: with the table's alternating bank-half order, neighbouring slots then gather from
 // opposite halves of the bank line in every trip.
+// s_g (coordinate gradient only): fx, fy of the sample; the four inside bits then ride in the low bits
+// of the parked top address (ROW >= 32 bytes leaves them free): bit 0, 1: columns x0, x0+1; bit 2, 3: rows.
+// Returns the index inside its run of the sample this lane fetched (coordinate gradient only, else 0).
 template <typename S, int D>
-__device__ __forceinline__ void stage_slot_descriptors(const float4 *__restrict__ desc_w,
-                                                       const uint32_t *__restrict__ desc_e, size_t d_row, int P,
-                                                       int c0, int g, int slot, int G_, float4 *s_w,
-                                                       int2 *s_e)
+__device__ __forceinline__ int stage_slot_descriptors(const float4 *__restrict__ desc_w,
+                                                      const uint32_t *__restrict__ desc_e, size_t d_row, int P,
+                                                      int c0, int g, int slot, int G_, float4 *s_w,
+                                                      int2 *s_e, const float4 *__restrict__ desc_g = nullptr,
+                                                      float2 *s_g = nullptr)
 {
     constexpr int kRow = D * S::kBytes;
     const int n = c0 + g;
@@ -184,10 +207,19 @@ __device__ __forceinline__ void stage_slot_descriptors(const float4 *__restrict_
     if (!valid) w = make_float4(0.f, 0.f, 0.f, 0.f);
     const int cnt = min(G_, P - c0);                       // samples of this pass (same for every row)
     const int trip = (cnt & 1) == 0 ? g ^ (slot & 1) : g;    // pair swap only when no pair straddles the end
+    int ex = (int)(c & kDescCodeMask) * kRow;
+    const int ey = (int)((c >> 16) & kDescCodeMask) * kRow;
+    float4 gw = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (desc_g) {
+        gw = desc_g[i];
+        ex |= (int)(((c >> 13) & 3u) | (((c >> 29) & 3u) << 2));
+    }
     wave_lds_sync();
     s_w[slot * (G_ + 1) + trip] = w;
-    s_e[slot * (G_ + 1) + trip] = make_int2((int)(c & 0xffffu) * kRow, (int)(c >> 16) * kRow);
+    s_e[slot * (G_ + 1) + trip] = make_int2(ex, ey);
+    if (desc_g) s_g[slot * (G_ + 1) + trip] = make_float2(gw.x, gw.y);
     wave_lds_sync();
+    return __float_as_int(gw.z);
 }
 
 template <typename S, int D, int DC>
@@ -323,16 +355,21 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
     }
 }
 
-template <typename S, int D, int DC>
+// CG: also the gradient of the coordinates (see bwd_dq_gather_kernel for the formula): per-tap dot
+// products instead of blend-then-dot, the four per-tap terms masked by the inside bits, combined with
+// fx, fy from the table and reduced over the slot. The lane that fetched a sample's table entry keeps
+// the sample's result, and after the pass every lane adds its own sample's pair to dcoords (zeroed before
+// the launch) with float atomics -- one wave-wide pair of atomics per pass, not one per trip.
+template <typename S, int D, int DC, bool CG>
 __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float4 *__restrict__ desc_w, const uint32_t *__restrict__ desc_e, const void *__restrict__ out_,
     const float *__restrict__ lse_, const void *__restrict__ dout_, void *__restrict__ dq_,
-    float *__restrict__ delta_, Dims dm)
+    float *__restrict__ delta_, const float4 *__restrict__ desc_g, float *__restrict__ dcoords_, Dims dm)
 {
     constexpr int G = D / DC, NS = kWave / G;
     constexpr int kRow = D * S::kBytes;
-    constexpr bool kPacked = S::kBytes == 2;
+    constexpr bool kPacked = S::kBytes == 2 && !CG;
     static_assert(G >= 2 && G <= 16 && G * DC == D, "lane split");
     extern __shared__ __attribute__((aligned(kPlaneLdsAlign))) unsigned char smem[];
     const int img_bytes = plane_lds_bytes<S, D>(dm.L);
@@ -340,6 +377,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
     float4 *s_w = reinterpret_cast<float4 *>(smem + img_bytes) + wave * kPlaneDescPlaces;
     int2 *s_e =
         reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kPlaneDescPlaces * 16) + wave * kPlaneDescPlaces;
+    float2 *s_g = reinterpret_cast<float2 *>(smem + img_bytes + kPlaneDescBytes) + wave * kPlaneDescPlaces;   // CG only
 
     const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * NS);
     const int nq = dm.V * dm.L;
@@ -380,12 +418,64 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
         stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
         __syncthreads();
         for (int c0 = 0; c0 < dm.P; c0 += G) {
-            stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g, slot, G, s_w,
-                                         s_e);
+            const int my_n = stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g,
+                                                          slot, G, s_w, s_e, CG ? desc_g : nullptr, s_g);
             const int cnt = min(G, dm.P - c0);
+            const int my_trip = (cnt & 1) == 0 ? g ^ (slot & 1) : g;     // where this lane's sample was parked
+            float my_gx = 0.f, my_gy = 0.f;
             for (int t = 0; t < cnt; ++t) {
                 const float4 w = s_w[slot * (G + 1) + t];
                 const int2 e = s_e[slot * (G + 1) + t];
+                if constexpr (CG) {
+                    const uint32_t inside = (uint32_t)e.x & 15u;
+                    const uint32_t at = (uint32_t)e.x - inside + lbase, ab = e.y + lbase;
+                    const unsigned char *kp[4] = { lds_at(at), lds_at((at ^ kRow) + 2 * kRow), lds_at(ab),
+                                                   lds_at((ab ^ kRow) + 2 * kRow) };
+                    const unsigned char *vp[4] = { lds_at(at ^ kRow), lds_at(at + 2 * kRow), lds_at(ab ^ kRow),
+                                                   lds_at(ab + 2 * kRow) };
+                    const float wt[4] = { w.x, w.y, w.z, w.w };
+                    float kk[DC], dk_t[4], dv_t[4];
+                    float dot = 0.f, dp = 0.f;
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) kk[d] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float tk[DC], tv[DC];
+                        load_chunk<S, DC>(kp[i], tk);
+                        load_chunk<S, DC>(vp[i], tv);
+                        dk_t[i] = 0.f;
+                        dv_t[i] = 0.f;
+#pragma unroll
+                        for (int d = 0; d < DC; ++d) {
+                            dk_t[i] = fmaf(qf[d], tk[d], dk_t[i]);
+                            dv_t[i] = fmaf(dof[d], tv[d], dv_t[i]);
+                            kk[d] = fmaf(wt[i], tk[d], kk[d]);
+                        }
+                        dot = fmaf(wt[i], dk_t[i], dot);
+                        dp = fmaf(wt[i], dv_t[i], dp);
+                    }
+                    dot = group_sum<G>(dot);
+                    dp = group_sum<G>(dp);
+                    const float p = __builtin_amdgcn_exp2f(dot * qscale - lse);
+                    const float ds = p * (dp - delta);
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
+                    // per-tap terms, zero for taps outside the image; taps 00, 01, 10, 11 = (row, column)
+                    const float a = ds * dm.sm_scale;
+                    const bool c0in = inside & 1u, c1in = inside & 2u, r0in = inside & 4u, r1in = inside & 8u;
+                    const float g0 = (c0in && r0in) ? fmaf(a, dk_t[0], p * dv_t[0]) : 0.f;
+                    const float g1 = (c1in && r0in) ? fmaf(a, dk_t[1], p * dv_t[1]) : 0.f;
+                    const float g2 = (c0in && r1in) ? fmaf(a, dk_t[2], p * dv_t[2]) : 0.f;
+                    const float g3 = (c1in && r1in) ? fmaf(a, dk_t[3], p * dv_t[3]) : 0.f;
+                    const float2 gf = s_g[slot * (G + 1) + t];              // fx, fy
+                    const float dx0 = g1 - g0, dy0 = g2 - g0;
+                    float gx = fmaf(gf.y, (g3 - g2) - dx0, dx0) * (float)(dm.Wimg - 1);
+                    float gy = fmaf(gf.x, (g3 - g1) - dy0, dy0) * (float)(dm.Himg - 1);
+                    gx = group_sum<G>(gx);
+                    gy = group_sum<G>(gy);
+                    if (t == my_trip) { my_gx = gx; my_gy = gy; }
+                    continue;
+                }
                 const uint32_t at = e.x + lbase, ab = e.y + lbase;
                 const unsigned char *top = lds_at(at), *bot = lds_at(ab);                      // K left; V right at +2*ROW
                 const unsigned char *topx = lds_at(at ^ kRow), *botx = lds_at(ab ^ kRow);      // V left; K right at +2*ROW
@@ -423,6 +513,11 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
                 const float ds = p * (dp - delta);
 #pragma unroll
                 for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
+            }
+            if (CG && have && c0 + g < dm.P) {
+                float *dst = dcoords_ + 2 * (crow + (size_t)s2 * dm.P + (size_t)my_n);
+                atomicAdd(dst, my_gx);
+                atomicAdd(dst + 1, my_gy);
             }
         }
     }

@@ -114,6 +114,8 @@ class _fused_deform_sdpa(torch.autograd.Function):
         if flags and dcoords is not None:
             raise RuntimeError("deform_sdpa_triton: the coordinate gradient has no deterministic implementation "
                                "(it sums over heads with float atomics); turn one of the two off")
+        if dcoords is not None:
+            flags |= _native.FLAG_COORDS_GRAD
         ws_bytes = lib.dsdpa_bwd_workspace_bytes(_DTYPE_CODE[q.dtype], B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P, flags)
         ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
         with torch.cuda.device(q.device):

@@ -85,7 +85,11 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
  * added up in ascending order of their index and the per-cell sums reach dk/dv in four passes of plain
  * stores (cells of one row/column parity share no pixel) instead of float atomics. Needs a larger
  * workspace (pass the same flags to dsdpa_bwd_workspace_bytes) and cannot be combined with dcoords. */
-enum { DSDPA_FLAG_DETERMINISTIC = 1 };
+enum { DSDPA_FLAG_DETERMINISTIC = 1, DSDPA_FLAG_COORDS_GRAD = 2 };
+/* DSDPA_FLAG_COORDS_GRAD: the workspace has room for the coordinate gradient's part of the per-coordinate
+ * table (16 more bytes per coordinate pair where the staged kernels run), so that a backward given dcoords
+ * stays on the staged dq kernel. Pass the same flags to dsdpa_bwd_workspace_bytes and to dsdpa_bwd_*;
+ * dcoords without the bit is computed by the slower gather dq kernel, the bit without dcoords does nothing. */
 
 /*
  * Backward: replaces everything `_fused_deform_sdpa.backward` enqueues,
@@ -97,8 +101,8 @@ enum { DSDPA_FLAG_DETERMINISTIC = 1 };
  * `dcoords` may be NULL (the reference's behaviour: no gradient for coords, ops/triton.py:464). When it
  * is given (fp32, shaped like coords) it receives the gradient of the normalised coordinates summed over
  * the heads -- what the reference's eager operator gets by differentiating through grid_sample,
- * ops/torch.py:14-15 -- and is fully overwritten too; the backward then takes the gather dq kernel for
- * every shape (float atomics across heads: not deterministic either).
+ * ops/torch.py:14-15 -- and is fully overwritten too (float atomics across heads: not deterministic
+ * either); see DSDPA_FLAG_COORDS_GRAD.
  * `workspace` must hold dsdpa_bwd_workspace_bytes(...) bytes (256-byte aligned):
  * the per-row delta = dout.out (one float per query row, the reference's `delta`,
  * ops/triton.py:430), the per-(batch, key view) ordering of the samples by

@@ -68,6 +68,13 @@ def test_workspace_bytes():
     plain = lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32, 0)
     det = lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32, _native.FLAG_DETERMINISTIC)
     assert det >= plain + r256(2 * 6 * 6 * 324 * 32 * 4) + r256(2 * 2 * 6 * 361 * 4)
+    # coordinate gradient: 16 more bytes per coordinate pair where the planes and the larger descriptor block fit
+    cg = lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32, _native.FLAG_COORDS_GRAD)
+    assert cg == plain + r256(2 * 6 * 324 * 6 * 32 * 16)
+    # 21x22 fp32 D32: 118784 plane bytes + 36864 fit, + 12288 more do not: no table at all with the flag
+    fits = lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 1, 2, 1, 21, 22, 32, 4, 0)
+    nofit = lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 1, 2, 1, 21, 22, 32, 4, _native.FLAG_COORDS_GRAD)
+    assert fits == expect(1, 2, 1, 21, 22, 32, 4, False) and nofit == fits - table(1, 2, 21, 22, 32, 4, False)
 
 
 def test_argument_validation_before_launch():

@@ -41,6 +41,7 @@ CASES = [
     (35, 2, 2, 1, 4, 7, 128, 40, 0.0, 1.0),
     (36, 1, 2, 1, 3, 3, 256, 9, -0.1, 1.1),
     (37, 1, 3, 2, 1, 11, 32, 5, -0.2, 1.2),      # single-row image: no y gradient
+    (38, 1, 2, 1, 21, 22, 32, 4, -0.1, 1.1),     # fp32: the planes fit in LDS only without the gradient's block
 ]
 
 
@@ -117,3 +118,33 @@ def test_coords_gradient_named_workloads(name):
         far = (x < -1) | (x > wl.W_IMG) | (y < -1) | (y > wl.H_IMG)
         assert far.any()
         assert (cg.grad.cpu()[far] == 0).all()
+
+
+def test_dcoords_without_the_workspace_flag_matches_with_it():
+    """C ABI: dcoords given but DSDPA_FLAG_COORDS_GRAD not set (workspace sized without it): the gather dq kernel
+    computes the gradient; with the flag the staged kernel does. Same numbers to float-atomic noise."""
+    say("[case] coords grad through the C ABI, with and without the workspace flag")
+    lib = _native.load()
+    g = torch.Generator().manual_seed(41)
+    B, V, H, Himg, Wimg, D, P = 1, 3, 2, 6, 7, 32, 11
+    L = Himg * Wimg
+    q, k, v, do = (torch.randn(B, V, H, L, D, generator=g).cuda() for _ in range(4))
+    c = (torch.rand(B, V, L, V, P, 2, generator=g) * 1.2 - 0.1).cuda()
+    out, lse = torch.empty_like(q), torch.empty(B, V, H, L, device="cuda")
+    fws = torch.empty(max(lib.dsdpa_fwd_workspace_bytes(0, B, V, H, Himg, Wimg, D, P), 1), dtype=torch.uint8,
+                      device="cuda")
+    _native.check(lib.dsdpa_fwd_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out.data_ptr(),
+                                    lse.data_ptr(), fws.data_ptr(), B, V, H, Himg, Wimg, D, P, 0.3, None))
+    res = {}
+    for flags in (0, _native.FLAG_COORDS_GRAD):
+        nbytes = lib.dsdpa_bwd_workspace_bytes(0, B, V, H, Himg, Wimg, D, P, flags)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        dq, dk, dv, dc = (torch.full_like(t, float("nan")) for t in (q, k, v, c))
+        _native.check(lib.dsdpa_bwd_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out.data_ptr(),
+                                        lse.data_ptr(), do.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                        dc.data_ptr(), ws.data_ptr(), B, V, H, Himg, Wimg, D, P, 0.3, flags, None))
+        torch.cuda.synchronize()
+        res[flags] = (nbytes, dq.cpu(), dc.cpu())
+    assert res[_native.FLAG_COORDS_GRAD][0] > res[0][0]
+    assert rel(res[0][1], res[_native.FLAG_COORDS_GRAD][1].numpy()) < 1e-5
+    assert rel(res[0][2], res[_native.FLAG_COORDS_GRAD][2].numpy()) < 1e-5
