@@ -108,6 +108,25 @@ def measure_gpu(wl, steps, warmup):
         torch.cuda.synchronize()
         fwd_only_ms = (time.perf_counter() - t0) * 1e3 / steps
 
+    # the three main kernels one after the other on one stream (in the timed region above the backward's
+    # dq and dk/dv kernels share the GPU, which stretches both)
+    import ops.triton as op_module
+    op_module.SINGLE_STREAM = True
+    try:
+        step()
+        torch.cuda.synchronize()
+        _native.timer_enable(True)
+        for _ in range(5):
+            step()
+        torch.cuda.synchronize()
+        _native.timer_enable(False)
+    finally:
+        op_module.SINGLE_STREAM = False
+    alone = {}
+    for which, name in enumerate(("fwd", "bwd_dkdv", "bwd_dq", "bwd_bin", "desc_table")):
+        ms, n = _native.timer_collect(which)
+        alone[name] = ms / max(n, 1)
+
     torch.cuda.reset_peak_memory_stats()
     base = torch.cuda.memory_allocated()
     step()
@@ -117,6 +136,7 @@ def measure_gpu(wl, steps, warmup):
         "ms_per_step": ms_step,
         "fwd_only_ms": fwd_only_ms,
         "kernels": kern,
+        "kernels_single_stream_ms": alone,
         "peak_extra_bytes": int(peak_extra),
     }
 
@@ -155,8 +175,8 @@ def measure_cpu(wl, budget_s=25.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="C2")
     ap.add_argument("--all", action="store_true", help="also report the other workloads on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -210,6 +230,11 @@ def main():
         "bound": "hbm", "kernel": dominant, "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": dom["frac"], "traffic": load_traffic(wl.name, dominant),
         "algorithmic_bytes": dom["algorithmic_bytes"], "kernel_ms": dom["kernel_ms"],
+        # the same kernel with the GPU to itself (backward on one stream): it shares the CUs with the dq kernel
+        # in the timed region
+        "kernel_ms_one_stream": g["kernels_single_stream_ms"][dominant],
+        "frac_one_stream": dom["algorithmic_bytes"] / (g["kernels_single_stream_ms"][dominant] * 1e-3) / 1e9
+                           / HBM_PEAK_GBS if g["kernels_single_stream_ms"][dominant] > 0 else None,
     }
     # per step: every timed item once, except the table fill (once in the forward, once in the backward)
     kernels_ms = sum(v["ms"] * v["per_step"] for v in g["kernels"].values())
@@ -261,6 +286,7 @@ def main():
                    "query_samples_per_step": qs,
                    "fwd_only_ms": g["fwd_only_ms"],
                    "kernel_ms": {k: round(v["ms"], 5) for k, v in g["kernels"].items()},
+                   "kernel_ms_one_stream": {k: round(v, 5) for k, v in g["kernels_single_stream_ms"].items()},
                    "fwd_bwd_frac_of_hbm_roofline_on_step_time": details["fwd_bwd_frac_of_roofline_on_step_time"],
                    "peak_extra_bytes": g["peak_extra_bytes"]},
         "roofline": roofline,

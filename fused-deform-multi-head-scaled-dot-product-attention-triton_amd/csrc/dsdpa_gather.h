@@ -352,7 +352,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
 #pragma unroll
     for (int d = 0; d < DC; ++d) delta = fmaf(dof[d], of[d], delta);
     delta = group_sum<G>(delta);
-    if (lane == 0) delta_[rc.row] = delta;
+    if (delta_ && lane == 0) delta_[rc.row] = delta;         // null: a launch of its own computes it
     const float qscale = dm.sm_scale * kLog2e;
     const float lse = lse_[rc.row];
 

@@ -55,6 +55,36 @@ struct ScopedKernelTimer {
     }
 };
 
+// Side lane of the backward: a second stream, per host thread and device, on which the cell binning runs
+// next to the dq kernel (neither needs the other; dk/dv needs both). Fork and join are events on the
+// caller's stream, so the caller sees one stream's worth of ordering. Created on first use, default
+// priority, never destroyed (a handful of handles per thread that ever ran a backward).
+struct SideLane {
+    hipStream_t stream = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+    bool failed = false;
+};
+inline SideLane *side_lane()
+{
+    constexpr int kMaxDevices = 64;
+    thread_local SideLane lanes[kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    SideLane &s = lanes[dev];
+    if (s.failed) return nullptr;
+    if (!s.stream) {
+        if (hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) != hipSuccess ||
+            hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&s.join, hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            s.failed = true;
+            s.stream = nullptr;
+            return nullptr;
+        }
+    }
+    return &s;
+}
+
 inline int check_launch()
 {
     hipError_t e = hipGetLastError();

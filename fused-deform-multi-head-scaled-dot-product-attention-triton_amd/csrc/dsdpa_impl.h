@@ -16,6 +16,15 @@ static_assert(kPlaneDescLdsBytes == (size_t)kPlaneDescBytes && kPlaneGradLdsByte
 // ------------------------------------------------------------------ small kernels
 static __global__ void fill_zero_kernel(ZeroJob job) { zero_buffers(job); }
 
+// A launch that may carry the kernel timer's events. Without them it is a plain launch: only those are
+// known to be recorded by a stream capture.
+#define DSDPA_LAUNCH(kern, grid, block, smem, st, ev0, ev1, ...)                                             \
+    do {                                                                                                     \
+        hipEvent_t ev0_ = (ev0), ev1_ = (ev1);                                                               \
+        if (ev0_ || ev1_) hipExtLaunchKernelGGL(kern, grid, block, smem, st, ev0_, ev1_, 0, __VA_ARGS__);    \
+        else hipLaunchKernelGGL(kern, grid, block, smem, st, __VA_ARGS__);                                   \
+    } while (0)
+
 // fp32 accumulators -> 16-bit storage, 8 elements per thread
 template <typename S>
 __global__ void cast_kernel(const float *__restrict__ src, void *__restrict__ dst, size_t n8)
@@ -30,6 +39,29 @@ __global__ void cast_kernel(const float *__restrict__ src, void *__restrict__ ds
         v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
         store_chunk<S, 8>((char *)dst + i * 16, v);
     }
+}
+
+// delta[row] = dout[row] . out[row] (the reference's _bwd_preprocess, ops/triton.py:197-215) as a launch of
+// its own, for when the dk/dv kernel does not run behind the dq kernel (which computes it on the way).
+// Four lanes per row, four elements per lane and step.
+template <typename S>
+__global__ __launch_bounds__(256) void delta_kernel(const void *__restrict__ out_, const void *__restrict__ dout_,
+                                                    float *__restrict__ delta_, size_t rows, int D)
+{
+    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t row = t >> 2;
+    const int j = (int)(t & 3);
+    const size_t r = row < rows ? row : rows - 1;
+    float acc = 0.f;
+    for (int e = j * 4; e < D; e += 16) {
+        float a[4], b[4];
+        load_chunk<S, 4>((const char *)out_ + (r * D + e) * S::kBytes, a);
+        load_chunk<S, 4>((const char *)dout_ + (r * D + e) * S::kBytes, b);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) acc = fmaf(a[d], b[d], acc);
+    }
+    acc = group_sum<4>(acc);
+    if (row < rows && j == 0) delta_[row] = acc;
 }
 
 static inline int make_dims(int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, Dims *dm)
@@ -63,8 +95,8 @@ int launch_fwd_gather(const void *q, const void *k, const void *v, const float *
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(0, st);
-    hipExtLaunchKernelGGL((fwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
-                          timer.start(), timer.stop(), 0,
+    DSDPA_LAUNCH((fwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                          timer.start(), timer.stop(),
                        q, k, v, coords, out, lse, dm);
     return check_launch();
 }
@@ -77,8 +109,8 @@ int launch_bwd_gather(const void *q, const void *k, const void *v, const float *
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(1, st);
-    hipExtLaunchKernelGGL((bwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
-                          timer.start(), timer.stop(), 0,
+    DSDPA_LAUNCH((bwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                          timer.start(), timer.stop(),
                        q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm);
     return check_launch();
 }
@@ -92,12 +124,12 @@ int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const floa
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(2, st);
     if (dcoords)
-        hipExtLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
-                              timer.start(), timer.stop(), 0,
+        DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                              timer.start(), timer.stop(),
                            q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm);
     else
-        hipExtLaunchKernelGGL((bwd_dq_gather_kernel<S, D, DC, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
-                              timer.start(), timer.stop(), 0,
+        DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                              timer.start(), timer.stop(),
                            q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm);
     return check_launch();
 }
@@ -157,8 +189,8 @@ int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const floa
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(1, st);
-    hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kTileWaves * kWave), smem, st,
-                          timer.start(), timer.stop(), 0,
+    DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(kTileWaves * kWave), smem, st,
+                          timer.start(), timer.stop(),
                        q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, tg);
     return check_launch();
 }
@@ -179,8 +211,8 @@ static inline int launch_plane_descriptors(const float *coords, const Dims &dm, 
     const long long blocks = (waves * kWave + kDescThreads - 1) / kDescThreads;
     if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
     ScopedKernelTimer timer(timer_slot, st);
-    hipExtLaunchKernelGGL(plane_descriptor_kernel, dim3((unsigned)blocks), dim3(kDescThreads), 0, st,
-                          timer.start(), timer.stop(), 0, coords, dm,
+    DSDPA_LAUNCH(plane_descriptor_kernel, dim3((unsigned)blocks), dim3(kDescThreads), 0, st,
+                          timer.start(), timer.stop(), coords, dm,
                        (float4 *)(table + dl.w), (uint32_t *)(table + dl.e),
                        coords_grad ? (float4 *)(table + dl.g) : (float4 *)nullptr, zero);
     return check_launch();
@@ -199,8 +231,8 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float4 *
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(0, st);
-    hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
-                          timer.start(), timer.stop(), 0, q, k, v, desc_w, desc_e, out, lse, dm);
+    DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
+                          timer.start(), timer.stop(), q, k, v, desc_w, desc_e, out, lse, dm);
     return check_launch();
 }
 
@@ -219,8 +251,8 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(2, st);
-    hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
-                          timer.start(), timer.stop(), 0, q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, desc_g,
+    DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
+                          timer.start(), timer.stop(), q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, desc_g,
                           dcoords, dm);
     return check_launch();
 }
@@ -302,24 +334,24 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(k1),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * hist_bytes));
         if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
-        hipExtLaunchKernelGGL(k0, dim3((unsigned)blocks), dim3(kBinLdsThreads), hist_bytes, st,
-                              timer.start(), nullptr, 0,
+        DSDPA_LAUNCH(k0, dim3((unsigned)blocks), dim3(kBinLdsThreads), hist_bytes, st,
+                              timer.start(), nullptr,
                            coords, dm, wl.NC, lchunk, nlc, counters, sorted);
         hipLaunchKernelGGL(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st, counters, start, wl.NC);
-        hipExtLaunchKernelGGL(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
-                              nullptr, timer.stop(), 0,
+        DSDPA_LAUNCH(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
+                              nullptr, timer.stop(),
                            coords, dm, wl.NC, lchunk, nlc, counters, sorted);
         return check_launch();
     }
     const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
     const long long blocks = (total + kBinThreads - 1) / kBinThreads;
     if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
-    hipExtLaunchKernelGGL(bin_samples_kernel<0>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
-                          timer.start(), nullptr, 0,
+    DSDPA_LAUNCH(bin_samples_kernel<0>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
+                          timer.start(), nullptr,
                        coords, dm, wl.NC, counters, sorted);
     hipLaunchKernelGGL(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st, counters, start, wl.NC);
-    hipExtLaunchKernelGGL(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
-                          nullptr, timer.stop(), 0,
+    DSDPA_LAUNCH(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
+                          nullptr, timer.stop(),
                        coords, dm, wl.NC, counters, sorted);
     return check_launch();
 }
@@ -350,8 +382,8 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
         cg.div_h = FastDiv::make((unsigned)dm.H);
         const unsigned blocks = (unsigned)((nwork + kCellWaves - 1) / kCellWaves);
         const bool first = colour <= 0, last = colour < 0 || colour == 3;
-        hipExtLaunchKernelGGL((bwd_dkdv_cell_kernel<S, D, DC>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
-                              first ? timer.start() : nullptr, last ? timer.stop() : nullptr, 0, q, k, v, coords,
+        DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
+                              first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
                               lse, delta, dout, start, sorted, dk_acc, dv_acc, dm, NC, cg);
     }
     return check_launch();
@@ -383,7 +415,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
 {
     if (!q || !k || !v || !coords || !out || !lse || !dout || !dq || !dk || !dv || !workspace)
         return DSDPA_ERR_NULL_POINTER;
-    if (flags & ~(unsigned)(DSDPA_FLAG_DETERMINISTIC | DSDPA_FLAG_COORDS_GRAD)) return DSDPA_ERR_UNSUPPORTED;
+    if (flags & ~(unsigned)(DSDPA_FLAG_DETERMINISTIC | DSDPA_FLAG_COORDS_GRAD | DSDPA_FLAG_SINGLE_STREAM)) return DSDPA_ERR_UNSUPPORTED;
     const bool deterministic = (flags & DSDPA_FLAG_DETERMINISTIC) != 0;
     if (deterministic && dcoords) return DSDPA_ERR_UNSUPPORTED;   // dcoords sums over heads with float atomics
     Dims dm;
@@ -410,28 +442,59 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     // one launch zeroes the dk/dv accumulators and, for the cell-binned path, the cell counters
     float *dk_acc = S::kBytes == 4 ? (float *)dk : (float *)(ws + wl.acc);
     float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
-    const ZeroJob zero{{dk_acc, dv_acc, (float *)(ws + wl.counters), dcoords},
-                       {n, n, cell_binned ? wl.counters_bytes / 4 : 0,
-                        dcoords ? (size_t)dm.B * dm.V * dm.L * dm.N * 2 : 0}};
-    // the tap-table launch, when there is one, clears them on the side; else a launch of its own
-    rc = staged ? launch_plane_descriptors(coords, dm, ws + wl.desc, wl.dl, cg_table, zero, 4, st) : zero_fill(zero, st);
+    // The binning (and the deterministic list ordering) runs beside the table fill and the dq kernel on the
+    // side lane: forked here, before anything is enqueued, joined before the dk/dv kernel. The side lane
+    // then clears the cell counters itself.
+    hipStream_t bst = st;
+    SideLane *side = cell_binned && !(flags & DSDPA_FLAG_SINGLE_STREAM) ? side_lane() : nullptr;
+    if (side && hipEventRecord(side->fork, st) == hipSuccess &&
+        hipStreamWaitEvent(side->stream, side->fork, 0) == hipSuccess)
+        bst = side->stream;
+    const bool side_on = bst != st;
+    const size_t ncounters = cell_binned ? wl.counters_bytes / 4 : 0;
+    const size_t ndc = dcoords ? (size_t)dm.B * dm.V * dm.L * dm.N * 2 : 0;
+    // what has to start at zero: on one stream everything in one job, which the tap-table launch (when
+    // there is one) takes along; with the side lane the dk/dv side clears its own buffers there
+    const ZeroJob zero_all{{dk_acc, dv_acc, (float *)(ws + wl.counters), dcoords}, {n, n, ncounters, ndc}};
+    const ZeroJob zero_main{{dcoords, nullptr, nullptr, nullptr}, {ndc, 0, 0, 0}};
+    const ZeroJob &zero = side_on ? zero_main : zero_all;
+    if (staged) rc = launch_plane_descriptors(coords, dm, ws + wl.desc, wl.dl, cg_table, zero, 4, st);
+    else if (!side_on || ndc) rc = zero_fill(zero, st);
     if (rc != DSDPA_OK) return rc;
-    if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
-    if (deterministic && (rc = launch_list_ordering(dm, wl, ws, st)) != DSDPA_OK) return rc;
+    if (side_on) {
+        // the dk/dv side: clears, delta, binning, ordering; the dk/dv kernel follows below
+        const ZeroJob zero_side{{dk_acc, dv_acc, (float *)(ws + wl.counters), nullptr}, {n, n, ncounters, 0}};
+        if ((rc = zero_fill(zero_side, bst)) != DSDPA_OK) return rc;
+        const size_t lanes = (size_t)dm.rows * 4;
+        hipLaunchKernelGGL((delta_kernel<S>), dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, bst, out, dout, delta,
+                           (size_t)dm.rows, D);
+        if ((rc = check_launch()) != DSDPA_OK) return rc;
+    }
+    if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, bst)) != DSDPA_OK) return rc;
+    if (deterministic && (rc = launch_list_ordering(dm, wl, ws, bst)) != DSDPA_OK) return rc;
+    float *dq_delta = side_on ? nullptr : delta;        // the dq kernel writes delta only when dk/dv runs behind it
+    const auto join_side = [&]() -> int {
+        if (!side_on) return DSDPA_OK;
+        hipError_t e = hipEventRecord(side->join, bst);
+        if (e == hipSuccess) e = hipStreamWaitEvent(st, side->join, 0);
+        if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+        return DSDPA_OK;
+    };
 #define DSDPA_BWD_CASE(DD)                                                                                      \
     case DD:                                                                                                    \
         if (fused_atomics && !dcoords) {                                                                        \
             rc = launch_bwd_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st);         \
         } else {                                                                                                \
-            rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, desc_g, \
-                                                     dcoords, dm, st)                                           \
-                        : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm,  \
-                                                      st);                                                      \
+            rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, dq_delta,     \
+                                                     desc_g, dcoords, dm, st)                                   \
+                        : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dq_delta, dcoords,   \
+                                                      dm, st);                                                  \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
                 rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, lse, delta, dout, start, sorted, dk_acc,      \
-                                                 dv_acc, dm, wl.NC, deterministic, st);                         \
+                                                 dv_acc, dm, wl.NC, deterministic, bst);                        \
             else if (rc == DSDPA_OK)                                                                            \
                 rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, st);    \
+            if (rc == DSDPA_OK) rc = join_side();                                                               \
         }                                                                                                       \
         break;
     switch (D) {

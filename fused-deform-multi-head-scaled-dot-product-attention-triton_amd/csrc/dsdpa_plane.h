@@ -409,7 +409,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
         delta = group_sum<G>(dl);              // the reference's _bwd_preprocess, fused
     }
     const float lse = lse_[row];
-    if (have && g == 0) delta_[row] = delta;
+    if (delta_ && have && g == 0) delta_[row] = delta;       // null: a launch of its own computes it
 
     for (int s2 = 0; s2 < dm.V; ++s2) {
         const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;

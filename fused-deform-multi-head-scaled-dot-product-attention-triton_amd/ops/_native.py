@@ -22,6 +22,7 @@ DSDPA_F32, DSDPA_BF16, DSDPA_F16 = 0, 1, 2
 PATH_AUTO, PATH_GATHER, PATH_LDS = 0, 1, 2
 FLAG_DETERMINISTIC = 1
 FLAG_COORDS_GRAD = 2
+FLAG_SINGLE_STREAM = 4
 
 _lib = None
 

@@ -64,6 +64,11 @@ def _check_inputs(q, k, v, coords, WIDTH, HEIGHT):
     return sfx
 
 
+# The backward runs its dk/dv side beside the dq side on a second stream of the library's (forked from and joined
+# to the caller's stream inside the call). True keeps every launch on the caller's stream (same results).
+SINGLE_STREAM = False
+
+
 class _fused_deform_sdpa(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, coords, WIDTH, HEIGHT, sm_scale, *extra):
@@ -116,6 +121,8 @@ class _fused_deform_sdpa(torch.autograd.Function):
                                "(it sums over heads with float atomics); turn one of the two off")
         if dcoords is not None:
             flags |= _native.FLAG_COORDS_GRAD
+        if SINGLE_STREAM:
+            flags |= _native.FLAG_SINGLE_STREAM
         ws_bytes = lib.dsdpa_bwd_workspace_bytes(_DTYPE_CODE[q.dtype], B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P, flags)
         ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
         with torch.cuda.device(q.device):

@@ -26,11 +26,18 @@
  *     inside the kernels, and out-of-image taps follow the eager reference's
  *     per-tap zero padding (ops/torch.py:14-15), not ops/triton.py:129;
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
- *     all work is enqueued on it and the call returns without synchronising;
+ *     the call returns without synchronising, and everything it enqueues is
+ *     ordered after what `stream` held before the call and before what is
+ *     enqueued on `stream` after it (the backward forks part of its work onto a
+ *     second stream of the library's and joins it again, see
+ *     DSDPA_FLAG_SINGLE_STREAM; a capture of `stream` records both);
  *   - D (head dim) must be one of 16, 32, 64, 128, 256 (ops/triton.py:386);
  *   - every entry point returns 0 on success or a DSDPA_ERR_* code, never
  *     throws, and is re-entrant; the only process-wide state is the kernel-path
- *     selector (dsdpa_set_path) and the optional kernel timer.
+ *     selector (dsdpa_set_path) and the optional kernel timer, the only
+ *     per-thread state the backward's second stream (one stream and two events
+ *     per host thread and device, created by the first backward call there
+ *     and kept until the process ends).
  */
 #ifndef DSDPA_H
 #define DSDPA_H
@@ -85,7 +92,11 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
  * added up in ascending order of their index and the per-cell sums reach dk/dv in four passes of plain
  * stores (cells of one row/column parity share no pixel) instead of float atomics. Needs a larger
  * workspace (pass the same flags to dsdpa_bwd_workspace_bytes) and cannot be combined with dcoords. */
-enum { DSDPA_FLAG_DETERMINISTIC = 1, DSDPA_FLAG_COORDS_GRAD = 2 };
+enum { DSDPA_FLAG_DETERMINISTIC = 1, DSDPA_FLAG_COORDS_GRAD = 2, DSDPA_FLAG_SINGLE_STREAM = 4 };
+/* DSDPA_FLAG_SINGLE_STREAM: enqueue every launch of the backward on `stream` itself. By default the dk/dv side
+ * (clearing the accumulators, delta, the cell binning, the dk/dv kernel) runs on a second stream of the
+ * library's beside the tap table and the dq kernel: neither side reads what the other writes, and the two
+ * main kernels leave each other idle issue slots (C2: 7 % off the fwd+bwd step). Same results either way. */
 /* DSDPA_FLAG_COORDS_GRAD: the workspace has room for the coordinate gradient's part of the per-coordinate
  * table (16 more bytes per coordinate pair where the staged kernels run), so that a backward given dcoords
  * stays on the staged dq kernel. Pass the same flags to dsdpa_bwd_workspace_bytes and to dsdpa_bwd_*;
