@@ -42,9 +42,9 @@ def log(*a):
 # profiles/hbm_traffic_C2.md. Only the kernels of the bench workload were measured.
 MEASURED_TRAFFIC_BYTES = {
     "C2": {
-        "fwd": int((35041.6 * 2.0 + 4009.5) * 1024),
-        "bwd_dq": int((38970.7 * 2.0 + 4009.5) * 1024),
-        "bwd_dkdv": int((42884.6 * 2.0 + 110976.0) * 1024),
+        "fwd": int((35033.1 * 2.0 + 4009.5) * 1024),
+        "bwd_dq": int((38970.6 * 2.0 + 3888.0) * 1024),
+        "bwd_dkdv": int((42882.5 * 2.0 + 110976.0) * 1024),
     },
 }
 
