@@ -142,3 +142,38 @@ def test_captured_graph_replays_to_the_eager_result(dtype):
         torch.cuda.synchronize()
         assert torch.equal(s_out, e_out) and torch.equal(s_dq, e_dq), f"replay {rep}"
         assert rel(s_dk, e_dk) < tol and rel(s_dv, e_dv) < tol, f"replay {rep}"
+
+
+def test_two_host_threads_with_their_own_streams():
+    """Two host threads run forward + backward at the same time, each on a stream of its own (the library keeps
+    one second stream per thread and device); both get the single-stream result."""
+    import threading
+    say("[case] two host threads")
+    cases = [make(91, 2, 3, 2, 9, 8, 32, 12), make(92, 1, 4, 3, 7, 11, 64, 9)]
+    dims = [(9, 8), (7, 11)]
+    refs = [c_abi_backward(*cases[i], *dims[i], _native.FLAG_SINGLE_STREAM) for i in range(2)]
+    torch.cuda.synchronize()
+    results, errors = [None, None], []
+
+    def work(i):
+        try:
+            torch.cuda.set_device(0)
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                for _ in range(8):
+                    r = c_abi_backward(*cases[i], *dims[i], 0, stream=st)
+            st.synchronize()
+            results[i] = r
+        except Exception as e:                   # surfaced in the main thread below
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    for i in range(2):
+        assert results[i] is not None
+        assert torch.equal(results[i][0], refs[i][0]) and torch.equal(results[i][1], refs[i][1])
+        assert rel(results[i][2], refs[i][2]) < 1e-5 and rel(results[i][3], refs[i][3]) < 1e-5
