@@ -16,7 +16,7 @@ resident in HBM. Prints ONE JSON line on stdout:
                  (grid_sample + softmax, oracle/torch_eager.py), same run
 
 Per-workload details (forward alone, backward alone, all five shapes with --all)
-go to stderr and, as JSON, to gpurun_out/bench_details.json when that folder exists.
+go to stderr and, with --details FILE, as JSON into that file.
 """
 import argparse
 import json
@@ -180,13 +180,14 @@ def main():
     ap.add_argument("--workload", default="C2")
     ap.add_argument("--all", action="store_true", help="also report the other workloads on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--details", default=None, help="also write the per-workload details as JSON into this file")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run a plain 256 MiB device copy a few times (known HBM traffic, used to scale "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU; run with --gpus 1 "
-                 "(the operator shards over (batch, head) with no exchange, see DESIGN.md)")
+                 "(the operator shards over (batch, head) with no exchange between the shards)")
 
     from workloads import WORKLOADS, oob_fractions
     wl = WORKLOADS[args.workload]
@@ -270,9 +271,8 @@ def main():
         cpu = measure_cpu(wl)
         log("[bench] cpu baseline", json.dumps(cpu))
 
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out_dir):
-        with open(os.path.join(out_dir, "bench_details.json"), "w") as f:
+    if args.details:
+        with open(args.details, "w") as f:
             json.dump({"gpu": all_details, "cpu": cpu}, f, indent=1)
 
     line = {
