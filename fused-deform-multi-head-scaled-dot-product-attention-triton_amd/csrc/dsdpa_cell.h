@@ -199,7 +199,7 @@ struct CellGrid {
 template <typename S, int D, int DC>
 __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 3 : 2)) void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
-    const float *__restrict__ coords_, const float *__restrict__ lse_, const float *__restrict__ delta_,
+    const float *__restrict__ coords_, const float2 *__restrict__ stats_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
     float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC, CellGrid cg)
 {
@@ -280,12 +280,11 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
     // (s1*H*L + l) * ROW < V*H*L*D*e <= 2^32 (the shape limits keep one batch item of a tensor below 2^30
     // elements): one add per gather instead of 64-bit address arithmetic per lane.
     constexpr unsigned kRowBytes = D * S::kBytes;
-    constexpr int kRowToFloatShift = __builtin_ctz(kRowBytes) - 2;         // row byte offset -> float offset
+    constexpr int kRowToPairShift = __builtin_ctz(kRowBytes) - 3;          // row byte offset -> offset of the row's (lse, delta)
     const size_t bh_row0 = ((size_t)b * dm.V * dm.H + h) * dm.L;              // row of (b, s1 = 0, h, l = 0)
     const char *q_bh = (const char *)q_ + bh_row0 * kRowBytes;
     const char *do_bh = (const char *)dout_ + bh_row0 * kRowBytes;
-    const char *lse_bh = (const char *)(lse_ + bh_row0);
-    const char *delta_bh = (const char *)(delta_ + bh_row0);
+    const char *stats_bh = (const char *)(stats_ + bh_row0);                 // (lse, delta) per row
     const unsigned lane_byte = (unsigned)lane_elem * S::kBytes;
     const unsigned view_rows = (unsigned)dm.H * (unsigned)dm.L;
     const float2 *coords = reinterpret_cast<const float2 *>(coords_);
@@ -326,11 +325,12 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
         for (int j0 = 0; j0 < cnt; j0 += NS) {
             const float4 w = s_w[wave][j0 + slot];
             const unsigned r = s_row[wave][j0 + slot];
-            const unsigned roff = r + lane_byte, foff = r >> kRowToFloatShift;
+            const unsigned roff = r + lane_byte, soff = r >> kRowToPairShift;
             float qf[DC], dof[DC];
             load_chunk<S, DC>(q_bh + roff, qf);
             load_chunk<S, DC>(do_bh + roff, dof);
-            const float lse = *(const float *)(lse_bh + foff), delta = *(const float *)(delta_bh + foff);
+            const float2 ld = *(const float2 *)(stats_bh + soff);
+            const float lse = ld.x, delta = ld.y;
             __builtin_amdgcn_sched_barrier(0);     // all four gathers in flight before the arithmetic starts
             float dot = 0.f, dp = 0.f;
             if constexpr (kPacked) {

@@ -319,7 +319,7 @@ template <typename S, int D, int DC, bool CG>
 __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
-    const void *__restrict__ dout_, void *__restrict__ dq_, float *__restrict__ delta_,
+    const void *__restrict__ dout_, void *__restrict__ dq_, float2 *__restrict__ stats_,
     float *__restrict__ dcoords_, Dims dm)
 {
     constexpr int G = D / DC;
@@ -352,9 +352,9 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
 #pragma unroll
     for (int d = 0; d < DC; ++d) delta = fmaf(dof[d], of[d], delta);
     delta = group_sum<G>(delta);
-    if (delta_ && lane == 0) delta_[rc.row] = delta;         // null: a launch of its own computes it
     const float qscale = dm.sm_scale * kLog2e;
     const float lse = lse_[rc.row];
+    if (stats_ && lane == 0) stats_[rc.row] = make_float2(lse, delta);     // null: a launch of its own does it
 
     float dqa[DC];
 #pragma unroll

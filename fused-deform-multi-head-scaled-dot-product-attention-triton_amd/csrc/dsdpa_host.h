@@ -156,7 +156,7 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     const size_t rows = B * V * H * Himg * Wimg;
     w.NC = (int)((Himg + 1) * (Wimg + 1));
     size_t off = 0;
-    w.delta = off; off += round256(rows * 4);
+    w.delta = off; off += round256(rows * 8);           // (lse, delta) per row
     w.counters = off; w.counters_bytes = round256(B * V * (size_t)w.NC * 4); off += w.counters_bytes;
     w.start = off; off += round256(B * V * ((size_t)w.NC + 1) * 4);
     w.sorted = off; off += round256(B * V * (V * Himg * Wimg * P) * 4);

@@ -41,12 +41,14 @@ __global__ void cast_kernel(const float *__restrict__ src, void *__restrict__ ds
     }
 }
 
-// delta[row] = dout[row] . out[row] (the reference's _bwd_preprocess, ops/triton.py:197-215) as a launch of
+// stats[row] = (lse[row], delta[row]), delta = dout[row] . out[row] (the reference's _bwd_preprocess,
+// ops/triton.py:197-215; the pair side by side so that the dk/dv kernels fetch both with one load), as a launch of
 // its own, for when the dk/dv kernel does not run behind the dq kernel (which computes it on the way).
 // Four lanes per row, four elements per lane and step.
 template <typename S>
 __global__ __launch_bounds__(256) void delta_kernel(const void *__restrict__ out_, const void *__restrict__ dout_,
-                                                    float *__restrict__ delta_, size_t rows, int D)
+                                                    const float *__restrict__ lse_, float2 *__restrict__ stats_,
+                                                    size_t rows, int D)
 {
     const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t row = t >> 2;
@@ -61,7 +63,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const void *__restrict__ out
         for (int d = 0; d < 4; ++d) acc = fmaf(a[d], b[d], acc);
     }
     acc = group_sum<4>(acc);
-    if (row < rows && j == 0) delta_[row] = acc;
+    if (row < rows && j == 0) stats_[row] = make_float2(lse_[row], acc);
 }
 
 static inline int make_dims(int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, Dims *dm)
@@ -117,7 +119,7 @@ int launch_bwd_gather(const void *q, const void *k, const void *v, const float *
 
 template <typename S, int D>
 int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const float *coords, const void *out,
-                         const float *lse, const void *dout, void *dq, float *delta, float *dcoords,
+                         const float *lse, const void *dout, void *dq, float2 *stats, float *dcoords,
                          const Dims &dm, hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
@@ -126,11 +128,11 @@ int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const floa
     if (dcoords)
         DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
-                           q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm);
+                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, dm);
     else
         DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
-                           q, k, v, coords, out, lse, dout, dq, delta, dcoords, dm);
+                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, dm);
     return check_launch();
 }
 
@@ -174,8 +176,8 @@ static inline TileGeom make_tile_geom(const Dims &dm, int D)
 }
 
 template <typename S, int D>
-int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const float *coords, const float *lse,
-                         const float *delta, const void *dout, float *dk_acc, float *dv_acc, const Dims &dm,
+int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const float *coords,
+                         const float2 *stats, const void *dout, float *dk_acc, float *dv_acc, const Dims &dm,
                          hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
@@ -191,7 +193,7 @@ int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const floa
     ScopedKernelTimer timer(1, st);
     DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(kTileWaves * kWave), smem, st,
                           timer.start(), timer.stop(),
-                       q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, tg);
+                       q, k, v, coords, stats, dout, dk_acc, dv_acc, dm, tg);
     return check_launch();
 }
 
@@ -239,7 +241,7 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float4 *
 template <typename S, int D>
 int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float4 *desc_w,
                         const uint32_t *desc_e, const void *out,
-                        const float *lse, const void *dout, void *dq, float *delta, const float4 *desc_g,
+                        const float *lse, const void *dout, void *dq, float2 *stats, const float4 *desc_g,
                         float *dcoords, const Dims &dm, hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
@@ -252,7 +254,7 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
     if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
     ScopedKernelTimer timer(2, st);
     DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
-                          timer.start(), timer.stop(), q, k, v, desc_w, desc_e, out, lse, dout, dq, delta, desc_g,
+                          timer.start(), timer.stop(), q, k, v, desc_w, desc_e, out, lse, dout, dq, stats, desc_g,
                           dcoords, dm);
     return check_launch();
 }
@@ -358,8 +360,8 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
 
 // deterministic: four launches, one per (row parity, column parity) of the cells, each with plain stores
 template <typename S, int D>
-int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const float *coords, const float *lse,
-                         const float *delta, const void *dout, const unsigned *start, const unsigned *sorted,
+int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const float *coords,
+                         const float2 *stats, const void *dout, const unsigned *start, const unsigned *sorted,
                          float *dk_acc, float *dv_acc, const Dims &dm, int NC, bool deterministic, hipStream_t st)
 {
     constexpr int DC = CellChunk<S, D>::value;
@@ -384,7 +386,7 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
         const bool first = colour <= 0, last = colour < 0 || colour == 3;
         DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
                               first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
-                              lse, delta, dout, start, sorted, dk_acc, dv_acc, dm, NC, cg);
+                              stats, dout, start, sorted, dk_acc, dv_acc, dm, NC, cg);
     }
     return check_launch();
 }
@@ -428,7 +430,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const bool cg_table = dcoords && (flags & DSDPA_FLAG_COORDS_GRAD) != 0;
     const WorkspaceLayout wl = workspace_layout(B, V, H, Himg, Wimg, D, P, S::kBytes != 4, deterministic, cg_table);
     char *ws = (char *)workspace;
-    float *delta = (float *)(ws + wl.delta);
+    float2 *stats = (float2 *)(ws + wl.delta);          // per row: lse, delta
     const int path = deterministic ? (int)DSDPA_PATH_AUTO : g_path.load();   // only the cell-binned path has a fixed order
     const bool fused_atomics = path == DSDPA_PATH_GATHER;
     const bool cell_binned = path == DSDPA_PATH_AUTO;
@@ -466,13 +468,13 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
         const ZeroJob zero_side{{dk_acc, dv_acc, (float *)(ws + wl.counters), nullptr}, {n, n, ncounters, 0}};
         if ((rc = zero_fill(zero_side, bst)) != DSDPA_OK) return rc;
         const size_t lanes = (size_t)dm.rows * 4;
-        hipLaunchKernelGGL((delta_kernel<S>), dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, bst, out, dout, delta,
-                           (size_t)dm.rows, D);
+        hipLaunchKernelGGL((delta_kernel<S>), dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, bst, out, dout, lse,
+                           stats, (size_t)dm.rows, D);
         if ((rc = check_launch()) != DSDPA_OK) return rc;
     }
     if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, bst)) != DSDPA_OK) return rc;
     if (deterministic && (rc = launch_list_ordering(dm, wl, ws, bst)) != DSDPA_OK) return rc;
-    float *dq_delta = side_on ? nullptr : delta;        // the dq kernel writes delta only when dk/dv runs behind it
+    float2 *dq_stats = side_on ? nullptr : stats;       // the dq kernel writes them only when dk/dv runs behind it
     const auto join_side = [&]() -> int {
         if (!side_on) return DSDPA_OK;
         hipError_t e = hipEventRecord(side->join, bst);
@@ -485,15 +487,15 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
         if (fused_atomics && !dcoords) {                                                                        \
             rc = launch_bwd_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st);         \
         } else {                                                                                                \
-            rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, dq_delta,     \
+            rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, dq_stats,     \
                                                      desc_g, dcoords, dm, st)                                   \
-                        : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dq_delta, dcoords,   \
+                        : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dq_stats, dcoords,   \
                                                       dm, st);                                                  \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
-                rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, lse, delta, dout, start, sorted, dk_acc,      \
+                rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, stats, dout, start, sorted, dk_acc,           \
                                                  dv_acc, dm, wl.NC, deterministic, bst);                        \
             else if (rc == DSDPA_OK)                                                                            \
-                rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, lse, delta, dout, dk_acc, dv_acc, dm, st);    \
+                rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, stats, dout, dk_acc, dv_acc, dm, st);         \
             if (rc == DSDPA_OK) rc = join_side();                                                               \
         }                                                                                                       \
         break;

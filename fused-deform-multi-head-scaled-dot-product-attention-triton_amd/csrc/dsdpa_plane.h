@@ -365,7 +365,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float4 *__restrict__ desc_w, const uint32_t *__restrict__ desc_e, const void *__restrict__ out_,
     const float *__restrict__ lse_, const void *__restrict__ dout_, void *__restrict__ dq_,
-    float *__restrict__ delta_, const float4 *__restrict__ desc_g, float *__restrict__ dcoords_, Dims dm)
+    float2 *__restrict__ stats_, const float4 *__restrict__ desc_g, float *__restrict__ dcoords_, Dims dm)
 {
     constexpr int G = D / DC, NS = kWave / G;
     constexpr int kRow = D * S::kBytes;
@@ -409,7 +409,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
         delta = group_sum<G>(dl);              // the reference's _bwd_preprocess, fused
     }
     const float lse = lse_[row];
-    if (delta_ && have && g == 0) delta_[row] = delta;       // null: a launch of its own computes it
+    if (stats_ && have && g == 0) stats_[row] = make_float2(lse, delta);     // null: a launch of its own does it
 
     for (int s2 = 0; s2 < dm.V; ++s2) {
         const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;

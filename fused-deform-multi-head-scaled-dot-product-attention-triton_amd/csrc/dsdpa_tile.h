@@ -32,7 +32,7 @@ __device__ __forceinline__ void lds_accumulate(double *p, float x) { atomicAdd(p
 template <typename S, int D, int DC>
 __global__ __launch_bounds__(kTileWaves *kWave) void bwd_dkdv_tile_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
-    const float *__restrict__ coords_, const float *__restrict__ lse_, const float *__restrict__ delta_,
+    const float *__restrict__ coords_, const float2 *__restrict__ stats_,
     const void *__restrict__ dout_, float *__restrict__ dk_acc, float *__restrict__ dv_acc,
     Dims dm, TileGeom tg)
 {
@@ -110,8 +110,9 @@ __global__ __launch_bounds__(kTileWaves *kWave) void bwd_dkdv_tile_kernel(
                 const size_t roff = (row * D + lane_elem) * S::kBytes;
                 load_chunk<S, DC>((const char *)q_ + roff, qf);
                 load_chunk<S, DC>((const char *)dout_ + roff, dof);
-                lse = lse_[row];
-                delta = delta_[row];
+                const float2 ld = stats_[row];
+                lse = ld.x;
+                delta = ld.y;
                 row_loaded = true;
             }
             for (int j0 = 0; j0 < cnt; j0 += NS) {

@@ -50,7 +50,7 @@ def test_workspace_bytes():
 
     def expect(B, V, H, Himg, Wimg, D, P, storage16):
         rows, NC = B * V * H * Himg * Wimg, (Himg + 1) * (Wimg + 1)
-        total = r256(rows * 4) + r256(B * V * NC * 4) + r256(B * V * (NC + 1) * 4) + r256(B * V * V * Himg * Wimg * P * 4)
+        total = r256(rows * 8) + r256(B * V * NC * 4) + r256(B * V * (NC + 1) * 4) + r256(B * V * V * Himg * Wimg * P * 4)
         total += r256(2 * rows * D * 4) if storage16 else 0
         return total + table(B, V, Himg, Wimg, D, P, storage16)
 
