@@ -441,12 +441,12 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const float4 *desc_g = (const float4 *)(ws + wl.desc + wl.dl.g);
     const unsigned *start = (const unsigned *)(ws + wl.start);
     const unsigned *sorted = (const unsigned *)(ws + (deterministic ? wl.sorted2 : wl.sorted));
-    // one launch zeroes the dk/dv accumulators and, for the cell-binned path, the cell counters
+    // fp32 storage: dk and dv are their own accumulators; 16-bit: fp32 accumulators in the workspace
     float *dk_acc = S::kBytes == 4 ? (float *)dk : (float *)(ws + wl.acc);
     float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
-    // The binning (and the deterministic list ordering) runs beside the table fill and the dq kernel on the
-    // side lane: forked here, before anything is enqueued, joined before the dk/dv kernel. The side lane
-    // then clears the cell counters itself.
+    // Two sides that do not read what the other writes: tap table -> dq on the caller's stream, and clears ->
+    // (lse, delta) pairs -> binning (-> list ordering) -> dk/dv on the side lane. Forked here, before anything is
+    // enqueued; joined after the dk/dv kernel (before the casts of 16-bit storage, which need both).
     hipStream_t bst = st;
     SideLane *side = cell_binned && !(flags & DSDPA_FLAG_SINGLE_STREAM) ? side_lane() : nullptr;
     if (side && hipEventRecord(side->fork, st) == hipSuccess &&
@@ -464,7 +464,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     else if (!side_on || ndc) rc = zero_fill(zero, st);
     if (rc != DSDPA_OK) return rc;
     if (side_on) {
-        // the dk/dv side: clears, delta, binning, ordering; the dk/dv kernel follows below
+        // the dk/dv side: its clears, and the (lse, delta) pairs that the dq kernel otherwise writes on the way
         const ZeroJob zero_side{{dk_acc, dv_acc, (float *)(ws + wl.counters), nullptr}, {n, n, ncounters, 0}};
         if ((rc = zero_fill(zero_side, bst)) != DSDPA_OK) return rc;
         const size_t lanes = (size_t)dm.rows * 4;
