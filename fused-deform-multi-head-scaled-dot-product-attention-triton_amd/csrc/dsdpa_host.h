@@ -105,6 +105,12 @@ inline bool plane_path_fits(size_t L, size_t D, size_t esize, bool coords_grad =
     return (L + 2) * 2 * D * esize + kPlaneDescLdsBytes + (coords_grad ? kPlaneGradLdsBytes : 0) <= kLdsBytes;
 }
 
+// With very few samples per view the staged kernels mostly stage: every workgroup loads all V plane pairs for
+// P samples per row and view, while the gather kernels touch only the rows they sample. Measured on 18x18,
+// D = 32 (forward, staged / gather ms): V = 12: P = 2 0.344 / 0.245, P = 4 0.431 / 0.414, P = 5 0.485 / 0.516;
+// V = 8: P = 3 0.173 / 0.162, P = 4 0.195 / 0.200; V = 6: equal up to P = 2, staged ahead from there.
+inline bool few_samples_prefer_gather(size_t V, size_t P) { return P <= 3 && V >= 8; }
+
 // Descriptor table of the plane kernels: per coordinate pair 16 bytes of weights and 4 of packed slot
 // codes (plus, for the coordinate gradient, 16 bytes of derivative weights), computed once per call by
 // plane_descriptor_kernel. Empty when the plane kernels do not apply.

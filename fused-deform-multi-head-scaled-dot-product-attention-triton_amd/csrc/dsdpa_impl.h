@@ -270,7 +270,9 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
     hipStream_t st = (hipStream_t)stream;
     const DescLayout dl = desc_layout(B, V, Himg, Wimg, D, P, S::kBytes);
     if (dl.bytes && !workspace) return DSDPA_ERR_NULL_POINTER;
-    const bool staged = g_path.load() != DSDPA_PATH_GATHER && dl.bytes != 0;
+    const int path = g_path.load();
+    const bool staged = path != DSDPA_PATH_GATHER && dl.bytes != 0 &&
+                        (path == DSDPA_PATH_LDS || !few_samples_prefer_gather(V, P));
     char *ws = (char *)workspace;
     if (staged && (rc = launch_plane_descriptors(coords, dm, ws, dl, false, ZeroJob{}, 4, st)) != DSDPA_OK) return rc;
     const float4 *desc_w = (const float4 *)(ws + dl.w);
@@ -435,7 +437,8 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const bool fused_atomics = path == DSDPA_PATH_GATHER;
     const bool cell_binned = path == DSDPA_PATH_AUTO;
     // (with the coordinate gradient the layout holds a table only where the larger LDS block still fits)
-    const bool staged = !fused_atomics && wl.dl.bytes != 0 && (!dcoords || cg_table);
+    const bool staged = !fused_atomics && wl.dl.bytes != 0 && (!dcoords || cg_table) &&
+                        (path == DSDPA_PATH_LDS || !few_samples_prefer_gather(V, P));
     const float4 *desc_w = (const float4 *)(ws + wl.desc + wl.dl.w);
     const uint32_t *desc_e = (const uint32_t *)(ws + wl.desc + wl.dl.e);
     const float4 *desc_g = (const float4 *)(ws + wl.desc + wl.dl.g);

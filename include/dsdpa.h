@@ -166,7 +166,9 @@ int dsdpa_version(void);
  * table, ops/triton.py:10-25.
  */
 /* Forward and backward-dq: AUTO and LDS stage each key view's K/V planes in LDS
- * when a plane pair fits, GATHER always reads the taps from global memory.
+ * when a plane pair fits (AUTO: unless there are at most 3 samples per view and 8
+ * or more views, where staging costs more than it saves), GATHER always reads the
+ * taps from global memory.
  * Backward dk/dv: AUTO = cell-binned register accumulation, LDS = tiles of the
  * plane accumulated in LDS with fp64 atomics, GATHER = global float atomics per
  * tap as in the reference (ops/triton.py:345-360). */

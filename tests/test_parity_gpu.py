@@ -75,6 +75,7 @@ SMALL = [
     (9, 1, 3, 2, 11, 1, 32, 5, -0.2, 1.2),      # single-column image
     (10, 1, 2, 2, 4, 5, 32, 129, -0.1, 1.1),    # many samples per view: three 64-sample pieces of the tap table
     (11, 1, 1, 2, 6, 6, 64, 200, 0.0, 1.0),     # one view, 200 samples
+    (12, 1, 9, 1, 4, 3, 32, 2, -0.1, 1.1),      # many views, two samples each: the gather kernels are chosen
 ]
 
 
