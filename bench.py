@@ -43,8 +43,8 @@ def log(*a):
 MEASURED_TRAFFIC_BYTES = {
     "C2": {
         "fwd": int((35033.1 * 2.0 + 4009.5) * 1024),
-        "bwd_dq": int((38970.6 * 2.0 + 3888.0) * 1024),
-        "bwd_dkdv": int((42882.5 * 2.0 + 110976.0) * 1024),
+        "bwd_dq": int((38971.0 * 2.0 + 3888.0) * 1024),
+        "bwd_dkdv": int((42852.5 * 2.0 + 110976.0) * 1024),
     },
 }
 
