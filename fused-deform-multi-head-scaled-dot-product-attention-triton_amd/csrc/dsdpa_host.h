@@ -25,7 +25,7 @@ struct EventPair { hipEvent_t start, stop; };
 struct KernelTimer {
     std::atomic<bool> on{false};
     std::mutex mu;
-    std::vector<EventPair> pairs[5];   // [0] forward, [1] backward dk/dv, [2] backward dq, [3] cell binning, [4] descriptor table
+    std::vector<EventPair> pairs[5];   // [0] forward, [1] backward dk/dv, [2] backward dq, [3] cell binning (one pair per launch), [4] descriptor table
 };
 extern KernelTimer g_timer;
 
@@ -37,18 +37,25 @@ struct ScopedKernelTimer {
     EventPair ev{nullptr, nullptr};
     int which;
     bool armed = false, record;
+    mutable bool handed_out = false;       // a launch took the events (or they were recorded around a run)
     ScopedKernelTimer(int which_, hipStream_t st_, bool record_ = false) : st(st_), which(which_), record(record_)
     {
         if (!g_timer.on.load(std::memory_order_relaxed)) return;
         if (hipEventCreate(&ev.start) != hipSuccess) return;
         if (hipEventCreate(&ev.stop) != hipSuccess) { (void)hipEventDestroy(ev.start); return; }
         armed = record ? hipEventRecord(ev.start, st) == hipSuccess : true;
+        handed_out = record && armed;
     }
-    hipEvent_t start() const { return armed && !record ? ev.start : nullptr; }
-    hipEvent_t stop() const { return armed && !record ? ev.stop : nullptr; }
+    hipEvent_t start() const { handed_out = armed; return armed && !record ? ev.start : nullptr; }
+    hipEvent_t stop() const { handed_out = armed; return armed && !record ? ev.stop : nullptr; }
     ~ScopedKernelTimer()
     {
         if (!armed) return;
+        if (!handed_out) {                  // the launch never happened (an early error return)
+            (void)hipEventDestroy(ev.start);
+            (void)hipEventDestroy(ev.stop);
+            return;
+        }
         if (record) (void)hipEventRecord(ev.stop, st);
         std::lock_guard<std::mutex> lock(g_timer.mu);
         g_timer.pairs[which].push_back(ev);

@@ -25,6 +25,26 @@ static __global__ void fill_zero_kernel(ZeroJob job) { zero_buffers(job); }
         else hipLaunchKernelGGL(kern, grid, block, smem, st, __VA_ARGS__);                                   \
     } while (0)
 
+// Lets a kernel instantiation use the whole 160 KB of LDS as dynamic shared memory. The attribute belongs to
+// the kernel, not to the launch, so it is set once per instantiation and device (`done`: one bit per device),
+// to the largest block any launch may ask for; a launch's own block size is an argument of that launch.
+template <typename K>
+int allow_full_lds(K kern, std::atomic<unsigned long long> &done)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        (void)hipGetLastError();
+        dev = 0;
+    }
+    const unsigned long long bit = 1ull << dev;
+    if (done.load(std::memory_order_acquire) & bit) return DSDPA_OK;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    done.fetch_or(bit, std::memory_order_release);
+    return DSDPA_OK;
+}
+
 // fp32 accumulators -> 16-bit storage, 8 elements per thread
 template <typename S>
 __global__ void cast_kernel(const float *__restrict__ src, void *__restrict__ dst, size_t n8)
@@ -187,9 +207,8 @@ int launch_bwd_dkdv_tile(const void *q, const void *k, const void *v, const floa
     const long long blocks = (long long)dm.B * dm.H * dm.V * tg.nty * tg.ntx * tg.qsplit;
     if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
     auto kern = bwd_dkdv_tile_kernel<S, D, DC>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    static std::atomic<unsigned long long> lds_set{0};
+    if (int rc = allow_full_lds(kern, lds_set)) return rc;
     ScopedKernelTimer timer(1, st);
     DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(kTileWaves * kWave), smem, st,
                           timer.start(), timer.stop(),
@@ -229,9 +248,8 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float4 *
     const int rows_per_block = kPlaneWaves * (kWave / (D / DC));
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
     auto kern = fwd_slot_kernel<S, D, DC>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    static std::atomic<unsigned long long> lds_set{0};
+    if (int rc = allow_full_lds(kern, lds_set)) return rc;
     ScopedKernelTimer timer(0, st);
     DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
                           timer.start(), timer.stop(), q, k, v, desc_w, desc_e, out, lse, dm);
@@ -249,9 +267,8 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
     const int rows_per_block = kPlaneWaves * (kWave / (D / DC));
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
     auto kern = dcoords ? bwd_dq_slot_kernel<S, D, DC, true> : bwd_dq_slot_kernel<S, D, DC, false>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+    static std::atomic<unsigned long long> lds_set[2];
+    if (int rc = allow_full_lds(kern, lds_set[dcoords ? 1 : 0])) return rc;
     ScopedKernelTimer timer(2, st);
     DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(kPlaneWaves * kWave), smem, st,
                           timer.start(), timer.stop(), q, k, v, desc_w, desc_e, out, lse, dout, dq, stats, desc_g,
@@ -319,7 +336,8 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
     unsigned *start = (unsigned *)(ws + wl.start);
     unsigned *sorted = (unsigned *)(ws + wl.sorted);
     const size_t hist_bytes = (size_t)dm.V * wl.NC * sizeof(unsigned);
-    ScopedKernelTimer timer(3, st);
+    // each of the three launches carries its own pair of events: the timer's slot 3 adds up their busy time
+    ScopedKernelTimer t_count(3, st), t_scan(3, st), t_fill(3, st);
     if (2 * hist_bytes <= (size_t)kLdsBytes - 1024) {
         // LDS-aggregated passes: a workgroup per run of about 4k samples of one (b, s1); 8k when the
         // histogram is large, since every workgroup walks all of it twice (measured on 18x18 and 48x48)
@@ -332,18 +350,16 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
         if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
         auto k0 = bin_samples_lds_kernel<0>;
         auto k1 = bin_samples_lds_kernel<1>;
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k0),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)hist_bytes);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k1),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * hist_bytes));
-        if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+        static std::atomic<unsigned long long> lds_set[2];
+        if (int rc = allow_full_lds(k0, lds_set[0])) return rc;
+        if (int rc = allow_full_lds(k1, lds_set[1])) return rc;
         DSDPA_LAUNCH(k0, dim3((unsigned)blocks), dim3(kBinLdsThreads), hist_bytes, st,
-                              timer.start(), nullptr,
+                              t_count.start(), t_count.stop(),
                            coords, dm, wl.NC, lchunk, nlc, counters, sorted);
-        hipLaunchKernelGGL(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st, counters, start, wl.NC);
+        DSDPA_LAUNCH(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st,
+                              t_scan.start(), t_scan.stop(), counters, start, wl.NC);
         DSDPA_LAUNCH(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
-                              nullptr, timer.stop(),
+                              t_fill.start(), t_fill.stop(),
                            coords, dm, wl.NC, lchunk, nlc, counters, sorted);
         return check_launch();
     }
@@ -351,11 +367,12 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
     const long long blocks = (total + kBinThreads - 1) / kBinThreads;
     if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
     DSDPA_LAUNCH(bin_samples_kernel<0>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
-                          timer.start(), nullptr,
+                          t_count.start(), t_count.stop(),
                        coords, dm, wl.NC, counters, sorted);
-    hipLaunchKernelGGL(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st, counters, start, wl.NC);
+    DSDPA_LAUNCH(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st,
+                          t_scan.start(), t_scan.stop(), counters, start, wl.NC);
     DSDPA_LAUNCH(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
-                          nullptr, timer.stop(),
+                          t_fill.start(), t_fill.stop(),
                        coords, dm, wl.NC, counters, sorted);
     return check_launch();
 }
@@ -412,6 +429,26 @@ static inline int launch_list_ordering(const Dims &dm, const WorkspaceLayout &wl
                            (unsigned *)(ws + wl.sorted2), ids, segs, seg_begin, seg_end, bits, st);
 }
 
+// Joins the backward's side lane to the caller's stream, once: by join() on the normal path, by the
+// destructor on every other way out of bwd_impl after the fork (an error return must not leave work on the
+// side lane that the caller's stream does not wait for: the caller may free the buffers it writes, and a
+// stream capture with an unjoined fork is invalid).
+struct SideJoin {
+    SideLane *side = nullptr;
+    hipStream_t main = nullptr;
+    bool pending = false;
+    int join()
+    {
+        if (!pending) return DSDPA_OK;
+        pending = false;
+        hipError_t e = hipEventRecord(side->join, side->stream);
+        if (e == hipSuccess) e = hipStreamWaitEvent(main, side->join, 0);
+        if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
+        return DSDPA_OK;
+    }
+    ~SideJoin() { (void)join(); }
+};
+
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
              const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
@@ -452,9 +489,14 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     // enqueued; joined after the dk/dv kernel (before the casts of 16-bit storage, which need both).
     hipStream_t bst = st;
     SideLane *side = cell_binned && !(flags & DSDPA_FLAG_SINGLE_STREAM) ? side_lane() : nullptr;
+    SideJoin joiner;
     if (side && hipEventRecord(side->fork, st) == hipSuccess &&
-        hipStreamWaitEvent(side->stream, side->fork, 0) == hipSuccess)
+        hipStreamWaitEvent(side->stream, side->fork, 0) == hipSuccess) {
         bst = side->stream;
+        joiner.side = side;
+        joiner.main = st;
+        joiner.pending = true;
+    }
     const bool side_on = bst != st;
     const size_t ncounters = cell_binned ? wl.counters_bytes / 4 : 0;
     const size_t ndc = dcoords ? (size_t)dm.B * dm.V * dm.L * dm.N * 2 : 0;
@@ -478,13 +520,6 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, bst)) != DSDPA_OK) return rc;
     if (deterministic && (rc = launch_list_ordering(dm, wl, ws, bst)) != DSDPA_OK) return rc;
     float2 *dq_stats = side_on ? nullptr : stats;       // the dq kernel writes them only when dk/dv runs behind it
-    const auto join_side = [&]() -> int {
-        if (!side_on) return DSDPA_OK;
-        hipError_t e = hipEventRecord(side->join, bst);
-        if (e == hipSuccess) e = hipStreamWaitEvent(st, side->join, 0);
-        if (e != hipSuccess) { g_last_hip_error = (int)e; return DSDPA_ERR_HIP; }
-        return DSDPA_OK;
-    };
 #define DSDPA_BWD_CASE(DD)                                                                                      \
     case DD:                                                                                                    \
         if (fused_atomics && !dcoords) {                                                                        \
@@ -499,7 +534,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
                                                  dv_acc, dm, wl.NC, deterministic, bst);                        \
             else if (rc == DSDPA_OK)                                                                            \
                 rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, stats, dout, dk_acc, dv_acc, dm, st);         \
-            if (rc == DSDPA_OK) rc = join_side();                                                               \
+            if (rc == DSDPA_OK) rc = joiner.join();                                                              \
         }                                                                                                       \
         break;
     switch (D) {

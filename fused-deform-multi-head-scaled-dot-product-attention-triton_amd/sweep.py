@@ -8,6 +8,10 @@ before use, and timing uses HIP events on the current stream (median of ``--rep`
 
     python sweep.py --b 2 --h 8 --d 32 --iw 18            # full sweep, prints a table per mode
     python sweep.py --quick                               # S, P in {2, 6, 12} only
+
+Besides the printed tables it leaves, in ``--save-path`` (default ``./results``), ``logs.txt`` with the ``[Mem]``
+lines and one latency CSV (and one peak-memory CSV) per mode and ``P_samples`` -- the files the reference's
+``perf_report`` run writes (``benchmark.py:106``).
 """
 import argparse
 import os
@@ -88,6 +92,23 @@ def bench_point(provider, mode, q, k, v, coords, W_IMG, H_IMG, sm_scale, warmup,
     return ms, peak_mb
 
 
+def write_csv_tables(rows, args, providers, S_LIST, P_LIST):
+    """One CSV per (mode, P_samples) line of the sweep, named and shaped like the tables the reference harness
+    leaves in its results directory (``benchmark.py:106``, ``perf_report(...).run(save_path=..., print_data=True)``:
+    x column ``S_views``, one latency column per provider), so that the published plots can be redrawn; plus the
+    peak-memory table of the same points (the reference keeps those figures as ``[Mem]`` lines only)."""
+    titles = {"fused": "HIP (coord-fused)", "torch": "Torch (grid_sample)"}
+    for mode in ("fwd", "bwd"):
+        for P in P_LIST:
+            name = f"coord-attn-B{args.b}-H{args.h}-D{args.d}-{mode}-W{args.iw}-P{P}"
+            for suffix, col in ((".csv", 4), ("-peak-mb.csv", 5)):
+                with open(os.path.join(args.save_path, name + suffix), "w") as f:
+                    f.write("S_views," + ",".join(titles[p] for p in providers) + "\n")
+                    for S in S_LIST:
+                        vals = {r[3]: r[col] for r in rows if r[:3] == (mode, P, S)}
+                        f.write(f"{S:.1f}," + ",".join(f"{vals[p]:.6f}" for p in providers) + "\n")
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description="Sweep of deformable multi-view SDPA: fused HIP kernels vs eager PyTorch.")
     ap.add_argument("--b", type=int, default=2, help="Batch size.")
@@ -128,6 +149,7 @@ def main(argv=None):
                           f"H={args.iw} P={P} D={args.d} | peak={peak:.1f} MB", file=log, flush=True)
                 del q, k, v, coords
     log.close()
+    write_csv_tables(rows, args, providers, S_LIST, P_LIST)
     for mode in ("fwd", "bwd"):
         print(f"\nlatency (ms), mode={mode}, B={args.b} H={args.h} D={args.d} W={args.iw} dtype={args.dtype}")
         print("  P   S " + " ".join(f"{p:>12s}" for p in providers) + "   peak MB " + " ".join(f"{p:>10s}" for p in providers))

@@ -97,20 +97,22 @@ def test_coords_gradient_skipped_when_coords_do_not_require_grad():
     assert c.grad is None and q.grad is not None
 
 
-@pytest.mark.parametrize("name", ["C2", "C3"])
-def test_coords_gradient_named_workloads(name):
-    """Full-size workload; the oracle runs on batch item 0 (all heads: the gradient sums over them)."""
+@pytest.mark.parametrize("name,batch", [("C2", 0), ("C2", 1), ("C3", 0), ("C4", 1), ("C5", 1)],
+                         ids=["C2-b0", "C2-b1", "C3-b0", "C4-b1", "C5-b1"])
+def test_coords_gradient_named_workloads(name, batch):
+    """Full-size workload; the oracle runs on one batch item (all its heads: the gradient sums over them),
+    the first or the last one."""
     wl = WORKLOADS[name]
-    say(f"[case] coords grad workload {name}")
+    say(f"[case] coords grad workload {name} batch item {batch}")
     q, k, v, c, do = gen_inputs(wl)
     dev = "cuda:0"
     qg, kg, vg, cg = (t.to(dev).requires_grad_(True) for t in (q, k, v, c))
     out = deform_sdpa_triton(qg, kg, vg, cg, wl.W_IMG, wl.H_IMG, wl.sm_scale, True)
     out.backward(do.to(dev))
     torch.cuda.synchronize()
-    f = lambda t: t[:1].float().numpy()
+    f = lambda t: t[batch:batch + 1].float().numpy()
     *_, dc_r = oracle_bwd(f(q), f(k), f(v), f(c), f(do), wl.W_IMG, wl.H_IMG, wl.sm_scale, with_coords=True)
-    assert rel(cg.grad[:1], dc_r) < TOL[wl.torch_dtype()]
+    assert rel(cg.grad[batch:batch + 1], dc_r) < TOL[wl.torch_dtype()]
     # the whole tensor: finite, and zero exactly where a sample has no tap inside the image
     assert torch.isfinite(cg.grad).all()
     if wl.coords == "border":

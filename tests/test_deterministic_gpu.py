@@ -12,6 +12,7 @@ import torch
 from oracle import oracle_bwd
 from ops.triton import deform_sdpa_triton
 from workloads import WORKLOADS, gen_inputs
+from parity_util import oracle_on_slices, slice_bh
 
 pytestmark = pytest.mark.gpu
 
@@ -92,6 +93,24 @@ def test_deterministic_backward_c2_bitwise_repeatable(deterministic):
     plain = grads(q, k, v, c, do, wl.W_IMG, wl.H_IMG, wl.sm_scale)
     for a, b in zip(first, plain):
         assert rel(a, b.double().cpu().numpy()) < 1e-3
+
+
+def test_deterministic_backward_c5_full_size(deterministic):
+    """Full-size C5 (clustered coordinates: cell lists of up to several thousand samples, the case the list
+    ordering exists for): the oracle's bars on two (batch, head) slices, and identical bits on a rerun."""
+    wl = WORKLOADS["C5"]
+    say("[case] deterministic C5")
+    q, k, v, c, do = gen_inputs(wl)
+    dev = [t.to("cuda:0") for t in (q, k, v, c, do)]
+    first = grads(*dev, wl.W_IMG, wl.H_IMG, wl.sm_scale)
+    again = grads(*dev, wl.W_IMG, wl.H_IMG, wl.sm_scale)
+    for a, b in zip(first, again):
+        assert torch.equal(a, b)
+    slices = [(0, 1), (wl.B - 1, wl.H - 1)]
+    ref = oracle_on_slices(q, k, v, c, do, wl.W_IMG, wl.H_IMG, wl.sm_scale, slices, forward=False)
+    for (b, h), (_, rdq, rdk, rdv) in ref.items():
+        for got, want in zip(first, (rdq, rdk, rdv)):
+            assert rel(slice_bh(got, b, h), want) < TOL[torch.bfloat16], (b, h)
 
 
 def test_deterministic_with_coords_gradient_is_refused(deterministic):

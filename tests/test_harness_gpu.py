@@ -32,6 +32,13 @@ def test_sweep_harness_check_lines(tmp_path, capsys):
     assert len(rows) == 2 * 3 * 3 * 2
     assert all(ms > 0 for (_, _, _, _, ms, _) in rows)
     assert os.path.exists(os.path.join(str(tmp_path), "logs.txt"))
+    # the per-line tables the reference's perf_report run leaves (benchmark.py:106)
+    for mode in ("fwd", "bwd"):
+        for P in (2, 6, 12):
+            path = os.path.join(str(tmp_path), f"coord-attn-B1-H2-D32-{mode}-W6-P{P}.csv")
+            lines = open(path).read().splitlines()
+            assert lines[0].startswith("S_views,") and len(lines) == 1 + 3
+            assert all(float(x) > 0 for l in lines[1:] for x in l.split(","))
 
 
 @pytest.mark.parametrize("P", [1, 2, 5, 12, 33, 64, 100])
