@@ -12,6 +12,38 @@ std::atomic<int> g_path{DSDPA_PATH_AUTO};
 KernelTimer g_timer;
 }  // namespace dsdpa
 
+// Built-in scratch of dsdpa_fwd_noalloc: the forward's workspace (the per-coordinate tap table) for callers
+// that cannot allocate. Every GPU the library runs on holds its own copy of the array, at its own address,
+// until the process ends. In host code the array's name is only a handle for hipGetSymbolAddress: the
+// device address is looked up once per device (with that device current) and kept in g_scratch_ptr; host
+// code passes that pointer, never the array's name, to kernels.
+static __device__ __align__(256) unsigned char scratch[DSDPA_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device; null (and the HIP error kept) if it cannot be had.
+void *scratch_on_current_device()
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        g_last_hip_error = (int)(e != hipSuccess ? e : hipErrorInvalidDevice);
+        return nullptr;
+    }
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+        g_last_hip_error = (int)(e != hipSuccess ? e : hipErrorInvalidSymbol);
+        return nullptr;
+    }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);      // (two threads racing here store the same address)
+    return p;
+}
+}  // namespace
+
 extern "C" {
 
 int dsdpa_fwd_f32(const float *q, const float *k, const float *v, const float *coords, float *out, float *lse, void *workspace,
@@ -56,6 +88,26 @@ int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coor
                          sm_scale, flags, stream);
 }
 
+int dsdpa_fwd_noalloc(int dtype, const void *q, const void *k, const void *v, const float *coords, void *out,
+                      float *lse, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+{
+    if (dtype != DSDPA_F32 && dtype != DSDPA_BF16 && dtype != DSDPA_F16) return DSDPA_ERR_DTYPE;
+    if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || P < 1) return DSDPA_ERR_BAD_SHAPE;
+    if (!(D == 16 || D == 32 || D == 64 || D == 128 || D == 256)) return DSDPA_ERR_HEAD_DIM;
+    const size_t need = desc_layout(B, V, Himg, Wimg, D, P, dtype != DSDPA_F32 ? 2 : 4).bytes;
+    if (need > (size_t)DSDPA_NOALLOC_SCRATCH_BYTES) return DSDPA_ERR_SCRATCH;
+    void *ws = nullptr;
+    if (need) {
+        ws = scratch_on_current_device();
+        if (!ws) return DSDPA_ERR_HIP;
+    }
+    switch (dtype) {
+    case DSDPA_F32: return fwd_impl<F32>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+    case DSDPA_BF16: return fwd_impl<BF16>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+    default: return fwd_impl<F16>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+    }
+}
+
 size_t dsdpa_fwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P)
 {
     if (dtype != DSDPA_F32 && dtype != DSDPA_BF16 && dtype != DSDPA_F16) return 0;
@@ -82,6 +134,7 @@ const char *dsdpa_error_string(int code)
     case DSDPA_ERR_HIP: return "a HIP launch failed (see dsdpa_last_hip_error)";
     case DSDPA_ERR_UNSUPPORTED: return "unknown flag, or a combination of options that is not supported";
     case DSDPA_ERR_DTYPE: return "unknown dtype code";
+    case DSDPA_ERR_SCRATCH: return "the shape needs more scratch memory than the library's built-in buffer holds";
     }
     return "unknown error code";
 }

@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libdsdpa.so")
 # every symbol include/dsdpa.h declares
 SYMBOLS = (
     "dsdpa_fwd_f32", "dsdpa_fwd_bf16", "dsdpa_fwd_f16",
-    "dsdpa_bwd_f32", "dsdpa_bwd_bf16", "dsdpa_bwd_f16",
+    "dsdpa_bwd_f32", "dsdpa_bwd_bf16", "dsdpa_bwd_f16", "dsdpa_fwd_noalloc",
     "dsdpa_fwd_workspace_bytes", "dsdpa_bwd_workspace_bytes", "dsdpa_error_string", "dsdpa_last_hip_error",
     "dsdpa_version", "dsdpa_set_path", "dsdpa_timer_enable", "dsdpa_timer_collect",
 )
@@ -23,6 +23,8 @@ PATH_AUTO, PATH_GATHER, PATH_LDS = 0, 1, 2
 FLAG_DETERMINISTIC = 1
 FLAG_COORDS_GRAD = 2
 FLAG_SINGLE_STREAM = 4
+ERR_SCRATCH = 8
+NOALLOC_SCRATCH_BYTES = 32 << 20
 
 _lib = None
 
@@ -51,6 +53,8 @@ def load():
         bwd = getattr(lib, "dsdpa_bwd_" + sfx)
         bwd.argtypes = [vp] * 12 + dims[:-1] + [u, vp]   # q k v coords out lse dout dq dk dv dcoords workspace, dims, flags, stream
         bwd.restype = i
+    lib.dsdpa_fwd_noalloc.argtypes = [i] + [vp] * 6 + dims      # dtype, q k v coords out lse, dims
+    lib.dsdpa_fwd_noalloc.restype = i
     lib.dsdpa_fwd_workspace_bytes.argtypes = [i] * 8
     lib.dsdpa_fwd_workspace_bytes.restype = ctypes.c_size_t
     lib.dsdpa_bwd_workspace_bytes.argtypes = [i] * 8 + [u]

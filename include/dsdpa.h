@@ -57,7 +57,8 @@ enum {
                                      rows exceed 2^31-1                                   */
     DSDPA_ERR_HIP = 5,            /* a HIP launch failed; see dsdpa_last_hip_error()      */
     DSDPA_ERR_DTYPE = 6,          /* unknown dtype code                                   */
-    DSDPA_ERR_UNSUPPORTED = 7     /* unknown flag bit, or DSDPA_FLAG_DETERMINISTIC with dcoords */
+    DSDPA_ERR_UNSUPPORTED = 7,    /* unknown flag bit, or DSDPA_FLAG_DETERMINISTIC with dcoords */
+    DSDPA_ERR_SCRATCH = 8         /* dsdpa_fwd_noalloc: the shape needs more than DSDPA_NOALLOC_SCRATCH_BYTES */
 };
 
 /* Storage types (accumulation is always fp32). Mirrors the reference's dtype
@@ -86,6 +87,23 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
                   void *out, float *lse, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
                   float sm_scale, void *stream);
+
+/*
+ * Forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same computation and results
+ * as dsdpa_fwd_{f32,bf16,f16} (`dtype` = DSDPA_F32 / DSDPA_BF16 / DSDPA_F16 selects which), but the
+ * workspace is not an argument: it is a buffer of DSDPA_NOALLOC_SCRATCH_BYTES built into the library, one
+ * copy per GPU, held until the process ends. The call allocates and frees nothing. A shape whose
+ * dsdpa_fwd_workspace_bytes() exceeds the buffer is refused with DSDPA_ERR_SCRATCH before anything is
+ * launched (shapes that need no workspace always pass). All calls on one GPU share that GPU's buffer: calls
+ * that overlap on one GPU (two streams, two threads) race on it; calls on one stream, or otherwise ordered,
+ * are fine, since every call rewrites all of the scratch it reads.
+ */
+#define DSDPA_NOALLOC_SCRATCH_BYTES (32u << 20)
+int dsdpa_fwd_noalloc(int dtype, const void *q, const void *k, const void *v, const float *coords,
+                      void *out, float *lse,
+                      int B, int V, int H, int Himg, int Wimg, int D, int P,
+                      float sm_scale, void *stream);
 
 /* Flags of the backward. The reference has one backward, with float atomics (ops/triton.py:345-360).
  * DSDPA_FLAG_DETERMINISTIC: bitwise reproducible dq, dk, dv: the samples of every bilinear cell are
