@@ -126,36 +126,56 @@ __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
 // One workgroup per (b, s2): exclusive scan of the NC cell counts. Writes
 // start[grp*(NC+1) + c] (with the total at c = NC) and resets counters to the
 // same starts, so that the fill pass can use them as cursors.
+//
+// It also makes the dk/dv kernel's work list of this (b, s2): one item (cell, piece) per run of at most
+// `piece` consecutive entries of a non-empty cell list, in cell order -- items[grp*wmax + i], i < nitems[grp].
+// Empty cells get no item (clustered coordinates leave most of the grid empty), and a list much longer than
+// the average is cut into pieces that different waves take, so that the longest list no longer sets the
+// kernel's duration. wmax >= NC + M/piece bounds the number of items (M = entries of all lists).
 static __global__ __launch_bounds__(1024) void bin_scan_kernel(unsigned *__restrict__ counters,
-                                                        unsigned *__restrict__ start, int NC)
+                                                        unsigned *__restrict__ start, int NC, unsigned piece,
+                                                        unsigned wmax, uint2 *__restrict__ items,
+                                                        unsigned *__restrict__ nitems)
 {
-    __shared__ unsigned s_part[1024];
-    __shared__ unsigned s_carry;
+    __shared__ unsigned s_part[1024], s_pcs[1024];
+    __shared__ unsigned s_carry, s_pcarry;
     unsigned *cnt = counters + (size_t)blockIdx.x * NC;
     unsigned *st = start + (size_t)blockIdx.x * (NC + 1);
-    if (threadIdx.x == 0) s_carry = 0;
+    uint2 *it = items + (size_t)blockIdx.x * wmax;
+    if (threadIdx.x == 0) { s_carry = 0; s_pcarry = 0; }
     __syncthreads();
     for (int base = 0; base < NC; base += 1024) {
         const int c = base + threadIdx.x;
         const unsigned v = c < NC ? cnt[c] : 0u;
+        const unsigned np = (v + piece - 1) / piece;               // pieces of this cell's list
         s_part[threadIdx.x] = v;
+        s_pcs[threadIdx.x] = np;
         __syncthreads();
-        for (int off = 1; off < 1024; off <<= 1) {             // Hillis-Steele inclusive scan
-            unsigned add = threadIdx.x >= (unsigned)off ? s_part[threadIdx.x - off] : 0u;
+        for (int off = 1; off < 1024; off <<= 1) {             // Hillis-Steele inclusive scans, both at once
+            const bool take = threadIdx.x >= (unsigned)off;
+            const unsigned add = take ? s_part[threadIdx.x - off] : 0u;
+            const unsigned padd = take ? s_pcs[threadIdx.x - off] : 0u;
             __syncthreads();
             s_part[threadIdx.x] += add;
+            s_pcs[threadIdx.x] += padd;
             __syncthreads();
         }
         const unsigned excl = s_carry + s_part[threadIdx.x] - v;
+        const unsigned pexcl = s_pcarry + s_pcs[threadIdx.x] - np;
         if (c < NC) {
             st[c] = excl;
             cnt[c] = excl;
+            for (unsigned i = 0; i < np; ++i)
+                if (pexcl + i < wmax) it[pexcl + i] = make_uint2((unsigned)c, i);
         }
         __syncthreads();
-        if (threadIdx.x == 1023) s_carry += s_part[1023];
+        if (threadIdx.x == 1023) { s_carry += s_part[1023]; s_pcarry += s_pcs[1023]; }
         __syncthreads();
     }
-    if (threadIdx.x == 0) st[NC] = s_carry;
+    if (threadIdx.x == 0) {
+        st[NC] = s_carry;
+        nitems[blockIdx.x] = min(s_pcarry, wmax);
+    }
 }
 
 // Deterministic backward: begin / end of every cell list as positions in the flat id array
@@ -183,6 +203,49 @@ __device__ __forceinline__ void load_tap_or_zero(const char *base, int pix, int 
     }
 }
 
+// A lane's part of one query row as it comes from memory: q and dout words (storage type), and the row's
+// (lse, delta) pair.
+template <int WORDS> struct RowFetch { uint32_t qw[WORDS], dw[WORDS]; float2 ld; };
+
+template <int WORDS>
+__device__ __forceinline__ void load_words(const void *p, uint32_t (&w)[WORDS])
+{
+    static_assert(WORDS == 2 || WORDS % 4 == 0, "8 bytes, or multiples of 16");
+    if constexpr (WORDS == 2) {
+        const uint2 t = *reinterpret_cast<const uint2 *>(p);
+        w[0] = t.x; w[1] = t.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < WORDS / 4; ++i) {
+            const uint4 t = reinterpret_cast<const uint4 *>(p)[i];
+            w[4 * i + 0] = t.x; w[4 * i + 1] = t.y; w[4 * i + 2] = t.z; w[4 * i + 3] = t.w;
+        }
+    }
+}
+
+// the words of load_words as DC fp32 values
+template <typename S, int DC>
+__device__ __forceinline__ void widen_words(const uint32_t (&w)[DC * S::kBytes / 4], float (&dst)[DC])
+{
+    if constexpr (S::kBytes == 4) {
+#pragma unroll
+        for (int d = 0; d < DC; ++d) dst[d] = __uint_as_float(w[d]);
+    } else {
+#pragma unroll
+        for (int j = 0; j < DC / 2; ++j) {
+            if constexpr (S::kBf16) {
+                dst[2 * j + 0] = __uint_as_float(w[j] << 16);
+                dst[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+            } else {
+                union { uint32_t u; _Float16 h[2]; } cv;
+                cv.u = w[j];
+                dst[2 * j + 0] = (float)cv.h[0];
+                dst[2 * j + 1] = (float)cv.h[1];
+            }
+        }
+    }
+}
+
 // Which cells one launch of the dk/dv kernel covers, and the divisors that decode a work index into
 // (b, h, s2, cell) with multiply-shift instead of integer division (the decode is scalar code every
 // wave runs before it knows whether its cell is empty).
@@ -190,42 +253,62 @@ __device__ __forceinline__ void load_tap_or_zero(const char *base, int pix, int 
 // colour 0..3 (deterministic backward): only the cells with (row parity, column parity) = colour; no
 // two of them share a pixel, so the flush is a plain read-add-write, and the four launches, one
 // after the other, add every pixel's four contributions in a fixed order.
+// colour < 0 also switches the decode to the work list made by bin_scan_kernel: work index -> (b, h, s2, item),
+// `ncells` then being the list's capacity wmax per (b, s2); items beyond the list's length leave at once.
 struct CellGrid {
     int colour, oy, ox, step, ncx, ncells;
     unsigned nwork;                         // B*H*V*ncells < 2^31
+    unsigned piece;                         // entries per work item (work-list mode)
     FastDiv div_cells, div_ncx, div_v, div_h;
 };
 
 template <typename S, int D, int DC>
-__global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 3 : 2)) void bwd_dkdv_cell_kernel(
+__global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 4) : (S::kBytes == 2 ? 3 : 2)) void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float2 *__restrict__ stats_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
+    const uint2 *__restrict__ items, const unsigned *__restrict__ nitems,
     float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC, CellGrid cg)
 {
     constexpr int G = D / DC;
     constexpr int NS = kWave / G;
-    static_assert(G >= 1 && G <= 64 && G * DC == D, "lane split");
+    static_assert(G >= 4 && G <= 64 && G * DC == D, "lane split (a block of four lanes must not straddle two samples)");
     __shared__ float4 s_w[kCellWaves][kWave];
     __shared__ unsigned s_row[kCellWaves][kWave];
+    __shared__ float2 s_f[S::kBytes == 2 ? kCellWaves : 1][kWave];          // 16-bit storage: (fx, fy) of the entry
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const unsigned work = (unsigned)xcd_logical_block(blockIdx.x, gridDim.x) * kCellWaves + wave;
     if (work >= cg.nwork) return;
     const int colour = cg.colour;
-    // plane-major: (b, h, s2, cell)
+    // plane-major: (b, h, s2, cell or work item)
     unsigned t = cg.div_cells.div(work);
     const int ci = (int)(work - t * (unsigned)cg.ncells);
-    const int cyi = (int)cg.div_ncx.div((unsigned)ci);
-    const int cy = cyi * cg.step + cg.oy, cx = (ci - cyi * cg.ncx) * cg.step + cg.ox;   // on the (Himg+1) x (Wimg+1) grid
-    const int cell = cy * (dm.Wimg + 1) + cx;
     const unsigned bh = cg.div_v.div(t);
     const int s2 = (int)(t - bh * (unsigned)dm.V);
     const int b = (int)cg.div_h.div(bh);
     const int h = (int)(bh - (unsigned)b * (unsigned)dm.H);
     const size_t grp = (size_t)b * dm.V + s2;
-    const unsigned lo = start[grp * (NC + 1) + cell], hi = start[grp * (NC + 1) + cell + 1];
-    if (lo == hi) return;
+    int cy, cx, cell;
+    unsigned lo, hi;
+    if (colour < 0) {
+        if ((unsigned)ci >= nitems[grp]) return;
+        const uint2 item = items[grp * (size_t)cg.ncells + ci];
+        cell = (int)item.x;
+        cy = (int)cg.div_ncx.div(item.x);                      // div_ncx: by Wimg + 1 in this mode
+        cx = cell - cy * (dm.Wimg + 1);
+        const unsigned l0 = start[grp * (NC + 1) + cell], l1 = start[grp * (NC + 1) + cell + 1];
+        lo = l0 + item.y * cg.piece;
+        hi = min(l1, lo + cg.piece);
+    } else {
+        const int cyi = (int)cg.div_ncx.div((unsigned)ci);
+        cy = cyi * cg.step + cg.oy;
+        cx = (ci - cyi * cg.ncx) * cg.step + cg.ox;            // on the (Himg+1) x (Wimg+1) grid
+        cell = cy * (dm.Wimg + 1) + cx;
+        lo = start[grp * (NC + 1) + cell];
+        hi = start[grp * (NC + 1) + cell + 1];
+    }
+    if (lo >= hi) return;
 
     const int g = lane % G, slot = lane / G, lane_elem = g * DC;
     const int y0 = cy - 1, x0 = cx - 1;
@@ -241,6 +324,15 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
     constexpr bool kPacked = S::kBytes == 2;
     float kt[4][kPacked ? 1 : DC], vt[4][kPacked ? 1 : DC], aK[4][DC], aV[4][DC];
     uint32_t ktp[4][kPacked ? DC / 2 : 1], vtp[4][kPacked ? DC / 2 : 1];
+    // The per-sample rank-1 updates aK[t][d] += c_t * q[d], aV[t][d] += c'_t * dout[d] run on the 4x4 block
+    // matrix instruction (see block_outer_fma): mK[d][t] / mV[d][t] are the same sums as aK[t][d] / aV[t][d].
+    floatx4 mK[DC], mV[DC];
+    // The row of the update that lane (lane & 3) supplies is a product a_x(fx) * a_y(fy) of two linear forms
+    // with per-lane constants, so no lane ever selects among the four: packed (the bilinear weight of tap
+    // lane & 3): a_x = 1 - fx or fx, a_y = 1 - fy or fy; fp32 (the moment 1, fx, fy, fx*fy): a_x = 1 or fx,
+    // a_y = 1 or fy.
+    const float row_sx = (lane & 1) ? 1.0f : (kPacked ? -1.0f : 0.0f), row_ox = (lane & 1) ? 0.0f : 1.0f;
+    const float row_sy = (lane & 2) ? 1.0f : (kPacked ? -1.0f : 0.0f), row_oy = (lane & 2) ? 0.0f : 1.0f;
 #pragma unroll
     for (int tpi = 0; tpi < 4; ++tpi) {
         if constexpr (kPacked) {
@@ -254,9 +346,9 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
             load_tap_or_zero<S, DC>(kb, tpix[tpi], D, lane_elem, tv[tpi], kt[tpi]);
             load_tap_or_zero<S, DC>(vb, tpix[tpi], D, lane_elem, tv[tpi], vt[tpi]);
         }
-#pragma unroll
-        for (int d = 0; d < DC; ++d) { aK[tpi][d] = 0.f; aV[tpi][d] = 0.f; }
     }
+#pragma unroll
+    for (int d = 0; d < DC; ++d) { mK[d] = floatx4{0.f, 0.f, 0.f, 0.f}; mV[d] = floatx4{0.f, 0.f, 0.f, 0.f}; }
     // fp32 storage: the cell's taps are turned, once, into the coefficients of the bilinear form
     //   blend(fx, fy) = T00 + fx*(T01 - T00) + fy*(T10 - T00) + fx*fy*(T00 - T01 - T10 + T11)
     // so that a sample's blend costs 3 multiply-adds per element instead of 4, and the sums are kept as the
@@ -280,6 +372,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
     // (s1*H*L + l) * ROW < V*H*L*D*e <= 2^32 (the shape limits keep one batch item of a tensor below 2^30
     // elements): one add per gather instead of 64-bit address arithmetic per lane.
     constexpr unsigned kRowBytes = D * S::kBytes;
+    constexpr int kRowWords = DC * S::kBytes / 4;                           // 32-bit words of a row held by one lane
     constexpr int kRowToPairShift = __builtin_ctz(kRowBytes) - 3;          // row byte offset -> offset of the row's (lse, delta)
     const size_t bh_row0 = ((size_t)b * dm.V * dm.H + h) * dm.L;              // row of (b, s1 = 0, h, l = 0)
     const char *q_bh = (const char *)q_ + bh_row0 * kRowBytes;
@@ -290,10 +383,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
     const float2 *coords = reinterpret_cast<const float2 *>(coords_);
 
     // Walk the list 64 entries at a time. Sample ids are fetched one chunk ahead
-    // (the coordinate load depends on them). A software-pipelined version of the
-    // inner loop (query rows of the next NS samples prefetched) was measured
-    // slower: the register copies it adds cost more VALU issue slots than the
-    // four resident waves per SIMD fail to hide.
+    // (the coordinate load depends on them).
     auto load_id = [&](unsigned cstart) -> unsigned {
         return cstart < hi ? list[min(cstart + (unsigned)lane, hi - 1u)] : 0u;
     };
@@ -315,35 +405,41 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
         // entries past the end of the list repeat its last sample with zero weights: they add nothing
         const bool live = c0 + (unsigned)lane < hi;
         wave_lds_sync();
-        if constexpr (kPacked)
+        if constexpr (kPacked) {
             s_w[wave][lane] = live ? make_float4(gx * gy, fx * gy, gx * fy, fx * fy) : make_float4(0.f, 0.f, 0.f, 0.f);
-        else
+            s_f[wave][lane] = make_float2(fx, live ? fy : __int_as_float(0x7fc00000));     // NaN marks a dead entry
+        } else {
             s_w[wave][lane] = make_float4(fx, fy, fx * fy, live ? 1.0f : 0.0f);
+        }
         s_row[wave][lane] = (s1 * view_rows + l) * kRowBytes;
         wave_lds_sync();
         const int cnt = (int)min((unsigned)kWave, hi - c0);
-        for (int j0 = 0; j0 < cnt; j0 += NS) {
-            const float4 w = s_w[wave][j0 + slot];
+        // The NS samples of a trip need their query rows (q, dout, lse, delta) from memory, a round trip of
+        // several hundred nanoseconds that the two or three other waves of the SIMD do not cover. So the rows
+        // of trip t+1 are requested before trip t is worked on: two sets of row registers, used in turn (the
+        // loop is unrolled by two so that no set is ever copied).
+        auto issue = [&](int j0, RowFetch<kRowWords> &f) {
             const unsigned r = s_row[wave][j0 + slot];
             const unsigned roff = r + lane_byte, soff = r >> kRowToPairShift;
+            load_words<kRowWords>(q_bh + roff, f.qw);
+            load_words<kRowWords>(do_bh + roff, f.dw);
+            f.ld = *(const float2 *)(stats_bh + soff);
+        };
+        auto consume = [&](int j0, const RowFetch<kRowWords> &f) {
+            const float4 w = s_w[wave][j0 + slot];
             float qf[DC], dof[DC];
-            load_chunk<S, DC>(q_bh + roff, qf);
-            load_chunk<S, DC>(do_bh + roff, dof);
-            const float2 ld = *(const float2 *)(stats_bh + soff);
-            const float lse = ld.x, delta = ld.y;
-            __builtin_amdgcn_sched_barrier(0);     // all four gathers in flight before the arithmetic starts
+            widen_words<S, DC>(f.qw, qf);
+            widen_words<S, DC>(f.dw, dof);
+            const float lse = f.ld.x, delta = f.ld.y;
             float dot = 0.f, dp = 0.f;
             if constexpr (kPacked) {
                 // q . k~ = sum_t w_t (q . K_t): packed dot products on the raw 16-bit pairs
-                uint32_t qp[DC / 2], dop[DC / 2];
-                load_packed<S, DC>(q_bh + roff, qp);
-                load_packed<S, DC>(do_bh + roff, dop);
-                dot = fmaf(w.x, packed_dot<S, DC>(qp, ktp[0]),
-                           fmaf(w.y, packed_dot<S, DC>(qp, ktp[1]),
-                                fmaf(w.z, packed_dot<S, DC>(qp, ktp[2]), w.w * packed_dot<S, DC>(qp, ktp[3]))));
-                dp = fmaf(w.x, packed_dot<S, DC>(dop, vtp[0]),
-                          fmaf(w.y, packed_dot<S, DC>(dop, vtp[1]),
-                               fmaf(w.z, packed_dot<S, DC>(dop, vtp[2]), w.w * packed_dot<S, DC>(dop, vtp[3]))));
+                dot = fmaf(w.x, packed_dot<S, DC>(f.qw, ktp[0]),
+                           fmaf(w.y, packed_dot<S, DC>(f.qw, ktp[1]),
+                                fmaf(w.z, packed_dot<S, DC>(f.qw, ktp[2]), w.w * packed_dot<S, DC>(f.qw, ktp[3]))));
+                dp = fmaf(w.x, packed_dot<S, DC>(f.dw, vtp[0]),
+                          fmaf(w.y, packed_dot<S, DC>(f.dw, vtp[1]),
+                               fmaf(w.z, packed_dot<S, DC>(f.dw, vtp[2]), w.w * packed_dot<S, DC>(f.dw, vtp[3]))));
             } else {
                 // w = (fx, fy, fx*fy, live)
 #pragma unroll
@@ -359,20 +455,49 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? 5 : (S::kBytes == 2 ? 
             float p_n = __builtin_amdgcn_exp2f(dot * qscale - lse);
             if constexpr (!kPacked) p_n *= w.w;                    // entries past the end of the list
             const float dss = p_n * (dp - delta) * dm.sm_scale;
-            // packed: per-tap weights; fp32: the moments 1, fx, fy, fx*fy
-            const float ck[4] = { kPacked ? w.x * dss : dss, kPacked ? w.y * dss : w.x * dss,
-                                  kPacked ? w.z * dss : w.y * dss, kPacked ? w.w * dss : w.z * dss };
-            const float cv[4] = { kPacked ? w.x * p_n : p_n, kPacked ? w.y * p_n : w.x * p_n,
-                                  kPacked ? w.z * p_n : w.y * p_n, kPacked ? w.w * p_n : w.z * p_n };
-#pragma unroll
-            for (int tpi = 0; tpi < 4; ++tpi) {
-#pragma unroll
-                for (int d = 0; d < DC; ++d) {
-                    aK[tpi][d] = fmaf(ck[tpi], qf[d], aK[tpi][d]);
-                    aV[tpi][d] = fmaf(cv[tpi], dof[d], aV[tpi][d]);
-                }
+            // this lane's row of the update: packed: the weight of tap (lane & 3); fp32: the moment
+            // (1, fx, fy, fx*fy)[lane & 3]. The four lanes of a block sit in one slot (G is a multiple of 4),
+            // so they share the sample and supply its four coefficients between them.
+            float fxs, fys;
+            if constexpr (kPacked) {
+                const float2 ff = s_f[wave][j0 + slot];
+                fxs = ff.x;
+                fys = ff.y;
+            } else {
+                fxs = w.x;
+                fys = w.y;
             }
+            float cl = fmaf(fxs, row_sx, row_ox) * fmaf(fys, row_sy, row_oy);
+            if constexpr (kPacked) cl = (fys == fys) ? cl : 0.0f;       // dead entry: p_n is finite, the row is 0
+            const float ck = cl * dss, cv = cl * p_n;
+#pragma unroll
+            for (int d = 0; d < DC; ++d) {
+                mK[d] = block_outer_fma(ck, qf[d], mK[d]);
+                mV[d] = block_outer_fma(cv, dof[d], mV[d]);
+            }
+        };
+        // Trips go in pairs, and every request is unconditional: entries past the end of the list (up to the
+        // end of the 64-entry block) are dead ones with valid row offsets and zero weights, and the last
+        // request of a block wraps to entry 0 and is never used. (A request under a branch makes the compiler
+        // wait for all outstanding loads at the join, which undoes the overlap.)
+        static_assert(kWave % (2 * NS) == 0, "a block of 64 entries is a whole number of trip pairs");
+        RowFetch<kRowWords> fa, fb;
+        issue(0, fa);
+        for (int j0 = 0; j0 < cnt; j0 += 2 * NS) {
+            issue(j0 + NS, fb);
+            __builtin_amdgcn_sched_barrier(0);         // (keeps the requests where they are written)
+            consume(j0, fa);
+            __builtin_amdgcn_sched_barrier(0);
+            issue((j0 + 2 * NS) & (kWave - 1), fa);
+            __builtin_amdgcn_sched_barrier(0);
+            consume(j0 + NS, fb);
+            __builtin_amdgcn_sched_barrier(0);
         }
+    }
+#pragma unroll
+    for (int tpi = 0; tpi < 4; ++tpi) {
+#pragma unroll
+        for (int d = 0; d < DC; ++d) { aK[tpi][d] = mK[d][tpi]; aV[tpi][d] = mV[d][tpi]; }
     }
     // sum the NS slots, then one flush per pixel of the cell
 #pragma unroll

@@ -325,6 +325,21 @@ __device__ __forceinline__ float group_sum(float x)
     return x;
 }
 
+// ------------------------------------------------------------------ 4x4 block matrix instructions
+// gfx950 has matrix instructions that treat a wave as 16 independent blocks of 4 lanes. Measured here, one of
+// them takes the issue port for about 1.3 times as long as one vector multiply-add and cannot overlap with
+// vector instructions of the same SIMD, but does the work of four: used as a wide multiply-add, not as a
+// GEMM (every sample has its own operands).
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+
+// v_mfma_f32_4x4x1_16b_f32: for every block b of four lanes, acc(lane 4b+j)[i] += a(lane 4b+i) * x(lane 4b+j),
+// i, j = 0..3: a 4x4 outer product per block. Lane 4b+i supplies row coefficient i, every lane its own x.
+__device__ __forceinline__ floatx4 block_outer_fma(float a, float x, floatx4 acc)
+{
+    return __builtin_amdgcn_mfma_f32_4x4x1f32(a, x, acc, 0, 0, 0);
+}
+
 // Orders this wave's LDS writes before its later LDS reads (and the reverse):
 // waits for the wave's outstanding LDS traffic and stops the compiler from
 // moving LDS accesses across. No workgroup barrier is involved.

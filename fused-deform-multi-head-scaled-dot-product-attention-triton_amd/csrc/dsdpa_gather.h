@@ -42,11 +42,14 @@ __device__ __forceinline__ RowCtx decode_row(int work, const Dims &dm, int D)
     return c;
 }
 
-// Each lane builds the descriptor of sample c0+lane and parks it in this wave's LDS slice.
-template <int D>
+// Each lane builds the descriptor of sample c0+lane and parks it in this wave's LDS slice: the four
+// weights and the four taps' BYTE offsets from plane (b, view 0, h), unsigned 32-bit (one batch item of a
+// tensor stays below 2^30 elements, so below 2^32 bytes). With a wave-uniform base pointer a gather is then
+// "scalar base + 32-bit lane offset", one add per tap instead of 64-bit address arithmetic.
+template <int D, int BYTES>
 __device__ __forceinline__ void stage_descriptors(const float2 *__restrict__ coords, const RowCtx &rc,
                                                   const Dims &dm, int c0, int lane,
-                                                  float4 *s_w, int4 *s_e)
+                                                  float4 *s_w, uint4 *s_e)
 {
     int n = c0 + lane;
     bool valid = n < dm.N;
@@ -55,23 +58,30 @@ __device__ __forceinline__ void stage_descriptors(const float2 *__restrict__ coo
     Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
     int ebase = (nc / dm.P) * rc.view_stride;
     float4 w = valid ? make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]) : make_float4(0.f, 0.f, 0.f, 0.f);
-    int4 e = make_int4(ebase + tp.pix[0] * D, ebase + tp.pix[1] * D, ebase + tp.pix[2] * D, ebase + tp.pix[3] * D);
+    uint4 e = make_uint4((unsigned)(ebase + tp.pix[0] * D) * BYTES, (unsigned)(ebase + tp.pix[1] * D) * BYTES,
+                         (unsigned)(ebase + tp.pix[2] * D) * BYTES, (unsigned)(ebase + tp.pix[3] * D) * BYTES);
     wave_lds_sync();          // the previous chunk's readers are done
     s_w[lane] = w;
     s_e[lane] = e;
     wave_lds_sync();
 }
 
-// Bilinear blend of the four taps of one sample, this lane's DC elements.
+__device__ __forceinline__ uint4 lane_offsets(const uint4 &e, unsigned lane_byte)
+{
+    return make_uint4(e.x + lane_byte, e.y + lane_byte, e.z + lane_byte, e.w + lane_byte);
+}
+
+// Bilinear blend of the four taps of one sample, this lane's DC elements. `e`: the taps' byte offsets from
+// the (uniform) base, this lane's part of the row included.
 template <typename S, int DC>
-__device__ __forceinline__ void blend_taps(const char *__restrict__ base, const int4 &e, const float4 &w,
-                                           int lane_elem, float (&dst)[DC])
+__device__ __forceinline__ void blend_taps(const char *__restrict__ base, const uint4 &e, const float4 &w,
+                                           float (&dst)[DC])
 {
     float t0[DC], t1[DC], t2[DC], t3[DC];
-    load_chunk<S, DC>(base + (size_t)(e.x + lane_elem) * S::kBytes, t0);
-    load_chunk<S, DC>(base + (size_t)(e.y + lane_elem) * S::kBytes, t1);
-    load_chunk<S, DC>(base + (size_t)(e.z + lane_elem) * S::kBytes, t2);
-    load_chunk<S, DC>(base + (size_t)(e.w + lane_elem) * S::kBytes, t3);
+    load_chunk<S, DC>(base + e.x, t0);
+    load_chunk<S, DC>(base + e.y, t1);
+    load_chunk<S, DC>(base + e.z, t2);
+    load_chunk<S, DC>(base + e.w, t3);
 #pragma unroll
     for (int d = 0; d < DC; ++d)
         dst[d] = fmaf(w.x, t0[d], fmaf(w.y, t1[d], fmaf(w.z, t2[d], w.w * t3[d])));
@@ -79,14 +89,14 @@ __device__ __forceinline__ void blend_taps(const char *__restrict__ base, const 
 
 // acc += sum_t c_t * tap_t for the four taps of one sample (no separate blend).
 template <typename S, int DC>
-__device__ __forceinline__ void accumulate_taps(const char *__restrict__ base, const int4 &e, const float4 &c,
-                                                int lane_elem, float (&acc)[DC])
+__device__ __forceinline__ void accumulate_taps(const char *__restrict__ base, const uint4 &e, const float4 &c,
+                                                float (&acc)[DC])
 {
     float t0[DC], t1[DC], t2[DC], t3[DC];
-    load_chunk<S, DC>(base + (size_t)(e.x + lane_elem) * S::kBytes, t0);
-    load_chunk<S, DC>(base + (size_t)(e.y + lane_elem) * S::kBytes, t1);
-    load_chunk<S, DC>(base + (size_t)(e.z + lane_elem) * S::kBytes, t2);
-    load_chunk<S, DC>(base + (size_t)(e.w + lane_elem) * S::kBytes, t3);
+    load_chunk<S, DC>(base + e.x, t0);
+    load_chunk<S, DC>(base + e.y, t1);
+    load_chunk<S, DC>(base + e.z, t2);
+    load_chunk<S, DC>(base + e.w, t3);
 #pragma unroll
     for (int d = 0; d < DC; ++d)
         acc[d] = fmaf(c.x, t0[d], fmaf(c.y, t1[d], fmaf(c.z, t2[d], fmaf(c.w, t3[d], acc[d]))));
@@ -103,13 +113,14 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
     constexpr int ITS = G;           // slot iterations per 64-sample chunk
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
     __shared__ float4 s_w[kGatherWaves][kWave];
-    __shared__ int4 s_e[kGatherWaves][kWave];
+    __shared__ uint4 s_e[kGatherWaves][kWave];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
     if (work >= dm.rows) return;
     const RowCtx rc = decode_row(work, dm, D);
     const int g = lane % G, slot = lane / G, lane_elem = g * DC;
+    const unsigned lane_byte = (unsigned)lane_elem * S::kBytes;
     const char *kb = (const char *)k_ + rc.kv_base * S::kBytes;
     const char *vb = (const char *)v_ + rc.kv_base * S::kBytes;
     const float2 *coords = (const float2 *)coords_;
@@ -133,7 +144,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
     for (int d = 0; d < DC; ++d) acc[d] = 0.f;
 
     for (int c0 = 0; c0 < dm.N; c0 += kWave) {
-        stage_descriptors<D>(coords, rc, dm, c0, lane, s_w[wave], s_e[wave]);
+        stage_descriptors<D, S::kBytes>(coords, rc, dm, c0, lane, s_w[wave], s_e[wave]);
         const int cnt = min(kWave, dm.N - c0);
         float sv[ITS];
         float mc = kNegBig;
@@ -143,16 +154,13 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
             if (it * NS < cnt) {
                 int j = it * NS + slot;
                 float4 w = s_w[wave][j];
-                int4 e = s_e[wave][j];
+                const uint4 e = lane_offsets(s_e[wave][j], lane_byte);
                 float dot = 0.f;
                 if constexpr (kPacked) {
-                    dot = qscale * tap_dot16<S, DC>(kb + (size_t)(e.x + lane_elem) * S::kBytes,
-                                                    kb + (size_t)(e.y + lane_elem) * S::kBytes,
-                                                    kb + (size_t)(e.z + lane_elem) * S::kBytes,
-                                                    kb + (size_t)(e.w + lane_elem) * S::kBytes, w, qp);
+                    dot = qscale * tap_dot16<S, DC>(kb + e.x, kb + e.y, kb + e.z, kb + e.w, w, qp);
                 } else {
                     float kk[DC];
-                    blend_taps<S, DC>(kb, e, w, lane_elem, kk);
+                    blend_taps<S, DC>(kb, e, w, kk);
 #pragma unroll
                     for (int d = 0; d < DC; ++d) dot = fmaf(qf[d], kk[d], dot);
                 }
@@ -174,9 +182,9 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
                 float p = (j < cnt) ? __builtin_amdgcn_exp2f(sv[it] - m) : 0.f;
                 lsum += p;
                 float4 w = s_w[wave][j];
-                int4 e = s_e[wave][j];
+                const uint4 e = lane_offsets(s_e[wave][j], lane_byte);
                 float4 c = make_float4(p * w.x, p * w.y, p * w.z, p * w.w);
-                accumulate_taps<S, DC>(vb, e, c, lane_elem, acc);
+                accumulate_taps<S, DC>(vb, e, c, acc);
             }
         }
     }
@@ -220,13 +228,14 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_gather_kernel(
     constexpr int ITS = G;
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
     __shared__ float4 s_w[kGatherWaves][kWave];
-    __shared__ int4 s_e[kGatherWaves][kWave];
+    __shared__ uint4 s_e[kGatherWaves][kWave];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
     if (work >= dm.rows) return;
     const RowCtx rc = decode_row(work, dm, D);
     const int g = lane % G, slot = lane / G, lane_elem = g * DC;
+    const unsigned lane_byte = (unsigned)lane_elem * S::kBytes;
     const char *kb = (const char *)k_ + rc.kv_base * S::kBytes;
     const char *vb = (const char *)v_ + rc.kv_base * S::kBytes;
     float *dkb = dk_acc + rc.kv_base + lane_elem;
@@ -251,17 +260,18 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_gather_kernel(
     for (int d = 0; d < DC; ++d) dqa[d] = 0.f;
 
     for (int c0 = 0; c0 < dm.N; c0 += kWave) {
-        stage_descriptors<D>(coords, rc, dm, c0, lane, s_w[wave], s_e[wave]);
+        stage_descriptors<D, S::kBytes>(coords, rc, dm, c0, lane, s_w[wave], s_e[wave]);
         const int cnt = min(kWave, dm.N - c0);
 #pragma unroll 2
         for (int it = 0; it < ITS; ++it) {
             if (it * NS < cnt) {
                 int j = it * NS + slot;
                 float4 w = s_w[wave][j];
-                int4 e = s_e[wave][j];
+                const uint4 eb = s_e[wave][j];
+                const uint4 e = lane_offsets(eb, lane_byte);
                 float kk[DC], vv[DC];
-                blend_taps<S, DC>(kb, e, w, lane_elem, kk);
-                blend_taps<S, DC>(vb, e, w, lane_elem, vv);
+                blend_taps<S, DC>(kb, e, w, kk);
+                blend_taps<S, DC>(vb, e, w, vv);
                 float dot = 0.f, dp = 0.f;
 #pragma unroll
                 for (int d = 0; d < DC; ++d) {
@@ -276,7 +286,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_gather_kernel(
                 for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
                 const float dss = ds * dm.sm_scale;
                 const float wt[4] = { w.x, w.y, w.z, w.w };
-                const int et[4] = { e.x, e.y, e.z, e.w };
+                const unsigned et[4] = { eb.x / S::kBytes, eb.y / S::kBytes, eb.z / S::kBytes, eb.w / S::kBytes };
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     if (wt[t] != 0.f) {
@@ -327,7 +337,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     constexpr int ITS = G;
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
     __shared__ float4 s_w[kGatherWaves][kWave];
-    __shared__ int4 s_e[kGatherWaves][kWave];
+    __shared__ uint4 s_e[kGatherWaves][kWave];
     __shared__ float4 s_gx[CG ? kGatherWaves : 1][kWave];
     __shared__ float4 s_gy[CG ? kGatherWaves : 1][kWave];
 
@@ -336,6 +346,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     if (work >= dm.rows) return;
     const RowCtx rc = decode_row(work, dm, D);
     const int g = lane % G, slot = lane / G, lane_elem = g * DC;
+    const unsigned lane_byte = (unsigned)lane_elem * S::kBytes;
     const char *kb = (const char *)k_ + rc.kv_base * S::kBytes;
     const char *vb = (const char *)v_ + rc.kv_base * S::kBytes;
     const float2 *coords = (const float2 *)coords_;
@@ -361,7 +372,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     for (int d = 0; d < DC; ++d) dqa[d] = 0.f;
 
     for (int c0 = 0; c0 < dm.N; c0 += kWave) {
-        stage_descriptors<D>(coords, rc, dm, c0, lane, s_w[wave], s_e[wave]);
+        stage_descriptors<D, S::kBytes>(coords, rc, dm, c0, lane, s_w[wave], s_e[wave]);
         if constexpr (CG) {
             // (stage_descriptors ends with a wave-level LDS sync; these two arrays are read after the
             // next one, and their previous readers finished before the sync at its start)
@@ -378,18 +389,18 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
             if (it * NS < cnt) {
                 int j = it * NS + slot;
                 float4 w = s_w[wave][j];
-                int4 e = s_e[wave][j];
+                const uint4 e = lane_offsets(s_e[wave][j], lane_byte);
                 float kk[DC];
                 float dot = 0.f, dp = 0.f;
                 if constexpr (CG) {
                     float t[4][DC], u[4][DC];
-                    const int eo[4] = { e.x, e.y, e.z, e.w };
+                    const unsigned eo[4] = { e.x, e.y, e.z, e.w };
                     const float wt[4] = { w.x, w.y, w.z, w.w };
                     float dk_t[4], dv_t[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        load_chunk<S, DC>(kb + (size_t)(eo[i] + lane_elem) * S::kBytes, t[i]);
-                        load_chunk<S, DC>(vb + (size_t)(eo[i] + lane_elem) * S::kBytes, u[i]);
+                        load_chunk<S, DC>(kb + eo[i], t[i]);
+                        load_chunk<S, DC>(vb + eo[i], u[i]);
                     }
 #pragma unroll
                     for (int d = 0; d < DC; ++d) kk[d] = 0.f;
@@ -427,18 +438,15 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                     }
                     continue;
                 }
-                blend_taps<S, DC>(kb, e, w, lane_elem, kk);
+                blend_taps<S, DC>(kb, e, w, kk);
 #pragma unroll
                 for (int d = 0; d < DC; ++d) dot = fmaf(qf[d], kk[d], dot);
                 if constexpr (kPacked) {
                     // dout . v~ needs no widened v~: four packed dot products on the raw taps
-                    dp = tap_dot16<S, DC>(vb + (size_t)(e.x + lane_elem) * S::kBytes,
-                                          vb + (size_t)(e.y + lane_elem) * S::kBytes,
-                                          vb + (size_t)(e.z + lane_elem) * S::kBytes,
-                                          vb + (size_t)(e.w + lane_elem) * S::kBytes, w, dop);
+                    dp = tap_dot16<S, DC>(vb + e.x, vb + e.y, vb + e.z, vb + e.w, w, dop);
                 } else {
                     float vv[DC];
-                    blend_taps<S, DC>(vb, e, w, lane_elem, vv);
+                    blend_taps<S, DC>(vb, e, w, vv);
 #pragma unroll
                     for (int d = 0; d < DC; ++d) dp = fmaf(dof[d], vv[d], dp);
                 }

@@ -44,12 +44,12 @@ __global__ __launch_bounds__(kTileWaves *kWave) void bwd_dkdv_tile_kernel(
     double *tileK = reinterpret_cast<double *>(smem);
     double *tileV = tileK + tile_elems;
     float4 *s_w_all = reinterpret_cast<float4 *>(tileV + tile_elems);
-    int4 *s_e_all = reinterpret_cast<int4 *>(s_w_all + kTileWaves * kWave);
+    uint4 *s_e_all = reinterpret_cast<uint4 *>(s_w_all + kTileWaves * kWave);
     int *s_loc_all = reinterpret_cast<int *>(s_e_all + kTileWaves * kWave);
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     float4 *s_w = s_w_all + wave * kWave;
-    int4 *s_e = s_e_all + wave * kWave;
+    uint4 *s_e = s_e_all + wave * kWave;
     int *s_loc = s_loc_all + wave * kWave;
 
     // block -> (plane, tile, query slice); plane-major so that an XCD's L2 keeps few planes
@@ -102,7 +102,8 @@ __global__ __launch_bounds__(kTileWaves *kWave) void bwd_dkdv_tile_kernel(
             wave_lds_sync();
             if (mine) {
                 s_w[pos] = make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]);
-                s_e[pos] = make_int4(tp.pix[0] * D, tp.pix[1] * D, tp.pix[2] * D, tp.pix[3] * D);
+                s_e[pos] = make_uint4((unsigned)(tp.pix[0] * D) * S::kBytes, (unsigned)(tp.pix[1] * D) * S::kBytes,
+                                      (unsigned)(tp.pix[2] * D) * S::kBytes, (unsigned)(tp.pix[3] * D) * S::kBytes);
                 s_loc[pos] = ((tp.y0 - ya) * tg.lw + (tp.x0 - xa)) * D;   // tile-local offset of tap 00
             }
             wave_lds_sync();
@@ -120,11 +121,11 @@ __global__ __launch_bounds__(kTileWaves *kWave) void bwd_dkdv_tile_kernel(
                 const bool live = j < cnt;
                 const int jj = live ? j : cnt - 1;
                 float4 w = s_w[jj];
-                int4 e = s_e[jj];
+                const uint4 e = lane_offsets(s_e[jj], (unsigned)lane_elem * S::kBytes);
                 const int loc = s_loc[jj];
                 float kk[DC], vv[DC];
-                blend_taps<S, DC>(kb, e, w, lane_elem, kk);
-                blend_taps<S, DC>(vb, e, w, lane_elem, vv);
+                blend_taps<S, DC>(kb, e, w, kk);
+                blend_taps<S, DC>(vb, e, w, vv);
                 float dot = 0.f, dp = 0.f;
 #pragma unroll
                 for (int d = 0; d < DC; ++d) {
