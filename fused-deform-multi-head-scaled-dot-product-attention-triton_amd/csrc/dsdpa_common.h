@@ -4,6 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace dsdpa {
 
@@ -338,6 +339,34 @@ typedef short shortx4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ floatx4 block_outer_fma(float a, float x, floatx4 acc)
 {
     return __builtin_amdgcn_mfma_f32_4x4x1f32(a, x, acc, 0, 0, 0);
+}
+
+// ------------------------------------------------------------------ reductions over the whole wave
+// Every lane ends up with the result. Five steps stay in the vector ALU (DPP / swizzle), the last is a shuffle.
+template <typename T, typename Op>
+__device__ __forceinline__ T wave_all(T x, Op op)
+{
+    static_assert(sizeof(T) == 4, "32-bit values");
+    auto dpp = [](T v, auto ctrl) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xf, 0xf, false));
+    };
+    x = op(x, dpp(x, std::integral_constant<int, 0xB1>{}));      // quad_perm [1,0,3,2]
+    x = op(x, dpp(x, std::integral_constant<int, 0x4E>{}));      // quad_perm [2,3,0,1]
+    x = op(x, dpp(x, std::integral_constant<int, 0x141>{}));     // row_half_mirror
+    x = op(x, dpp(x, std::integral_constant<int, 0x140>{}));     // row_mirror
+    x = op(x, __builtin_bit_cast(T, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x401F)));   // lane ^ 16
+    x = op(x, __builtin_bit_cast(T, __shfl_xor(__builtin_bit_cast(int, x), 32, kWave)));
+    return x;
+}
+__device__ __forceinline__ float wave_max(float x) { return wave_all(x, [](float a, float b) { return fmaxf(a, b); }); }
+__device__ __forceinline__ float wave_sum(float x) { return wave_all(x, [](float a, float b) { return a + b; }); }
+// two unsigned 16-bit fields per word, minimum taken field by field
+__device__ __forceinline__ uint32_t wave_min_u16x2(uint32_t x)
+{
+    return wave_all(x, [](uint32_t a, uint32_t b) {
+        const uint32_t lo = min(a & 0xffffu, b & 0xffffu), hi = min(a >> 16, b >> 16);
+        return lo | (hi << 16);
+    });
 }
 
 // Orders this wave's LDS writes before its later LDS reads (and the reverse):

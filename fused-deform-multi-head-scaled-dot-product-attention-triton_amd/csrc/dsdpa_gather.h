@@ -47,6 +47,20 @@ __device__ __forceinline__ RowCtx decode_row(int work, const Dims &dm, int D)
 // tensor stays below 2^30 elements, so below 2^32 bytes). With a wave-uniform base pointer a gather is then
 // "scalar base + 32-bit lane offset", one add per tap instead of 64-bit address arithmetic.
 template <int D, int BYTES>
+__device__ __forceinline__ void park_descriptors(const Taps &tp, bool valid, int nc, const RowCtx &rc,
+                                                 const Dims &dm, int lane, float4 *s_w, uint4 *s_e)
+{
+    int ebase = (nc / dm.P) * rc.view_stride;
+    float4 w = valid ? make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]) : make_float4(0.f, 0.f, 0.f, 0.f);
+    uint4 e = make_uint4((unsigned)(ebase + tp.pix[0] * D) * BYTES, (unsigned)(ebase + tp.pix[1] * D) * BYTES,
+                         (unsigned)(ebase + tp.pix[2] * D) * BYTES, (unsigned)(ebase + tp.pix[3] * D) * BYTES);
+    wave_lds_sync();          // the previous chunk's readers are done
+    s_w[lane] = w;
+    s_e[lane] = e;
+    wave_lds_sync();
+}
+
+template <int D, int BYTES>
 __device__ __forceinline__ void stage_descriptors(const float2 *__restrict__ coords, const RowCtx &rc,
                                                   const Dims &dm, int c0, int lane,
                                                   float4 *s_w, uint4 *s_e)
@@ -56,14 +70,165 @@ __device__ __forceinline__ void stage_descriptors(const float2 *__restrict__ coo
     int nc = valid ? n : dm.N - 1;
     float2 xy = coords[rc.crow + nc];
     Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
-    int ebase = (nc / dm.P) * rc.view_stride;
-    float4 w = valid ? make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]) : make_float4(0.f, 0.f, 0.f, 0.f);
-    uint4 e = make_uint4((unsigned)(ebase + tp.pix[0] * D) * BYTES, (unsigned)(ebase + tp.pix[1] * D) * BYTES,
-                         (unsigned)(ebase + tp.pix[2] * D) * BYTES, (unsigned)(ebase + tp.pix[3] * D) * BYTES);
-    wave_lds_sync();          // the previous chunk's readers are done
-    s_w[lane] = w;
-    s_e[lane] = e;
-    wave_lds_sync();
+    park_descriptors<D, BYTES>(tp, valid, nc, rc, dm, lane, s_w, s_e);
+}
+
+// ------------------------------------------------------------------ window mode
+// When the samples of a chunk (up to 64 samples of one query row, all in one key view) fall into a small
+// window of the image -- deformable sampling around a reference point does -- the chunk is worked on per
+// PIXEL of the window instead of per tap: one q.K[pixel] dot product per pixel, each sample's logit blended
+// from four of those scalars, the softmax weights times the bilinear weights scattered into one
+// coefficient per pixel, and one multiply-add of V[pixel] per pixel. A window of w x h pixels costs w*h
+// rows of K and of V, read as contiguous runs, where the taps cost 4 per sample: about 120 against 256 for
+// 64 samples with a standard deviation of two pixels. Chosen per chunk, from the bounding box of its taps.
+//
+// The window is walked in UNITS of four pixels that are neighbours in a row (one 16-byte load per pixel
+// at constant offsets from the unit's first): its rows are padded to a whole number of units, and it is
+// moved left where that would cross the right edge of the image, so every pixel of every unit lies
+// inside the image. Tables are indexed by entry = (row - ymin) * 4 * nu + (column - xmin).
+constexpr int kWinUnits = 64;                  // units per window: the tables of a wave hold 256 pixels
+
+struct Window { int xmin, ymin, nu, nunits; };     // wave-uniform; nu = units per window row
+
+// Bounding box of the clamped tap pixels of the lanes with `counted` set (a live sample with a tap inside the
+// image), as padded units. Needs Wimg, Himg < 65536. nunits = 0: no window (the image is narrower than
+// the padded rows).
+__device__ __forceinline__ Window chunk_window(const Taps &tp, bool counted, int Wimg, int Himg)
+{
+    const int cx0 = min(max(tp.x0, 0), Wimg - 1), cx1 = min(max(tp.x0 + 1, 0), Wimg - 1);
+    const int cy0 = min(max(tp.y0, 0), Himg - 1), cy1 = min(max(tp.y0 + 1, 0), Himg - 1);
+    uint32_t lo = counted ? (uint32_t)cx0 | ((uint32_t)cy0 << 16) : 0xffffffffu;
+    uint32_t hi = counted ? (uint32_t)(0xffff - cx1) | ((uint32_t)(0xffff - cy1) << 16) : 0xffffffffu;
+    lo = __builtin_amdgcn_readfirstlane(wave_min_u16x2(lo));
+    hi = __builtin_amdgcn_readfirstlane(wave_min_u16x2(hi));
+    Window w;
+    int xmax = 0, ymax = 0;
+    w.xmin = 0;
+    w.ymin = 0;
+    if (lo != 0xffffffffu) {                   // else: no sample has a tap inside the image; any one unit will do
+        w.xmin = (int)(lo & 0xffffu);
+        w.ymin = (int)(lo >> 16);
+        xmax = 0xffff - (int)(hi & 0xffffu);
+        ymax = 0xffff - (int)(hi >> 16);
+    }
+    w.nu = (xmax - w.xmin + 4) >> 2;
+    w.xmin = min(w.xmin, Wimg - 4 * w.nu);
+    w.nunits = w.xmin >= 0 ? w.nu * (ymax - w.ymin + 1) : 0;
+    return w;
+}
+
+// The four taps' entries in the window's tables (clamped pixels: inside the window whenever the sample
+// counts; the others carry weight 0 and are only kept inside the tables).
+__device__ __forceinline__ int4 window_entries(const Taps &tp, const Window &win, int Wimg, int Himg)
+{
+    const int cx0 = min(max(tp.x0, 0), Wimg - 1) - win.xmin, cx1 = min(max(tp.x0 + 1, 0), Wimg - 1) - win.xmin;
+    const int cy0 = (min(max(tp.y0, 0), Himg - 1) - win.ymin) * 4 * win.nu;
+    const int cy1 = (min(max(tp.y0 + 1, 0), Himg - 1) - win.ymin) * 4 * win.nu;
+    const int last = 4 * win.nunits - 1;
+    return make_int4(min(max(cy0 + cx0, 0), last), min(max(cy0 + cx1, 0), last), min(max(cy1 + cx0, 0), last),
+                     min(max(cy1 + cx1, 0), last));
+}
+
+// The unit this slot takes in the step that starts at unit u0 (held at the last unit beyond the window),
+// and the byte offset of its first pixel from plane (b, view 0, h).
+template <int ROW_BYTES>
+__device__ __forceinline__ unsigned window_unit(const Window &win, int u0, int slot, int Wimg, unsigned view_byte,
+                                                float rnu, int *unit)
+{
+    const int u = min(u0 + slot, win.nunits - 1);
+    const int wy = (int)(((float)u + 0.5f) * rnu);             // u / nu: exact for these small numbers
+    const int wxu = u - wy * win.nu;
+    *unit = u;
+    return view_byte + (unsigned)((win.ymin + wy) * Wimg + win.xmin + 4 * wxu) * ROW_BYTES;
+}
+
+// q.K for the four pixels of this slot's unit, summed over the slot: t[4*unit + k].
+template <typename S, int DC, int G, int ROW_BYTES>
+__device__ __forceinline__ void window_dots(const char *__restrict__ base, unsigned off, const float (&xf)[DC],
+                                            const uint32_t *xp, float (&d)[4])
+{
+    if constexpr (S::kBytes == 2) {
+        uint32_t r[4][DC / 2];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) load_packed<S, DC>(base + off + k * ROW_BYTES, r[k]);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < DC / 2; ++i) {
+                if constexpr (S::kBf16)
+                    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(dsdpa_bf16x2, xp[i]),
+                                                          __builtin_bit_cast(dsdpa_bf16x2, r[k][i]), acc, false);
+                else
+                    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(dsdpa_f16x2, xp[i]),
+                                                 __builtin_bit_cast(dsdpa_f16x2, r[k][i]), acc, false);
+            }
+            d[k] = acc;
+        }
+    } else {
+        float r[4][DC];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) load_chunk<S, DC>(base + off + k * ROW_BYTES, r[k]);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            float acc = 0.f;
+#pragma unroll
+            for (int e = 0; e < DC; ++e) acc = fmaf(xf[e], r[k][e], acc);
+            d[k] = acc;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) d[k] = group_sum<G>(d[k]);
+}
+
+// 16-bit storage, at least four lanes per slot: the weighted sum of four rows on the 4x4x4 block matrix
+// instruction. For every block of four lanes it computes C[i][j] += sum_k A[i][k] * B[k][j]: k runs over the
+// four rows (pixels of a unit, or taps of a sample), j over the block's lanes, each with its own
+// elements of those rows, and the two rows of A that are used are the high and the low part of the four
+// coefficients (each a 16-bit float; together 16 bits of mantissa), so that acc[e][0] + acc[e][1] is the sum
+// with coefficients good to 2^-16. Lane 4b+i supplies row i of A: `coef` is this lane's row (the high parts
+// in lanes 4b, the low parts in lanes 4b+1, zero elsewhere). The rows come as packed pairs, which two byte
+// permutes per pair of rows turn into "four rows' values of one element".
+template <typename S, int DC>
+__device__ __forceinline__ void block_blend4(const uint32_t (&r)[4][DC / 2], shortx4 coef, floatx4 (&acc)[DC])
+{
+#pragma unroll
+    for (int i = 0; i < DC / 2; ++i) {
+        const uint32_t lo01 = __builtin_amdgcn_perm(r[1][i], r[0][i], 0x05040100u);
+        const uint32_t lo23 = __builtin_amdgcn_perm(r[3][i], r[2][i], 0x05040100u);
+        const uint32_t hi01 = __builtin_amdgcn_perm(r[1][i], r[0][i], 0x07060302u);
+        const uint32_t hi23 = __builtin_amdgcn_perm(r[3][i], r[2][i], 0x07060302u);
+        const uint2 be = make_uint2(lo01, lo23), bo = make_uint2(hi01, hi23);
+        if constexpr (S::kBf16) {
+            acc[2 * i] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(coef, __builtin_bit_cast(shortx4, be), acc[2 * i], 0, 0, 0);
+            acc[2 * i + 1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(coef, __builtin_bit_cast(shortx4, bo), acc[2 * i + 1], 0, 0, 0);
+        } else {
+            typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+            acc[2 * i] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, coef), __builtin_bit_cast(halfx4, be), acc[2 * i], 0, 0, 0);
+            acc[2 * i + 1] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, coef), __builtin_bit_cast(halfx4, bo), acc[2 * i + 1], 0, 0, 0);
+        }
+    }
+}
+
+// Four fp32 coefficients as the block matrix instruction's rows: .x, .y = the high parts (storage type, by
+// truncation for bf16 / rounding for fp16) as four packed 16-bit floats, .z, .w = the same of the remainders.
+template <typename S>
+__device__ __forceinline__ uint4 split_coefficients(float c0, float c1, float c2, float c3)
+{
+    if constexpr (S::kBf16) {
+        const uint32_t u0 = __float_as_uint(c0), u1 = __float_as_uint(c1), u2 = __float_as_uint(c2), u3 = __float_as_uint(c3);
+        const float l0 = c0 - __uint_as_float(u0 & 0xffff0000u), l1 = c1 - __uint_as_float(u1 & 0xffff0000u);
+        const float l2 = c2 - __uint_as_float(u2 & 0xffff0000u), l3 = c3 - __uint_as_float(u3 & 0xffff0000u);
+        return make_uint4(__builtin_amdgcn_perm(u1, u0, 0x07060302u), __builtin_amdgcn_perm(u3, u2, 0x07060302u),
+                          __builtin_amdgcn_perm(__float_as_uint(l1), __float_as_uint(l0), 0x07060302u),
+                          __builtin_amdgcn_perm(__float_as_uint(l3), __float_as_uint(l2), 0x07060302u));
+    } else {
+        union { uint32_t u; _Float16 h[2]; } a, b, c, d;
+        a.h[0] = (_Float16)c0; a.h[1] = (_Float16)c1; b.h[0] = (_Float16)c2; b.h[1] = (_Float16)c3;
+        c.h[0] = (_Float16)(c0 - (float)a.h[0]); c.h[1] = (_Float16)(c1 - (float)a.h[1]);
+        d.h[0] = (_Float16)(c2 - (float)b.h[0]); d.h[1] = (_Float16)(c3 - (float)b.h[1]);
+        return make_uint4(a.u, b.u, c.u, d.u);
+    }
 }
 
 __device__ __forceinline__ uint4 lane_offsets(const uint4 &e, unsigned lane_byte)
@@ -103,7 +268,10 @@ __device__ __forceinline__ void accumulate_taps(const char *__restrict__ base, c
 }
 
 // ------------------------------------------------------------------ forward
-template <typename S, int D, int DC>
+// WIN: chunks are cut per key view (up to 64 samples of one view each) and every chunk may take the window
+// mode above; chosen by the host for P >= 64, where a view's samples fill whole chunks. Without WIN the
+// chunks are 64 consecutive samples of the row, whatever views they belong to, and always gather.
+template <typename S, int D, int DC, bool WIN>
 __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, void *__restrict__ out_, float *__restrict__ lse_, Dims dm)
@@ -114,6 +282,10 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
     __shared__ float4 s_w[kGatherWaves][kWave];
     __shared__ uint4 s_e[kGatherWaves][kWave];
+    constexpr int kTab = WIN ? kGatherWaves : 1, kTabUnits = WIN ? kWinUnits : 1;
+    __shared__ __attribute__((aligned(16))) float s_dot[kTab][4 * kTabUnits];      // window mode: q.K per pixel
+    __shared__ __attribute__((aligned(16))) double s_coef[kTab][4 * kTabUnits];    // window mode: coefficient of V per pixel
+    __shared__ uint4 s_blend[kTab][2 * kTabUnits];                                  // ... per unit, as the V pass reads them
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
@@ -143,9 +315,117 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
 #pragma unroll
     for (int d = 0; d < DC; ++d) acc[d] = 0.f;
 
-    for (int c0 = 0; c0 < dm.N; c0 += kWave) {
-        stage_descriptors<D, S::kBytes>(coords, rc, dm, c0, lane, s_w[wave], s_e[wave]);
-        const int cnt = min(kWave, dm.N - c0);
+    const bool window_ok = WIN && dm.Wimg < 65536 && dm.Himg < 65536;
+    const int view_chunks = (dm.P + kWave - 1) / kWave;
+    const int nchunks = WIN ? dm.V * view_chunks : (dm.N + kWave - 1) / kWave;
+    int next_view = 0, next_p0 = 0;                      // WIN: key view and first sample in it of the next chunk
+    for (int ci = 0; ci < nchunks; ++ci) {
+        const int s2c = next_view, p0 = next_p0;         // WIN: this chunk's
+        const int c0 = WIN ? s2c * dm.P + p0 : ci * kWave;
+        const int cnt = WIN ? min(kWave, dm.P - p0) : min(kWave, dm.N - c0);
+        if (WIN) {
+            next_p0 += kWave;
+            if (next_p0 >= dm.P) { next_p0 = 0; ++next_view; }
+        }
+        // this lane's sample of the chunk
+        const bool live = lane < cnt;
+        const int nc = c0 + (live ? lane : cnt - 1);
+        const float2 xy = coords[rc.crow + nc];
+        const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
+        if (window_ok) {                                 // (the chunk lies in one key view)
+            const bool counted = live && ((tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f));
+            const Window win = chunk_window(tp, counted, dm.Wimg, dm.Himg);
+            if (win.nunits > 0 && win.nunits <= kWinUnits && 4 * win.nunits <= 3 * cnt) {
+                constexpr int kRow = D * S::kBytes;
+                constexpr bool kBlock = kPacked && G >= 4;         // V rows blended by the block matrix instruction
+                float *tS = s_dot[wave];
+                double *tA = s_coef[wave];
+                uint4 *tC = s_blend[wave];
+                const float rnu = 1.0f / (float)win.nu;
+                const unsigned view_byte = (unsigned)s2c * (unsigned)rc.view_stride * S::kBytes;
+                // one q.K dot product per pixel of the window
+                for (int u0 = 0; u0 < win.nunits; u0 += NS) {
+                    int unit;
+                    const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                    float d4[4];
+                    window_dots<S, DC, G, kRow>(kb, off, qf, qp, d4);
+                    if (g == 0) *reinterpret_cast<float4 *>(tS + 4 * unit) = make_float4(d4[0], d4[1], d4[2], d4[3]);
+                }
+                for (int e = lane; e < 4 * win.nunits; e += kWave) tA[e] = 0.0;
+                wave_lds_sync();
+                // the samples, one per lane: logit from four of the pixel scalars, then the softmax bookkeeping
+                // of the chunk with ONE running maximum for all slots (they are brought to a common one first)
+                const int4 te = window_entries(tp, win, dm.Wimg, dm.Himg);
+                const float w0 = live ? tp.w[0] : 0.f, w1 = live ? tp.w[1] : 0.f;
+                const float w2 = live ? tp.w[2] : 0.f, w3 = live ? tp.w[3] : 0.f;
+                float logit = fmaf(w0, tS[te.x], fmaf(w1, tS[te.y], fmaf(w2, tS[te.z], w3 * tS[te.w])));
+                if constexpr (kPacked) logit *= qscale;
+                const float m_new = fmaxf(wave_max(m), wave_max(live ? logit : kNegBig));
+                const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+                m = m_new;
+                lsum *= alpha;
+#pragma unroll
+                for (int d = 0; d < DC; ++d) acc[d] *= alpha;
+                const float p = live ? __builtin_amdgcn_exp2f(logit - m_new) : 0.f;
+                const float psum = wave_sum(p);
+                if (slot == 0) lsum += psum;
+                // coefficient of every pixel: sum over the samples of p times the tap's bilinear weight
+                if (w0 != 0.f) atomicAdd(&tA[te.x], (double)(p * w0));
+                if (w1 != 0.f) atomicAdd(&tA[te.y], (double)(p * w1));
+                if (w2 != 0.f) atomicAdd(&tA[te.z], (double)(p * w2));
+                if (w3 != 0.f) atomicAdd(&tA[te.w], (double)(p * w3));
+                wave_lds_sync();
+                // the coefficients of each unit in the form the V pass wants them (one unit per lane)
+                if (lane < win.nunits) {
+                    const float c0 = (float)tA[4 * lane], c1 = (float)tA[4 * lane + 1];
+                    const float c2 = (float)tA[4 * lane + 2], c3 = (float)tA[4 * lane + 3];
+                    if constexpr (kBlock) {
+                        tC[2 * lane] = split_coefficients<S>(c0, c1, c2, c3);      // rows 0, 1: high and low parts
+                        tC[2 * lane + 1] = make_uint4(0u, 0u, 0u, 0u);             // rows 2, 3
+                    } else {
+                        tC[2 * lane] = make_uint4(__float_as_uint(c0), __float_as_uint(c1), __float_as_uint(c2), __float_as_uint(c3));
+                    }
+                }
+                wave_lds_sync();
+                // one weighted sum of V rows per unit
+                if constexpr (kBlock) {
+                    floatx4 macc[DC];
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) macc[d] = floatx4{0.f, 0.f, 0.f, 0.f};
+                    for (int u0 = 0; u0 < win.nunits; u0 += NS) {
+                        int unit;
+                        const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                        uint2 cf = reinterpret_cast<const uint2 *>(tC)[4 * unit + (lane & 3)];
+                        if (u0 + slot >= win.nunits) cf = make_uint2(0u, 0u);
+                        uint32_t r[4][DC / 2];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) load_packed<S, DC>(vb + off + k * kRow, r[k]);
+                        block_blend4<S, DC>(r, __builtin_bit_cast(shortx4, cf), macc);
+                    }
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) acc[d] += macc[d][0] + macc[d][1];
+                } else {
+                    for (int u0 = 0; u0 < win.nunits; u0 += NS) {
+                        int unit;
+                        const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                        uint4 cu = tC[2 * unit];
+                        if (u0 + slot >= win.nunits) cu = make_uint4(0u, 0u, 0u, 0u);
+                        const float cf[4] = { __uint_as_float(cu.x), __uint_as_float(cu.y), __uint_as_float(cu.z), __uint_as_float(cu.w) };
+                        float r[4][DC];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) load_chunk<S, DC>(vb + off + k * kRow, r[k]);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+#pragma unroll
+                            for (int d = 0; d < DC; ++d) acc[d] = fmaf(cf[k], r[k][d], acc[d]);
+                        }
+                    }
+                }
+                wave_lds_sync();
+                continue;
+            }
+        }
+        park_descriptors<D, S::kBytes>(tp, live, nc, rc, dm, lane, s_w[wave], s_e[wave]);
         float sv[ITS];
         float mc = kNegBig;
 #pragma unroll
@@ -325,7 +605,10 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_gather_kernel(
 // elements, combines them with the (slot-uniform) ds, p and tap derivatives and only the two results
 // are reduced over the slot. The H heads share the coordinates: float atomics into dcoords (zeroed by
 // the caller of the kernel).
-template <typename S, int D, int DC, bool CG>
+// WIN (never together with CG): chunks per key view and the window mode, as in the forward: q.K and dout.V
+// per pixel of the window, each sample's logit and dp blended from those scalars, ds times the bilinear weights
+// scattered into one coefficient per pixel, dq += coefficient * K[pixel] per pixel.
+template <typename S, int D, int DC, bool CG, bool WIN>
 __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
@@ -340,6 +623,12 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     __shared__ uint4 s_e[kGatherWaves][kWave];
     __shared__ float4 s_gx[CG ? kGatherWaves : 1][kWave];
     __shared__ float4 s_gy[CG ? kGatherWaves : 1][kWave];
+    static_assert(!(CG && WIN), "the window mode has no coordinate gradient");
+    constexpr int kTab = WIN ? kGatherWaves : 1, kTabUnits = WIN ? kWinUnits : 1;
+    __shared__ __attribute__((aligned(16))) float s_dotk[kTab][4 * kTabUnits];     // window mode: q.K per pixel
+    __shared__ __attribute__((aligned(16))) float s_dotv[kTab][4 * kTabUnits];     // window mode: dout.V per pixel
+    __shared__ __attribute__((aligned(16))) double s_coef[kTab][4 * kTabUnits];    // window mode: coefficient of K per pixel
+    __shared__ uint4 s_blend[kTab][2 * kTabUnits];                                  // ... per unit, as the last pass reads them
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
@@ -353,12 +642,13 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
 
     constexpr bool kPacked = S::kBytes == 2 && !CG;
     float qf[DC], dof[DC], of[DC];
-    uint32_t dop[kPacked ? DC / 2 : 1];
+    uint32_t dop[kPacked ? DC / 2 : 1], qp[kPacked && WIN ? DC / 2 : 1];
     const size_t roff = (rc.row * D + lane_elem) * S::kBytes;
     load_chunk<S, DC>((const char *)q_ + roff, qf);
     load_chunk<S, DC>((const char *)dout_ + roff, dof);
     load_chunk<S, DC>((const char *)out_ + roff, of);
     if constexpr (kPacked) load_packed<S, DC>((const char *)dout_ + roff, dop);
+    if constexpr (kPacked && WIN) load_packed<S, DC>((const char *)q_ + roff, qp);
     float delta = 0.f;
 #pragma unroll
     for (int d = 0; d < DC; ++d) delta = fmaf(dof[d], of[d], delta);
@@ -371,19 +661,119 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
 #pragma unroll
     for (int d = 0; d < DC; ++d) dqa[d] = 0.f;
 
-    for (int c0 = 0; c0 < dm.N; c0 += kWave) {
-        stage_descriptors<D, S::kBytes>(coords, rc, dm, c0, lane, s_w[wave], s_e[wave]);
+    const bool window_ok = WIN && dm.Wimg < 65536 && dm.Himg < 65536;
+    const int view_chunks = (dm.P + kWave - 1) / kWave;
+    const int nchunks = WIN ? dm.V * view_chunks : (dm.N + kWave - 1) / kWave;
+    int next_view = 0, next_p0 = 0;                      // WIN: key view and first sample in it of the next chunk
+    for (int ci = 0; ci < nchunks; ++ci) {
+        const int s2c = next_view, p0 = next_p0;         // WIN: this chunk's
+        const int c0 = WIN ? s2c * dm.P + p0 : ci * kWave;
+        const int cnt = WIN ? min(kWave, dm.P - p0) : min(kWave, dm.N - c0);
+        if (WIN) {
+            next_p0 += kWave;
+            if (next_p0 >= dm.P) { next_p0 = 0; ++next_view; }
+        }
+        // this lane's sample of the chunk
+        const bool live = lane < cnt;
+        const int nc = c0 + (live ? lane : cnt - 1);
+        const float2 xy0 = coords[rc.crow + nc];
+        const Taps tp = make_taps(xy0.x, xy0.y, dm.Wimg, dm.Himg);
+        if constexpr (WIN) {
+            const bool counted = live && ((tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f));
+            const Window win = window_ok ? chunk_window(tp, counted, dm.Wimg, dm.Himg) : Window{0, 0, 0, 0};
+            if (win.nunits > 0 && win.nunits <= kWinUnits && 4 * win.nunits <= 3 * cnt) {
+                constexpr int kRow = D * S::kBytes;
+                constexpr bool kBlock = kPacked && G >= 4;
+                float *tS = s_dotk[wave], *tT = s_dotv[wave];
+                double *tA = s_coef[wave];
+                uint4 *tC = s_blend[wave];
+                const float rnu = 1.0f / (float)win.nu;
+                const unsigned view_byte = (unsigned)s2c * (unsigned)rc.view_stride * S::kBytes;
+                // q.K and dout.V per pixel of the window
+                for (int u0 = 0; u0 < win.nunits; u0 += NS) {
+                    int unit;
+                    const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                    float dk4[4], dv4[4];
+                    window_dots<S, DC, G, kRow>(kb, off, qf, qp, dk4);
+                    window_dots<S, DC, G, kRow>(vb, off, dof, dop, dv4);
+                    if (g == 0) {
+                        *reinterpret_cast<float4 *>(tS + 4 * unit) = make_float4(dk4[0], dk4[1], dk4[2], dk4[3]);
+                        *reinterpret_cast<float4 *>(tT + 4 * unit) = make_float4(dv4[0], dv4[1], dv4[2], dv4[3]);
+                    }
+                }
+                for (int e = lane; e < 4 * win.nunits; e += kWave) tA[e] = 0.0;
+                wave_lds_sync();
+                // the samples, one per lane
+                const int4 te = window_entries(tp, win, dm.Wimg, dm.Himg);
+                const float w0 = live ? tp.w[0] : 0.f, w1 = live ? tp.w[1] : 0.f;
+                const float w2 = live ? tp.w[2] : 0.f, w3 = live ? tp.w[3] : 0.f;
+                const float dot = fmaf(w0, tS[te.x], fmaf(w1, tS[te.y], fmaf(w2, tS[te.z], w3 * tS[te.w])));
+                const float dp = fmaf(w0, tT[te.x], fmaf(w1, tT[te.y], fmaf(w2, tT[te.z], w3 * tT[te.w])));
+                const float p = live ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
+                const float ds = p * (dp - delta);
+                if (w0 != 0.f) atomicAdd(&tA[te.x], (double)(ds * w0));
+                if (w1 != 0.f) atomicAdd(&tA[te.y], (double)(ds * w1));
+                if (w2 != 0.f) atomicAdd(&tA[te.z], (double)(ds * w2));
+                if (w3 != 0.f) atomicAdd(&tA[te.w], (double)(ds * w3));
+                wave_lds_sync();
+                if (lane < win.nunits) {
+                    const float c0f = (float)tA[4 * lane], c1f = (float)tA[4 * lane + 1];
+                    const float c2f = (float)tA[4 * lane + 2], c3f = (float)tA[4 * lane + 3];
+                    if constexpr (kBlock) {
+                        tC[2 * lane] = split_coefficients<S>(c0f, c1f, c2f, c3f);
+                        tC[2 * lane + 1] = make_uint4(0u, 0u, 0u, 0u);
+                    } else {
+                        tC[2 * lane] = make_uint4(__float_as_uint(c0f), __float_as_uint(c1f), __float_as_uint(c2f), __float_as_uint(c3f));
+                    }
+                }
+                wave_lds_sync();
+                // dq += coefficient * K per pixel
+                if constexpr (kBlock) {
+                    floatx4 macc[DC];
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) macc[d] = floatx4{0.f, 0.f, 0.f, 0.f};
+                    for (int u0 = 0; u0 < win.nunits; u0 += NS) {
+                        int unit;
+                        const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                        uint2 cf = reinterpret_cast<const uint2 *>(tC)[4 * unit + (lane & 3)];
+                        if (u0 + slot >= win.nunits) cf = make_uint2(0u, 0u);
+                        uint32_t r[4][DC / 2];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) load_packed<S, DC>(kb + off + k * kRow, r[k]);
+                        block_blend4<S, DC>(r, __builtin_bit_cast(shortx4, cf), macc);
+                    }
+#pragma unroll
+                    for (int d = 0; d < DC; ++d) dqa[d] += macc[d][0] + macc[d][1];
+                } else {
+                    for (int u0 = 0; u0 < win.nunits; u0 += NS) {
+                        int unit;
+                        const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                        uint4 cu = tC[2 * unit];
+                        if (u0 + slot >= win.nunits) cu = make_uint4(0u, 0u, 0u, 0u);
+                        const float cf[4] = { __uint_as_float(cu.x), __uint_as_float(cu.y), __uint_as_float(cu.z), __uint_as_float(cu.w) };
+                        float r[4][DC];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) load_chunk<S, DC>(kb + off + k * kRow, r[k]);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+#pragma unroll
+                            for (int d = 0; d < DC; ++d) dqa[d] = fmaf(cf[k], r[k][d], dqa[d]);
+                        }
+                    }
+                }
+                wave_lds_sync();
+                continue;
+            }
+        }
+        park_descriptors<D, S::kBytes>(tp, live, nc, rc, dm, lane, s_w[wave], s_e[wave]);
         if constexpr (CG) {
             // (stage_descriptors ends with a wave-level LDS sync; these two arrays are read after the
             // next one, and their previous readers finished before the sync at its start)
-            const int n = min(c0 + lane, dm.N - 1);
-            const float2 xy = coords[rc.crow + n];
-            const TapGrads tg = make_tap_grads(xy.x, xy.y, dm.Wimg, dm.Himg);
+            const TapGrads tg = make_tap_grads(xy0.x, xy0.y, dm.Wimg, dm.Himg);
             s_gx[wave][lane] = make_float4(tg.gx[0], tg.gx[1], tg.gx[2], tg.gx[3]);
             s_gy[wave][lane] = make_float4(tg.gy[0], tg.gy[1], tg.gy[2], tg.gy[3]);
             wave_lds_sync();
         }
-        const int cnt = min(kWave, dm.N - c0);
 #pragma unroll
         for (int it = 0; it < ITS; ++it) {
             if (it * NS < cnt) {

@@ -110,6 +110,11 @@ template <typename S, int D> struct Chunk {
     static constexpr int value = (D / kMin > 16) ? D / 16 : kMin;
 };
 
+// The gather kernels cut a row's samples into chunks per key view, each of which may be worked on per pixel of
+// the window its samples fall into, when a view has at least a chunk's worth of samples; with fewer, chunks of
+// 64 consecutive samples (several views each) keep the lanes busy and always gather.
+static inline bool gather_window_mode(int P) { return P >= kWave; }
+
 template <typename S, int D>
 int launch_fwd_gather(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
                       const Dims &dm, hipStream_t st)
@@ -117,9 +122,14 @@ int launch_fwd_gather(const void *q, const void *k, const void *v, const float *
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(0, st);
-    DSDPA_LAUNCH((fwd_gather_kernel<S, D, DC>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
-                          timer.start(), timer.stop(),
-                       q, k, v, coords, out, lse, dm);
+    if (gather_window_mode(dm.P))
+        DSDPA_LAUNCH((fwd_gather_kernel<S, D, DC, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                              timer.start(), timer.stop(),
+                           q, k, v, coords, out, lse, dm);
+    else
+        DSDPA_LAUNCH((fwd_gather_kernel<S, D, DC, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                              timer.start(), timer.stop(),
+                           q, k, v, coords, out, lse, dm);
     return check_launch();
 }
 
@@ -146,11 +156,15 @@ int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const floa
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(2, st);
     if (dcoords)
-        DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+        DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, true, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                              timer.start(), timer.stop(),
+                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, dm);
+    else if (gather_window_mode(dm.P))
+        DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, false, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
                            q, k, v, coords, out, lse, dout, dq, stats, dcoords, dm);
     else
-        DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+        DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, false, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
                            q, k, v, coords, out, lse, dout, dq, stats, dcoords, dm);
     return check_launch();

@@ -96,6 +96,45 @@ def test_small_cases_vs_oracle(case, dtype, path):
     assert rel(dv, rdv) < TOL_BWD[dtype]
 
 
+# Clustered coordinates with at least 64 samples per view: the gather kernels then cut chunks per key view and
+# work on the pixels of the window a chunk's samples fall into (fp32: multiply-adds; 16-bit storage: the 4x4x4
+# block matrix instruction), or gather tap by tap where the window is too large or the image too narrow.
+WINDOWS = [
+    # seed B  V  H  Himg Wimg D    P    sigma  centres lo, hi
+    (31, 1, 2, 2, 24, 20, 32, 64, 0.04, 0.3, 0.7),
+    (32, 1, 3, 1, 16, 40, 128, 100, 0.03, 0.0, 1.0),       # clusters on the border: windows cut by the image edge
+    (33, 2, 2, 2, 30, 30, 64, 70, 0.02, -0.05, 1.05),      # centres outside the image: samples with no tap inside
+    (34, 1, 2, 1, 40, 3, 16, 64, 0.05, 0.2, 0.8),          # image narrower than one unit of a window row
+    (35, 1, 1, 2, 12, 12, 256, 130, 0.3, 0.5, 0.5),        # wide spread: windows too large, every chunk gathers
+    (36, 1, 2, 2, 33, 29, 64, 64, 0.004, 0.1, 0.9),        # very tight clusters: windows of one or two units
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("case", WINDOWS, ids=[f"w{c[0]}" for c in WINDOWS])
+def test_clustered_windows_vs_oracle(case, dtype):
+    seed, B, V, H, Himg, Wimg, D, P, sigma, lo, hi = case
+    say(f"[case] windows seed={seed} B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} sigma={sigma} {dtype}")
+    g = torch.Generator().manual_seed(seed)
+    L = Himg * Wimg
+    q, k, v = (torch.randn(B, V, H, L, D, generator=g).to(dtype) for _ in range(3))
+    mu = torch.rand(B, V, L, V, 1, 2, generator=g) * (hi - lo) + lo
+    c = mu + sigma * torch.randn(B, V, L, V, P, 2, generator=g)
+    c[0, 0, 1, 0, 3, 0] = float("nan")                     # one NaN coordinate inside a cluster
+    do = torch.randn(B, V, H, L, D, generator=g).to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    prev = _native.set_path(_native.PATH_GATHER)
+    try:
+        out, dq, dk, dv = run_op(q, k, v, c, do, Wimg, Himg, scale)
+    finally:
+        _native.set_path(prev)
+    ro, _, rdq, rdk, rdv = oracle_all(q, k, v, c, do, Wimg, Himg, scale)
+    assert rel(out, ro) < TOL_FWD[dtype]
+    assert rel(dq, rdq) < TOL_BWD[dtype]
+    assert rel(dk, rdk) < TOL_BWD[dtype]
+    assert rel(dv, rdv) < TOL_BWD[dtype]
+
+
 GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
 
 
