@@ -360,12 +360,13 @@ __device__ __forceinline__ T wave_all(T x, Op op)
 }
 __device__ __forceinline__ float wave_max(float x) { return wave_all(x, [](float a, float b) { return fmaxf(a, b); }); }
 __device__ __forceinline__ float wave_sum(float x) { return wave_all(x, [](float a, float b) { return a + b; }); }
-// two unsigned 16-bit fields per word, minimum taken field by field
+// two unsigned 16-bit fields per word, minimum taken field by field (one packed 16-bit minimum per step)
 __device__ __forceinline__ uint32_t wave_min_u16x2(uint32_t x)
 {
+    typedef unsigned short dsdpa_u16x2 __attribute__((ext_vector_type(2)));
     return wave_all(x, [](uint32_t a, uint32_t b) {
-        const uint32_t lo = min(a & 0xffffu, b & 0xffffu), hi = min(a >> 16, b >> 16);
-        return lo | (hi << 16);
+        return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(dsdpa_u16x2, a),
+                                                                        __builtin_bit_cast(dsdpa_u16x2, b)));
     });
 }
 
