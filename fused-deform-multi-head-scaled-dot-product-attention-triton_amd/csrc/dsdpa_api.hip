@@ -47,49 +47,50 @@ void *scratch_on_current_device()
 extern "C" {
 
 int dsdpa_fwd_f32(const float *q, const float *k, const float *v, const float *coords, float *out, float *lse, void *workspace,
-                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides, void *stream)
 {
-    return fwd_impl<F32>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+    return fwd_impl<F32>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
 }
 
 int dsdpa_fwd_bf16(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse, void *workspace,
-                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides, void *stream)
 {
-    return fwd_impl<BF16>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+    return fwd_impl<BF16>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
 }
 
 int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse, void *workspace,
-                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides, void *stream)
 {
-    return fwd_impl<F16>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+    return fwd_impl<F16>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
 }
 
 int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords, const float *out,
                   const float *lse, const float *dout, float *dq, float *dk, float *dv, float *dcoords, void *workspace,
-                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, unsigned flags, void *stream)
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides, unsigned flags, void *stream)
 {
     return bwd_impl<F32>(q, k, v, coords, out, lse, dout, dq, dk, dv, dcoords, workspace, B, V, H, Himg, Wimg, D, P,
-                         sm_scale, flags, stream);
+                         sm_scale, strides, flags, stream);
 }
 
 int dsdpa_bwd_bf16(const void *q, const void *k, const void *v, const float *coords, const void *out,
                    const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
-                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, unsigned flags, void *stream)
+                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides, unsigned flags, void *stream)
 {
     return bwd_impl<BF16>(q, k, v, coords, out, lse, dout, dq, dk, dv, dcoords, workspace, B, V, H, Himg, Wimg, D, P,
-                          sm_scale, flags, stream);
+                          sm_scale, strides, flags, stream);
 }
 
 int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coords, const void *out,
                   const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
-                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, unsigned flags, void *stream)
+                  int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides, unsigned flags, void *stream)
 {
     return bwd_impl<F16>(q, k, v, coords, out, lse, dout, dq, dk, dv, dcoords, workspace, B, V, H, Himg, Wimg, D, P,
-                         sm_scale, flags, stream);
+                         sm_scale, strides, flags, stream);
 }
 
 int dsdpa_fwd_noalloc(int dtype, const void *q, const void *k, const void *v, const float *coords, void *out,
-                      float *lse, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+                      float *lse, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale,
+                      const long long *strides, void *stream)
 {
     if (dtype != DSDPA_F32 && dtype != DSDPA_BF16 && dtype != DSDPA_F16) return DSDPA_ERR_DTYPE;
     if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || P < 1) return DSDPA_ERR_BAD_SHAPE;
@@ -102,9 +103,9 @@ int dsdpa_fwd_noalloc(int dtype, const void *q, const void *k, const void *v, co
         if (!ws) return DSDPA_ERR_HIP;
     }
     switch (dtype) {
-    case DSDPA_F32: return fwd_impl<F32>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
-    case DSDPA_BF16: return fwd_impl<BF16>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
-    default: return fwd_impl<F16>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, stream);
+    case DSDPA_F32: return fwd_impl<F32>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
+    case DSDPA_BF16: return fwd_impl<BF16>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
+    default: return fwd_impl<F16>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
     }
 }
 
@@ -134,6 +135,7 @@ const char *dsdpa_error_string(int code)
     case DSDPA_ERR_HIP: return "a HIP launch failed (see dsdpa_last_hip_error)";
     case DSDPA_ERR_UNSUPPORTED: return "unknown flag, or a combination of options that is not supported";
     case DSDPA_ERR_DTYPE: return "unknown dtype code";
+    case DSDPA_ERR_BAD_STRIDES: return "strides: the head dimension must be contiguous and every row 16-byte aligned";
     case DSDPA_ERR_SCRATCH: return "the shape needs more scratch memory than the library's built-in buffer holds";
     }
     return "unknown error code";
@@ -141,7 +143,7 @@ const char *dsdpa_error_string(int code)
 
 int dsdpa_last_hip_error(void) { return g_last_hip_error; }
 
-int dsdpa_version(void) { return 100; }
+int dsdpa_version(void) { return 200; }
 
 int dsdpa_timer_enable(int on)
 {

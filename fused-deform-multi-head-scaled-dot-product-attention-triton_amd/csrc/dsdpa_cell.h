@@ -274,7 +274,8 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 
     constexpr int NS = kWave / G;
     static_assert(G >= 4 && G <= 64 && G * DC == D, "lane split (a block of four lanes must not straddle two samples)");
     __shared__ float4 s_w[kCellWaves][kWave];
-    __shared__ unsigned s_row[kCellWaves][kWave];
+    __shared__ unsigned s_row[kCellWaves][kWave];           // byte offset of the entry's query row in dout (and its (lse, delta))
+    __shared__ unsigned s_qrow[kCellWaves][kWave];          // ... in q (which may be strided)
     __shared__ float2 s_f[S::kBytes == 2 ? kCellWaves : 1][kWave];          // 16-bit storage: (fx, fy) of the entry
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
@@ -316,9 +317,10 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 
     const bool tv[4] = { vy0 && vx0, vy0 && vx1, vy1 && vx0, vy1 && vx1 };
     const int tpix[4] = { y0 * dm.Wimg + x0, y0 * dm.Wimg + x0 + 1, (y0 + 1) * dm.Wimg + x0,
                           (y0 + 1) * dm.Wimg + x0 + 1 };
-    const size_t plane_base = ((grp * dm.H) + h) * (size_t)dm.L * D;          // elements; grp = b*V + s2
-    const char *kb = (const char *)k_ + plane_base * S::kBytes;
-    const char *vb = (const char *)v_ + plane_base * S::kBytes;
+    const size_t plane_base = ((grp * dm.H) + h) * (size_t)dm.L * D;          // elements in dk/dv; grp = b*V + s2
+    const size_t kv_base = dm.kv_plane(b, s2, h);                               // ... in k and v
+    const char *kb = (const char *)k_ + kv_base * S::kBytes;
+    const char *vb = (const char *)v_ + kv_base * S::kBytes;
     // fp32 storage: the taps widened in registers; 16-bit storage: the taps as packed pairs (half the
     // registers) feeding the packed dot-product instructions
     constexpr bool kPacked = S::kBytes == 2;
@@ -339,12 +341,12 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 
 #pragma unroll
             for (int i = 0; i < DC / 2; ++i) { ktp[tpi][i] = 0u; vtp[tpi][i] = 0u; }
             if (tv[tpi]) {
-                load_packed<S, DC>(kb + ((size_t)tpix[tpi] * D + lane_elem) * S::kBytes, ktp[tpi]);
-                load_packed<S, DC>(vb + ((size_t)tpix[tpi] * D + lane_elem) * S::kBytes, vtp[tpi]);
+                load_packed<S, DC>(kb + ((size_t)tpix[tpi] * dm.kv_sl + lane_elem) * S::kBytes, ktp[tpi]);
+                load_packed<S, DC>(vb + ((size_t)tpix[tpi] * dm.kv_sl + lane_elem) * S::kBytes, vtp[tpi]);
             }
         } else {
-            load_tap_or_zero<S, DC>(kb, tpix[tpi], D, lane_elem, tv[tpi], kt[tpi]);
-            load_tap_or_zero<S, DC>(vb, tpix[tpi], D, lane_elem, tv[tpi], vt[tpi]);
+            load_tap_or_zero<S, DC>(kb, tpix[tpi], dm.kv_sl, lane_elem, tv[tpi], kt[tpi]);
+            load_tap_or_zero<S, DC>(vb, tpix[tpi], dm.kv_sl, lane_elem, tv[tpi], vt[tpi]);
         }
     }
 #pragma unroll
@@ -375,7 +377,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 
     constexpr int kRowWords = DC * S::kBytes / 4;                           // 32-bit words of a row held by one lane
     constexpr int kRowToPairShift = __builtin_ctz(kRowBytes) - 3;          // row byte offset -> offset of the row's (lse, delta)
     const size_t bh_row0 = ((size_t)b * dm.V * dm.H + h) * dm.L;              // row of (b, s1 = 0, h, l = 0)
-    const char *q_bh = (const char *)q_ + bh_row0 * kRowBytes;
+    const char *q_bh = (const char *)q_ + dm.q_row(b, 0, h, 0) * S::kBytes;
     const char *do_bh = (const char *)dout_ + bh_row0 * kRowBytes;
     const char *stats_bh = (const char *)(stats_ + bh_row0);                 // (lse, delta) per row
     const unsigned lane_byte = (unsigned)lane_elem * S::kBytes;
@@ -412,6 +414,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 
             s_w[wave][lane] = make_float4(fx, fy, fx * fy, live ? 1.0f : 0.0f);
         }
         s_row[wave][lane] = (s1 * view_rows + l) * kRowBytes;
+        s_qrow[wave][lane] = (s1 * (unsigned)dm.q_sv + l * (unsigned)dm.q_sl) * S::kBytes;
         wave_lds_sync();
         const int cnt = (int)min((unsigned)kWave, hi - c0);
         // The NS samples of a trip need their query rows (q, dout, lse, delta) from memory, a round trip of
@@ -421,7 +424,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 
         auto issue = [&](int j0, RowFetch<kRowWords> &f) {
             const unsigned r = s_row[wave][j0 + slot];
             const unsigned roff = r + lane_byte, soff = r >> kRowToPairShift;
-            load_words<kRowWords>(q_bh + roff, f.qw);
+            load_words<kRowWords>(q_bh + (s_qrow[wave][j0 + slot] + lane_byte), f.qw);
             load_words<kRowWords>(do_bh + roff, f.dw);
             f.ld = *(const float2 *)(stats_bh + soff);
         };

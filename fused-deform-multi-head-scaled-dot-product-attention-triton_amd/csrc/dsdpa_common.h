@@ -37,6 +37,19 @@ struct Dims {
     int rows;                           // B*V*H*L query rows
     float sm_scale;
     FastDiv divP, divL;                 // for decoding sample ids (s1*L + l)*P + p
+    // Element strides of the inputs q and k/v (k and v share one set) over (batch, view, head, pixel); the head
+    // dimension itself is contiguous. Everything else (out, lse, dout, the gradients) is contiguous
+    // [B][V][H][L][D]. Offsets inside one (batch, head) -- view*sv + pixel*sl -- fit 32 bits.
+    long long q_sb, q_sh, kv_sb, kv_sh;
+    int q_sv, q_sl, kv_sv, kv_sl;
+    __device__ __forceinline__ size_t q_row(int b, int s1, int h, int l) const
+    {
+        return (size_t)((long long)b * q_sb + (long long)h * q_sh) + (size_t)((unsigned)s1 * (unsigned)q_sv + (unsigned)l * (unsigned)q_sl);
+    }
+    __device__ __forceinline__ size_t kv_plane(int b, int view, int h) const
+    {
+        return (size_t)((long long)b * kv_sb + (long long)h * kv_sh) + (size_t)((unsigned)view * (unsigned)kv_sv);
+    }
 };
 
 // ------------------------------------------------------------------ storage types

@@ -3,8 +3,8 @@
 
 namespace dsdpa {
 template int fwd_impl<F16>(const void *, const void *, const void *, const float *, void *, float *, void *, int, int, int, int,
-                           int, int, int, float, void *);
+                           int, int, int, float, const long long *, void *);
 template int bwd_impl<F16>(const void *, const void *, const void *, const float *, const void *, const float *,
                            const void *, void *, void *, void *, float *, void *, int, int, int, int, int, int, int, float,
-                           unsigned, void *);
+                           const long long *, unsigned, void *);
 }  // namespace dsdpa

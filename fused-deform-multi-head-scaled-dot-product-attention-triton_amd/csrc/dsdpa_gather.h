@@ -18,10 +18,12 @@ namespace dsdpa {
 constexpr int kGatherWaves = 4;   // waves (= query rows) per workgroup
 
 struct RowCtx {
-    size_t row;        // linear query row in [B][V][H][L]
-    size_t kv_base;    // element offset of plane (b, view 0, h) in k/v/dk/dv
+    size_t row;        // linear query row in [B][V][H][L] (out, lse, dout, dq)
+    size_t q_off;      // element offset of the query row in q
+    size_t kv_base;    // element offset of plane (b, view 0, h) in k and v
+    size_t acc_base;   // the same in the contiguous dk/dv accumulators
     size_t crow;       // float2 offset of coords[b][s1][l][0][0]
-    int view_stride;   // elements between consecutive views of one (b, h)
+    int view_stride;   // elements between consecutive views of one (b, h) in k and v
 };
 
 // Logical work item -> query row; order (b, h, s1, l), l fastest, so that
@@ -36,9 +38,11 @@ __device__ __forceinline__ RowCtx decode_row(int work, const Dims &dm, int D)
     int b = t / dm.H;
     RowCtx c;
     c.row = (((size_t)b * dm.V + s1) * dm.H + h) * dm.L + l;
-    c.kv_base = ((size_t)b * dm.V * dm.H + h) * (size_t)dm.L * D;
+    c.q_off = dm.q_row(b, s1, h, l);
+    c.kv_base = dm.kv_plane(b, 0, h);
+    c.acc_base = ((size_t)b * dm.V * dm.H + h) * (size_t)dm.L * D;
     c.crow = (((size_t)b * dm.V + s1) * dm.L + l) * (size_t)dm.N;
-    c.view_stride = dm.H * dm.L * D;
+    c.view_stride = dm.kv_sv;
     return c;
 }
 
@@ -52,8 +56,8 @@ __device__ __forceinline__ void park_descriptors(const Taps &tp, bool valid, int
 {
     int ebase = (nc / dm.P) * rc.view_stride;
     float4 w = valid ? make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]) : make_float4(0.f, 0.f, 0.f, 0.f);
-    uint4 e = make_uint4((unsigned)(ebase + tp.pix[0] * D) * BYTES, (unsigned)(ebase + tp.pix[1] * D) * BYTES,
-                         (unsigned)(ebase + tp.pix[2] * D) * BYTES, (unsigned)(ebase + tp.pix[3] * D) * BYTES);
+    uint4 e = make_uint4((unsigned)(ebase + tp.pix[0] * dm.kv_sl) * BYTES, (unsigned)(ebase + tp.pix[1] * dm.kv_sl) * BYTES,
+                         (unsigned)(ebase + tp.pix[2] * dm.kv_sl) * BYTES, (unsigned)(ebase + tp.pix[3] * dm.kv_sl) * BYTES);
     wave_lds_sync();          // the previous chunk's readers are done
     s_w[lane] = w;
     s_e[lane] = e;
@@ -131,26 +135,25 @@ __device__ __forceinline__ int4 window_entries(const Taps &tp, const Window &win
 
 // The unit this slot takes in the step that starts at unit u0 (held at the last unit beyond the window),
 // and the byte offset of its first pixel from plane (b, view 0, h).
-template <int ROW_BYTES>
 __device__ __forceinline__ unsigned window_unit(const Window &win, int u0, int slot, int Wimg, unsigned view_byte,
-                                                float rnu, int *unit)
+                                                float rnu, unsigned px_bytes, int *unit)
 {
     const int u = min(u0 + slot, win.nunits - 1);
     const int wy = (int)(((float)u + 0.5f) * rnu);             // u / nu: exact for these small numbers
     const int wxu = u - wy * win.nu;
     *unit = u;
-    return view_byte + (unsigned)((win.ymin + wy) * Wimg + win.xmin + 4 * wxu) * ROW_BYTES;
+    return view_byte + (unsigned)((win.ymin + wy) * Wimg + win.xmin + 4 * wxu) * px_bytes;
 }
 
 // q.K for the four pixels of this slot's unit, summed over the slot: t[4*unit + k].
-template <typename S, int DC, int G, int ROW_BYTES>
-__device__ __forceinline__ void window_dots(const char *__restrict__ base, unsigned off, const float (&xf)[DC],
-                                            const uint32_t *xp, float (&d)[4])
+template <typename S, int DC, int G>
+__device__ __forceinline__ void window_dots(const char *__restrict__ base, unsigned off, unsigned px_bytes,
+                                            const float (&xf)[DC], const uint32_t *xp, float (&d)[4])
 {
     if constexpr (S::kBytes == 2) {
         uint32_t r[4][DC / 2];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) load_packed<S, DC>(base + off + k * ROW_BYTES, r[k]);
+        for (int k = 0; k < 4; ++k) load_packed<S, DC>(base + off + k * px_bytes, r[k]);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             float acc = 0.f;
@@ -168,7 +171,7 @@ __device__ __forceinline__ void window_dots(const char *__restrict__ base, unsig
     } else {
         float r[4][DC];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) load_chunk<S, DC>(base + off + k * ROW_BYTES, r[k]);
+        for (int k = 0; k < 4; ++k) load_chunk<S, DC>(base + off + k * px_bytes, r[k]);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             float acc = 0.f;
@@ -304,9 +307,9 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
     uint32_t qp[kPacked ? DC / 2 : 1];
     const float qscale = dm.sm_scale * kLog2e;
     if constexpr (kPacked) {
-        load_packed<S, DC>((const char *)q_ + (rc.row * D + lane_elem) * S::kBytes, qp);
+        load_packed<S, DC>((const char *)q_ + (rc.q_off + lane_elem) * S::kBytes, qp);
     } else {
-        load_chunk<S, DC>((const char *)q_ + (rc.row * D + lane_elem) * S::kBytes, qf);
+        load_chunk<S, DC>((const char *)q_ + (rc.q_off + lane_elem) * S::kBytes, qf);
 #pragma unroll
         for (int d = 0; d < DC; ++d) qf[d] *= qscale;
     }
@@ -336,7 +339,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
             const bool counted = live && ((tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f));
             const Window win = chunk_window(tp, counted, dm.Wimg, dm.Himg);
             if (win.nunits > 0 && win.nunits <= kWinUnits && 4 * win.nunits <= 3 * cnt) {
-                constexpr int kRow = D * S::kBytes;
+                const unsigned kRow = (unsigned)dm.kv_sl * S::kBytes;       // bytes between neighbouring pixels of K and V
                 constexpr bool kBlock = kPacked && G >= 4;         // V rows blended by the block matrix instruction
                 float *tS = s_dot[wave];
                 double *tA = s_coef[wave];
@@ -346,9 +349,9 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
                 // one q.K dot product per pixel of the window
                 for (int u0 = 0; u0 < win.nunits; u0 += NS) {
                     int unit;
-                    const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                    const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
                     float d4[4];
-                    window_dots<S, DC, G, kRow>(kb, off, qf, qp, d4);
+                    window_dots<S, DC, G>(kb, off, kRow, qf, qp, d4);
                     if (g == 0) *reinterpret_cast<float4 *>(tS + 4 * unit) = make_float4(d4[0], d4[1], d4[2], d4[3]);
                 }
                 for (int e = lane; e < 4 * win.nunits; e += kWave) tA[e] = 0.0;
@@ -394,7 +397,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
                     for (int d = 0; d < DC; ++d) macc[d] = floatx4{0.f, 0.f, 0.f, 0.f};
                     for (int u0 = 0; u0 < win.nunits; u0 += NS) {
                         int unit;
-                        const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                        const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
                         uint2 cf = reinterpret_cast<const uint2 *>(tC)[4 * unit + (lane & 3)];
                         if (u0 + slot >= win.nunits) cf = make_uint2(0u, 0u);
                         uint32_t r[4][DC / 2];
@@ -407,7 +410,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
                 } else {
                     for (int u0 = 0; u0 < win.nunits; u0 += NS) {
                         int unit;
-                        const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                        const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
                         uint4 cu = tC[2 * unit];
                         if (u0 + slot >= win.nunits) cu = make_uint4(0u, 0u, 0u, 0u);
                         const float cf[4] = { __uint_as_float(cu.x), __uint_as_float(cu.y), __uint_as_float(cu.z), __uint_as_float(cu.w) };
@@ -518,13 +521,14 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_gather_kernel(
     const unsigned lane_byte = (unsigned)lane_elem * S::kBytes;
     const char *kb = (const char *)k_ + rc.kv_base * S::kBytes;
     const char *vb = (const char *)v_ + rc.kv_base * S::kBytes;
-    float *dkb = dk_acc + rc.kv_base + lane_elem;
-    float *dvb = dv_acc + rc.kv_base + lane_elem;
+    float *dkb = dk_acc + rc.acc_base + lane_elem;        // (this kernel runs on contiguous k/v only: the taps'
+    float *dvb = dv_acc + rc.acc_base + lane_elem;        //  offsets in k/v are then their offsets in dk/dv too)
     const float2 *coords = (const float2 *)coords_;
 
     float qf[DC], dof[DC], of[DC];
     const size_t roff = (rc.row * D + lane_elem) * S::kBytes;
-    load_chunk<S, DC>((const char *)q_ + roff, qf);
+    const size_t q_roff = (rc.q_off + lane_elem) * S::kBytes;
+    load_chunk<S, DC>((const char *)q_ + q_roff, qf);
     load_chunk<S, DC>((const char *)dout_ + roff, dof);
     load_chunk<S, DC>((const char *)out_ + roff, of);
     // delta = dout . out  (the reference's _bwd_preprocess, fused here)
@@ -644,11 +648,12 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     float qf[DC], dof[DC], of[DC];
     uint32_t dop[kPacked ? DC / 2 : 1], qp[kPacked && WIN ? DC / 2 : 1];
     const size_t roff = (rc.row * D + lane_elem) * S::kBytes;
-    load_chunk<S, DC>((const char *)q_ + roff, qf);
+    const size_t q_roff = (rc.q_off + lane_elem) * S::kBytes;
+    load_chunk<S, DC>((const char *)q_ + q_roff, qf);
     load_chunk<S, DC>((const char *)dout_ + roff, dof);
     load_chunk<S, DC>((const char *)out_ + roff, of);
     if constexpr (kPacked) load_packed<S, DC>((const char *)dout_ + roff, dop);
-    if constexpr (kPacked && WIN) load_packed<S, DC>((const char *)q_ + roff, qp);
+    if constexpr (kPacked && WIN) load_packed<S, DC>((const char *)q_ + q_roff, qp);
     float delta = 0.f;
 #pragma unroll
     for (int d = 0; d < DC; ++d) delta = fmaf(dof[d], of[d], delta);
@@ -682,7 +687,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
             const bool counted = live && ((tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f));
             const Window win = window_ok ? chunk_window(tp, counted, dm.Wimg, dm.Himg) : Window{0, 0, 0, 0};
             if (win.nunits > 0 && win.nunits <= kWinUnits && 4 * win.nunits <= 3 * cnt) {
-                constexpr int kRow = D * S::kBytes;
+                const unsigned kRow = (unsigned)dm.kv_sl * S::kBytes;       // bytes between neighbouring pixels of K and V
                 constexpr bool kBlock = kPacked && G >= 4;
                 float *tS = s_dotk[wave], *tT = s_dotv[wave];
                 double *tA = s_coef[wave];
@@ -692,10 +697,10 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                 // q.K and dout.V per pixel of the window
                 for (int u0 = 0; u0 < win.nunits; u0 += NS) {
                     int unit;
-                    const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                    const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
                     float dk4[4], dv4[4];
-                    window_dots<S, DC, G, kRow>(kb, off, qf, qp, dk4);
-                    window_dots<S, DC, G, kRow>(vb, off, dof, dop, dv4);
+                    window_dots<S, DC, G>(kb, off, kRow, qf, qp, dk4);
+                    window_dots<S, DC, G>(vb, off, kRow, dof, dop, dv4);
                     if (g == 0) {
                         *reinterpret_cast<float4 *>(tS + 4 * unit) = make_float4(dk4[0], dk4[1], dk4[2], dk4[3]);
                         *reinterpret_cast<float4 *>(tT + 4 * unit) = make_float4(dv4[0], dv4[1], dv4[2], dv4[3]);
@@ -734,7 +739,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                     for (int d = 0; d < DC; ++d) macc[d] = floatx4{0.f, 0.f, 0.f, 0.f};
                     for (int u0 = 0; u0 < win.nunits; u0 += NS) {
                         int unit;
-                        const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                        const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
                         uint2 cf = reinterpret_cast<const uint2 *>(tC)[4 * unit + (lane & 3)];
                         if (u0 + slot >= win.nunits) cf = make_uint2(0u, 0u);
                         uint32_t r[4][DC / 2];
@@ -747,7 +752,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                 } else {
                     for (int u0 = 0; u0 < win.nunits; u0 += NS) {
                         int unit;
-                        const unsigned off = window_unit<kRow>(win, u0, slot, dm.Wimg, view_byte, rnu, &unit) + lane_byte;
+                        const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
                         uint4 cu = tC[2 * unit];
                         if (u0 + slot >= win.nunits) cu = make_uint4(0u, 0u, 0u, 0u);
                         const float cf[4] = { __uint_as_float(cu.x), __uint_as_float(cu.y), __uint_as_float(cu.z), __uint_as_float(cu.w) };

@@ -215,12 +215,15 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
 // One storage type's forward / backward entry (argument checks, kernel selection, launches); each is
 // instantiated in its own translation unit (dsdpa_f32.hip, dsdpa_bf16.hip, dsdpa_f16.hip) so that the
 // three compile in parallel.
+// `strides`: null (everything contiguous) or the 8 element strides of q and of k/v over (batch, view, head, pixel).
 template <typename S>
 int fwd_impl(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
-             void *workspace, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream);
+             void *workspace, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale,
+             const long long *strides, void *stream);
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
              const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
-             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, unsigned flags, void *stream);
+             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides,
+             unsigned flags, void *stream);
 
 }  // namespace dsdpa

@@ -100,6 +100,34 @@ static inline int make_dims(int B, int V, int H, int Himg, int Wimg, int D, int 
     dm->L = (int)L; dm->P = P; dm->N = (int)N; dm->rows = (int)rows; dm->sm_scale = sm_scale;
     dm->divP = FastDiv::make((unsigned)P);
     dm->divL = FastDiv::make((unsigned)L);
+    dm->q_sl = dm->kv_sl = D;
+    dm->q_sh = dm->kv_sh = L * D;
+    dm->q_sv = dm->kv_sv = (int)((long long)H * L * D);
+    dm->q_sb = dm->kv_sb = slab;
+    return DSDPA_OK;
+}
+
+// Strides of q and of k/v as the caller gives them: element strides over (batch, view, head, pixel), q's four
+// then k/v's four; the head dimension must be contiguous (a row is read with 16-byte loads). The kernels
+// address a pixel of a (batch, head) as view*sv + pixel*sl in 32 bits, and every row start must be a
+// multiple of 16 bytes.
+static inline int apply_strides(const long long *st, int D, int esize, Dims *dm, bool *contiguous)
+{
+    *contiguous = true;
+    if (!st) return DSDPA_OK;
+    const long long align = 16 / esize;
+    for (int t = 0; t < 2; ++t) {
+        const long long sb = st[4 * t], sv = st[4 * t + 1], sh = st[4 * t + 2], sl = st[4 * t + 3];
+        if (sb < 0 || sv < 0 || sh < 0 || sl < D) return DSDPA_ERR_BAD_STRIDES;
+        if (sb % align || sv % align || sh % align || sl % align) return DSDPA_ERR_BAD_STRIDES;
+        const long long reach = (long long)(dm->V - 1) * sv + (long long)(dm->L - 1) * sl + D;   // inside one (b, h)
+        if (reach > (1ll << 30) || sv > (1ll << 30)) return DSDPA_ERR_TOO_LARGE;
+        if (t == 0) { dm->q_sb = sb; dm->q_sv = (int)sv; dm->q_sh = sh; dm->q_sl = (int)sl; }
+        else { dm->kv_sb = sb; dm->kv_sv = (int)sv; dm->kv_sh = sh; dm->kv_sl = (int)sl; }
+    }
+    const long long L = dm->L, H = dm->H;
+    *contiguous = dm->q_sl == D && dm->q_sh == L * D && dm->q_sv == H * L * D && dm->q_sb == (long long)dm->V * H * L * D &&
+                  dm->kv_sl == D && dm->kv_sh == L * D && dm->kv_sv == H * L * D && dm->kv_sb == (long long)dm->V * H * L * D;
     return DSDPA_OK;
 }
 
@@ -292,12 +320,15 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
 
 template <typename S>
 int fwd_impl(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
-             void *workspace, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, void *stream)
+             void *workspace, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale,
+             const long long *strides, void *stream)
 {
     if (!q || !k || !v || !coords || !out || !lse) return DSDPA_ERR_NULL_POINTER;
     Dims dm;
     int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
     if (rc != DSDPA_OK) return rc;
+    bool contiguous;
+    if ((rc = apply_strides(strides, D, S::kBytes, &dm, &contiguous)) != DSDPA_OK) return rc;
     hipStream_t st = (hipStream_t)stream;
     const DescLayout dl = desc_layout(B, V, Himg, Wimg, D, P, S::kBytes);
     if (dl.bytes && !workspace) return DSDPA_ERR_NULL_POINTER;
@@ -471,7 +502,8 @@ struct SideJoin {
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
              const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,
-             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, unsigned flags, void *stream)
+             int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides,
+             unsigned flags, void *stream)
 {
     if (!q || !k || !v || !coords || !out || !lse || !dout || !dq || !dk || !dv || !workspace)
         return DSDPA_ERR_NULL_POINTER;
@@ -482,6 +514,8 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     int rc = make_dims(B, V, H, Himg, Wimg, D, P, sm_scale, &dm);
     if (rc != DSDPA_OK) return rc;
     if ((long long)dm.L * dm.N > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;   // sample ids are 32-bit
+    bool contiguous;
+    if ((rc = apply_strides(strides, D, S::kBytes, &dm, &contiguous)) != DSDPA_OK) return rc;
     hipStream_t st = (hipStream_t)stream;
     const size_t n = (size_t)dm.rows * D;
     // the staged dq kernel computes dcoords only when the caller sized the workspace for it (same flags)
@@ -490,10 +524,12 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     char *ws = (char *)workspace;
     float2 *stats = (float2 *)(ws + wl.delta);          // per row: lse, delta
     const int path = deterministic ? (int)DSDPA_PATH_AUTO : g_path.load();   // only the cell-binned path has a fixed order
-    const bool fused_atomics = path == DSDPA_PATH_GATHER;
-    const bool cell_binned = path == DSDPA_PATH_AUTO;
+    // (the per-tap atomic backward, kept as the reference's scheme for measurements, takes a tap's offset in k/v
+    // for its offset in dk/dv: with strided k/v the gather dq kernel and the cell-binned dk/dv take its place)
+    const bool fused_atomics = path == DSDPA_PATH_GATHER && contiguous;
+    const bool cell_binned = path == DSDPA_PATH_AUTO || (path == DSDPA_PATH_GATHER && !contiguous);
     // (with the coordinate gradient the layout holds a table only where the larger LDS block still fits)
-    const bool staged = !fused_atomics && wl.dl.bytes != 0 && (!dcoords || cg_table) &&
+    const bool staged = path != DSDPA_PATH_GATHER && wl.dl.bytes != 0 && (!dcoords || cg_table) &&
                         (path == DSDPA_PATH_LDS || !few_samples_prefer_gather(V, P));
     const float4 *desc_w = (const float4 *)(ws + wl.desc + wl.dl.w);
     const uint32_t *desc_e = (const uint32_t *)(ws + wl.desc + wl.dl.e);

@@ -53,17 +53,18 @@ constexpr int kPlaneGradBytes = kPlaneWaves * kPlaneDescPlaces * 8;         // f
 template <typename S, int D>
 __host__ __device__ constexpr int plane_lds_bytes(int L) { return (L + 2) * 2 * D * S::kBytes; }
 
-// global [L][D] plane -> LDS rows 1..L of the interleaved image (which = 0: K half, 1: V half)
+// global plane of L rows of D elements, `px_bytes` apart -> LDS rows 1..L of the interleaved image
+// (which = 0: K half, 1: V half)
 template <typename S, int D>
-__device__ __forceinline__ void stage_plane(unsigned char *lds, const char *src, int L, int which)
+__device__ __forceinline__ void stage_plane(unsigned char *lds, const char *src, int L, unsigned px_bytes, int which)
 {
     constexpr int kRow = D * S::kBytes;
     constexpr int kChunksPerRow = kRow / 16;
-    const uint4 *s4 = reinterpret_cast<const uint4 *>(src);
     const int n16 = L * kChunksPerRow;
     for (int i = threadIdx.x; i < n16; i += kPlaneWaves * kWave) {
-        const int q = i / kChunksPerRow + 1, c = i % kChunksPerRow;
-        *reinterpret_cast<uint4 *>(lds + (size_t)q * 2 * kRow + ((q & 1) ^ which) * kRow + c * 16) = s4[i];
+        const int p = i / kChunksPerRow, q = p + 1, c = i % kChunksPerRow;
+        const uint4 t = *reinterpret_cast<const uint4 *>(src + (size_t)p * px_bytes + c * 16);
+        *reinterpret_cast<uint4 *>(lds + (size_t)q * 2 * kRow + ((q & 1) ^ which) * kRow + c * 16) = t;
     }
 }
 
@@ -256,9 +257,9 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
     float qf[DC], acc[DC];
     uint32_t qp[kPacked ? DC / 2 : 1];
     if constexpr (kPacked) {
-        load_packed<S, DC>((const char *)q_ + (row * D + lane_elem) * S::kBytes, qp);
+        load_packed<S, DC>((const char *)q_ + (dm.q_row(pb.b, (int)s1, pb.h, (int)l) + lane_elem) * S::kBytes, qp);
     } else {
-        load_chunk<S, DC>((const char *)q_ + (row * D + lane_elem) * S::kBytes, qf);
+        load_chunk<S, DC>((const char *)q_ + (dm.q_row(pb.b, (int)s1, pb.h, (int)l) + lane_elem) * S::kBytes, qf);
 #pragma unroll
         for (int d = 0; d < DC; ++d) qf[d] *= qscale;
     }
@@ -267,10 +268,11 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
     for (int d = 0; d < DC; ++d) acc[d] = 0.f;
 
     for (int s2 = 0; s2 < dm.V; ++s2) {
-        const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;
+        const size_t plane = dm.kv_plane(pb.b, s2, pb.h) * S::kBytes;
+        const unsigned px_bytes = (unsigned)dm.kv_sl * S::kBytes;
         __syncthreads();                                       // the previous view's readers are done
-        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, 0);
-        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
+        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, px_bytes, 0);
+        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, px_bytes, 1);
         __syncthreads();
         for (int c0 = 0; c0 < dm.P; c0 += G) {
             stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g, slot, G, s_w,
@@ -399,7 +401,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
     float delta;
     {
         float of[DC];
-        load_chunk<S, DC>((const char *)q_ + roff, qf);
+        load_chunk<S, DC>((const char *)q_ + (dm.q_row(pb.b, (int)s1, pb.h, (int)l) + lane_elem) * S::kBytes, qf);
         load_chunk<S, DC>((const char *)dout_ + roff, dof);
         if constexpr (kPacked) load_packed<S, DC>((const char *)dout_ + roff, dop);
         load_chunk<S, DC>((const char *)out_ + roff, of);
@@ -412,10 +414,11 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
     if (stats_ && have && g == 0) stats_[row] = make_float2(lse, delta);     // null: a launch of its own does it
 
     for (int s2 = 0; s2 < dm.V; ++s2) {
-        const size_t plane = (((size_t)pb.b * dm.V + s2) * dm.H + pb.h) * (size_t)dm.L * D * S::kBytes;
+        const size_t plane = dm.kv_plane(pb.b, s2, pb.h) * S::kBytes;
+        const unsigned px_bytes = (unsigned)dm.kv_sl * S::kBytes;
         __syncthreads();
-        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, 0);
-        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, 1);
+        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, px_bytes, 0);
+        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, px_bytes, 1);
         __syncthreads();
         for (int c0 = 0; c0 < dm.P; c0 += G) {
             const int my_n = stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g,

@@ -67,9 +67,9 @@ __global__ __launch_bounds__(kTileWaves *kWave) void bwd_dkdv_tile_kernel(
     for (int i = threadIdx.x; i < 2 * tile_elems; i += blockDim.x) tileK[i] = 0.0;
     __syncthreads();
 
-    const size_t plane_base = (((size_t)b * dm.V + s2) * dm.H + h) * (size_t)dm.L * D;   // elements
-    const char *kb = (const char *)k_ + plane_base * S::kBytes;
-    const char *vb = (const char *)v_ + plane_base * S::kBytes;
+    const size_t plane_base = (((size_t)b * dm.V + s2) * dm.H + h) * (size_t)dm.L * D;   // elements in dk/dv
+    const char *kb = (const char *)k_ + dm.kv_plane(b, s2, h) * S::kBytes;
+    const char *vb = (const char *)v_ + dm.kv_plane(b, s2, h) * S::kBytes;
     const int g = lane % G, slot = lane / G, lane_elem = g * DC;
     const float qscale = dm.sm_scale * kLog2e;
     const float2 *coords = (const float2 *)coords_;
@@ -102,14 +102,14 @@ __global__ __launch_bounds__(kTileWaves *kWave) void bwd_dkdv_tile_kernel(
             wave_lds_sync();
             if (mine) {
                 s_w[pos] = make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]);
-                s_e[pos] = make_uint4((unsigned)(tp.pix[0] * D) * S::kBytes, (unsigned)(tp.pix[1] * D) * S::kBytes,
-                                      (unsigned)(tp.pix[2] * D) * S::kBytes, (unsigned)(tp.pix[3] * D) * S::kBytes);
+                s_e[pos] = make_uint4((unsigned)(tp.pix[0] * dm.kv_sl) * S::kBytes, (unsigned)(tp.pix[1] * dm.kv_sl) * S::kBytes,
+                                      (unsigned)(tp.pix[2] * dm.kv_sl) * S::kBytes, (unsigned)(tp.pix[3] * dm.kv_sl) * S::kBytes);
                 s_loc[pos] = ((tp.y0 - ya) * tg.lw + (tp.x0 - xa)) * D;   // tile-local offset of tap 00
             }
             wave_lds_sync();
             if (!row_loaded) {
                 const size_t roff = (row * D + lane_elem) * S::kBytes;
-                load_chunk<S, DC>((const char *)q_ + roff, qf);
+                load_chunk<S, DC>((const char *)q_ + (dm.q_row(b, s1, h, l) + lane_elem) * S::kBytes, qf);
                 load_chunk<S, DC>((const char *)dout_ + roff, dof);
                 const float2 ld = stats_[row];
                 lse = ld.x;

@@ -24,6 +24,7 @@ FLAG_DETERMINISTIC = 1
 FLAG_COORDS_GRAD = 2
 FLAG_SINGLE_STREAM = 4
 ERR_SCRATCH = 8
+ERR_BAD_STRIDES = 9
 NOALLOC_SCRATCH_BYTES = 32 << 20
 
 _lib = None
@@ -44,14 +45,15 @@ def load():
             "There is no fallback path for the fused operator.")
     lib = ctypes.CDLL(LIB_PATH)
     vp, i, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
-    dims = [i, i, i, i, i, i, i, f, vp]            # B V H Himg Wimg D P sm_scale stream
+    ll = ctypes.POINTER(ctypes.c_longlong)
+    dims = [i, i, i, i, i, i, i, f, ll, vp]        # B V H Himg Wimg D P sm_scale strides stream
     u = ctypes.c_uint
     for sfx in ("f32", "bf16", "f16"):
         fwd = getattr(lib, "dsdpa_fwd_" + sfx)
         fwd.argtypes = [vp] * 7 + dims          # q k v coords out lse workspace
         fwd.restype = i
         bwd = getattr(lib, "dsdpa_bwd_" + sfx)
-        bwd.argtypes = [vp] * 12 + dims[:-1] + [u, vp]   # q k v coords out lse dout dq dk dv dcoords workspace, dims, flags, stream
+        bwd.argtypes = [vp] * 12 + dims[:-1] + [u, vp]   # q k v coords out lse dout dq dk dv dcoords workspace, dims (with strides), flags, stream
         bwd.restype = i
     lib.dsdpa_fwd_noalloc.argtypes = [i] + [vp] * 6 + dims      # dtype, q k v coords out lse, dims
     lib.dsdpa_fwd_noalloc.restype = i
@@ -73,6 +75,23 @@ def load():
     lib.dsdpa_timer_collect.restype = i
     _lib = lib
     return lib
+
+
+def strides_arg(q, k, v):
+    """The `strides` argument of the entry points for q, k, v given as (B, V, H, L, D) tensors: None when all three
+    are contiguous, else a ctypes array of q's and k/v's element strides over (batch, view, head, pixel), or
+    False when the kernels cannot read the tensors in place (the head dimension is not contiguous, k and v are
+    laid out differently, or a row start is not 16-byte aligned): the caller then copies."""
+    if q.is_contiguous() and k.is_contiguous() and v.is_contiguous():
+        return None
+    align = 16 // q.element_size()
+    for t in (q, k, v):
+        st = t.stride()
+        if st[4] != 1 or t.data_ptr() % 16 or any(x % align or x < 0 for x in st[:4]) or st[3] < t.shape[4]:
+            return False
+    if k.stride() != v.stride():
+        return False
+    return (ctypes.c_longlong * 8)(*q.stride()[:4], *k.stride()[:4])
 
 
 def check(code):

@@ -19,9 +19,10 @@ Contract mirrored from ``_fused_deform_sdpa`` (``ops/triton.py:377-466``):
 Differences, all on purpose: coords are not cloned or pre-scaled (the kernels
 un-normalise), ``out``/``dq`` are not zero-filled first, no scaled copy of K is
 made, out-of-image taps follow the eager operator's per-tap zero padding
-(``ops/torch.py:14-15``) rather than ``ops/triton.py:129,135-136``, q/k/v/dout
-are made contiguous instead of asserted, and only the log-sum-exp is saved on
-top of the inputs and output.
+(``ops/torch.py:14-15``) rather than ``ops/triton.py:129,135-136``, strided
+q/k/v are read in place where the head dimension is contiguous (and copied
+otherwise) instead of asserted, dout is made contiguous, and only the
+log-sum-exp is saved on top of the inputs and output.
 """
 import torch
 
@@ -84,10 +85,15 @@ class _fused_deform_sdpa(torch.autograd.Function):
         lib = _native.load()
         B, V, H, L, D = q.shape
         P = coords.shape[-2]
-        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        # strided q, k, v are read in place where the kernels can (the reference's forward takes their strides,
+        # ops/triton.py:396-405): head dimension contiguous, rows 16-byte aligned, k and v laid out alike
+        strides = _native.strides_arg(q, k, v)
+        if strides is False:
+            q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+            strides = None
         if coords.dtype != torch.float32:
             coords = coords.float()
-        out = torch.empty_like(q)
+        out = torch.empty(q.shape, device=q.device, dtype=q.dtype)          # contiguous whatever q's layout
         lse = torch.empty((B, V, H, L), device=q.device, dtype=torch.float32)
         ws_bytes = lib.dsdpa_fwd_workspace_bytes(_DTYPE_CODE[q.dtype], B, V, H, HEIGHT, WIDTH, D, P)
         ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)     # scratch, not saved for backward
@@ -95,7 +101,7 @@ class _fused_deform_sdpa(torch.autograd.Function):
             rc = getattr(lib, "dsdpa_fwd_" + sfx)(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), coords.data_ptr(), out.data_ptr(), lse.data_ptr(),
                 ws.data_ptr() if ws_bytes else None,
-                B, V, H, HEIGHT, WIDTH, D, P, float(sm_scale), _stream_ptr(q.device))
+                B, V, H, HEIGHT, WIDTH, D, P, float(sm_scale), strides, _stream_ptr(q.device))
         _native.check(rc)
         ctx.save_for_backward(q, k, v, coords, out, lse)
         ctx.sm_scale = float(sm_scale)
@@ -112,7 +118,8 @@ class _fused_deform_sdpa(torch.autograd.Function):
         do = do.contiguous()
         if do.dtype != q.dtype:
             do = do.to(q.dtype)
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dq, dk, dv = (torch.empty(q.shape, device=q.device, dtype=q.dtype) for _ in range(3))
+        strides = _native.strides_arg(q, k, v)          # (what forward saved: contiguous, or readable in place)
         dcoords = torch.empty_like(coords) if ctx.coords_grad and ctx.needs_input_grad[3] else None
         # torch.use_deterministic_algorithms(True) selects the bitwise reproducible backward
         flags = _native.FLAG_DETERMINISTIC if torch.are_deterministic_algorithms_enabled() else 0
@@ -130,7 +137,7 @@ class _fused_deform_sdpa(torch.autograd.Function):
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), coords.data_ptr(), out.data_ptr(), lse.data_ptr(),
                 do.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                 dcoords.data_ptr() if dcoords is not None else None, ws.data_ptr(),
-                B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P, ctx.sm_scale, flags, _stream_ptr(q.device))
+                B, V, H, ctx.HEIGHT, ctx.WIDTH, D, P, ctx.sm_scale, strides, flags, _stream_ptr(q.device))
         _native.check(rc)
         grads = (dq, dk, dv, dcoords, None, None, None)
         return grads if ctx.n_inputs == 7 else grads + (None,)

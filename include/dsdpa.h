@@ -13,8 +13,9 @@
  *   - plain pointers and sizes only; every pointer is DEVICE memory owned by
  *     the caller; nothing is allocated or freed by the library (scratch
  *     memory comes in as the `workspace` arguments);
- *   - tensors are contiguous, row-major:
- *         q, k, v, out, dout, dq, dk, dv : [B][V][H][L][D],  L = Himg*Wimg
+ *   - tensors are row-major:
+ *         q, k, v, out, dout, dq, dk, dv : [B][V][H][L][D],  L = Himg*Wimg, contiguous -- except that the
+ *                  inputs q, k, v may be strided over (batch, view, head, pixel), see `strides` below
  *         coords : [B][V][L][V][P][2] float32, (x, y) normalised to [0, 1],
  *                  x along WIDTH (columns), y along HEIGHT (rows); shared by
  *                  all heads (ops/torch.py:10, ops/triton.py:51)
@@ -31,6 +32,12 @@
  *     enqueued on `stream` after it (the backward forks part of its work onto a
  *     second stream of the library's and joins it again, see
  *     DSDPA_FLAG_SINGLE_STREAM; a capture of `stream` records both);
+ *   - `strides` (a HOST pointer, read during the call) is NULL when q, k and v are contiguous, or holds 8
+ *     element strides: q's over (batch, view, head, pixel), then those shared by k and v. The head dimension
+ *     itself must be contiguous and every row start a multiple of 16 bytes (DSDPA_ERR_BAD_STRIDES). The
+ *     reference's forward takes the strides of q, k, v (ops/triton.py:396-405); its backward asserts that
+ *     they are equal (ops/triton.py:425-426), which is not required here. A permuted projection output
+ *     (B, V, L, H, D) -> (B, V, H, L, D) is read in place, without a copy;
  *   - D (head dim) must be one of 16, 32, 64, 128, 256 (ops/triton.py:386);
  *   - every entry point returns 0 on success or a DSDPA_ERR_* code, never
  *     throws, and is re-entrant; the only process-wide state is the kernel-path
@@ -58,7 +65,8 @@ enum {
     DSDPA_ERR_HIP = 5,            /* a HIP launch failed; see dsdpa_last_hip_error()      */
     DSDPA_ERR_DTYPE = 6,          /* unknown dtype code                                   */
     DSDPA_ERR_UNSUPPORTED = 7,    /* unknown flag bit, or DSDPA_FLAG_DETERMINISTIC with dcoords */
-    DSDPA_ERR_SCRATCH = 8         /* dsdpa_fwd_noalloc: the shape needs more than DSDPA_NOALLOC_SCRATCH_BYTES */
+    DSDPA_ERR_SCRATCH = 8,        /* dsdpa_fwd_noalloc: the shape needs more than DSDPA_NOALLOC_SCRATCH_BYTES */
+    DSDPA_ERR_BAD_STRIDES = 9     /* strides: head dimension not contiguous, or a row start not 16-byte aligned */
 };
 
 /* Storage types (accumulation is always fp32). Mirrors the reference's dtype
@@ -78,15 +86,15 @@ enum { DSDPA_F32 = 0, DSDPA_BF16 = 1, DSDPA_F16 = 2 };
 int dsdpa_fwd_f32(const float *q, const float *k, const float *v, const float *coords,
                   float *out, float *lse, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
-                  float sm_scale, void *stream);
+                  float sm_scale, const long long *strides, void *stream);
 int dsdpa_fwd_bf16(const void *q, const void *k, const void *v, const float *coords,
                    void *out, float *lse, void *workspace,
                    int B, int V, int H, int Himg, int Wimg, int D, int P,
-                   float sm_scale, void *stream);
+                   float sm_scale, const long long *strides, void *stream);
 int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coords,
                   void *out, float *lse, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
-                  float sm_scale, void *stream);
+                  float sm_scale, const long long *strides, void *stream);
 
 /*
  * Forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
@@ -103,7 +111,7 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
 int dsdpa_fwd_noalloc(int dtype, const void *q, const void *k, const void *v, const float *coords,
                       void *out, float *lse,
                       int B, int V, int H, int Himg, int Wimg, int D, int P,
-                      float sm_scale, void *stream);
+                      float sm_scale, const long long *strides, void *stream);
 
 /* Flags of the backward. The reference has one backward, with float atomics (ops/triton.py:345-360).
  * DSDPA_FLAG_DETERMINISTIC: bitwise reproducible dq, dk, dv: the samples of every bilinear cell are
@@ -146,17 +154,17 @@ int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *c
                   const float *out, const float *lse, const float *dout,
                   float *dq, float *dk, float *dv, float *dcoords, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
-                  float sm_scale, unsigned flags, void *stream);
+                  float sm_scale, const long long *strides, unsigned flags, void *stream);
 int dsdpa_bwd_bf16(const void *q, const void *k, const void *v, const float *coords,
                    const void *out, const float *lse, const void *dout,
                    void *dq, void *dk, void *dv, float *dcoords, void *workspace,
                    int B, int V, int H, int Himg, int Wimg, int D, int P,
-                   float sm_scale, unsigned flags, void *stream);
+                   float sm_scale, const long long *strides, unsigned flags, void *stream);
 int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coords,
                   const void *out, const float *lse, const void *dout,
                   void *dq, void *dk, void *dv, float *dcoords, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P,
-                  float sm_scale, unsigned flags, void *stream);
+                  float sm_scale, const long long *strides, unsigned flags, void *stream);
 
 /* Bytes of device workspace dsdpa_fwd_* needs for a storage dtype: 20 bytes per coordinate pair when the
  * K and V planes of one view fit in LDS (the staged kernels), else 0; 0 also if an argument is invalid.

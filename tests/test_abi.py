@@ -29,9 +29,9 @@ def test_header_symbols_all_exported():
 
 def test_version_and_error_strings():
     lib = _native.load()
-    assert lib.dsdpa_version() >= 100
+    assert lib.dsdpa_version() >= 200
     assert lib.dsdpa_error_string(0) == b"ok"
-    for code in range(1, 7):
+    for code in range(1, 10):
         assert len(lib.dsdpa_error_string(code)) > 3
     assert b"unknown" in lib.dsdpa_error_string(99)
 
@@ -85,22 +85,31 @@ def test_argument_validation_before_launch():
     """Bad arguments are rejected with an error code before anything touches the GPU."""
     lib = _native.load()
     fake = ctypes.c_void_p(0x1000)   # never dereferenced: validation fails first
-    ok_dims = (1, 2, 2, 3, 4, 32, 2, 0.5, None)
-    bwd_dims = (1, 2, 2, 3, 4, 32, 2, 0.5, 0, None)          # ... sm_scale, flags, stream
+    ok_dims = (1, 2, 2, 3, 4, 32, 2, 0.5, None, None)              # ... sm_scale, strides, stream
+    bwd_dims = (1, 2, 2, 3, 4, 32, 2, 0.5, None, 0, None)    # ... sm_scale, strides, flags, stream
     assert lib.dsdpa_fwd_f32(None, fake, fake, fake, fake, fake, fake, *ok_dims) == 1
     assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, None, *ok_dims) == 1    # this shape needs the workspace
-    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 0, 2, 2, 3, 4, 32, 2, 0.5, None) == 2
-    assert lib.dsdpa_fwd_bf16(fake, fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 48, 2, 0.5, None) == 3
-    assert lib.dsdpa_fwd_f16(fake, fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 8, 2, 0.5, None) == 3
-    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 1, 64, 64, 1024, 1024, 256, 2, 0.5, None) == 4
+    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 0, 2, 2, 3, 4, 32, 2, 0.5, None, None) == 2
+    assert lib.dsdpa_fwd_bf16(fake, fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 48, 2, 0.5, None, None) == 3
+    assert lib.dsdpa_fwd_f16(fake, fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 8, 2, 0.5, None, None) == 3
+    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 1, 64, 64, 1024, 1024, 256, 2, 0.5, None, None) == 4
+    # strides (host array: q's then k/v's element strides over batch, view, head, pixel)
+    ll8 = ctypes.c_longlong * 8
+    L, D = 12, 32
+    contiguous = ll8(2 * 2 * L * D, 2 * L * D, L * D, D, 2 * 2 * L * D, 2 * L * D, L * D, D)
+    odd_row = ll8(2 * 2 * L * D, 2 * L * D, L * D, D + 2, 2 * 2 * L * D, 2 * L * D, L * D, D)     # rows not 16-byte aligned
+    short_row = ll8(2 * 2 * L * D, 2 * L * D, L * D, D - 4, 2 * 2 * L * D, 2 * L * D, L * D, D)   # rows overlap
+    assert lib.dsdpa_fwd_f32(None, fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 32, 2, 0.5, contiguous, None) == 1
+    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 32, 2, 0.5, odd_row, None) == 9
+    assert lib.dsdpa_fwd_f32(fake, fake, fake, fake, fake, fake, fake, 1, 2, 2, 3, 4, 32, 2, 0.5, short_row, None) == 9
     # backward: the workspace is required
     args = [fake] * 10
     assert lib.dsdpa_bwd_bf16(*args, None, None, *bwd_dims) == 1
     assert lib.dsdpa_bwd_f32(*args, fake, None, *bwd_dims) == 1
     assert lib.dsdpa_bwd_f32(*args[:9], None, None, fake, *bwd_dims) == 1
-    assert lib.dsdpa_bwd_f32(*args, None, fake, 1, 2, 2, 3, 4, 33, 2, 0.5, 0, None) == 3     # dcoords is optional
-    assert lib.dsdpa_bwd_f32(*args, None, fake, 1, 2, 2, 3, 4, 32, 2, 0.5, 8, None) == 7     # unknown flag
-    assert lib.dsdpa_bwd_f32(*args, fake, fake, 1, 2, 2, 3, 4, 32, 2, 0.5, _native.FLAG_DETERMINISTIC, None) == 7
+    assert lib.dsdpa_bwd_f32(*args, None, fake, 1, 2, 2, 3, 4, 33, 2, 0.5, None, 0, None) == 3     # dcoords is optional
+    assert lib.dsdpa_bwd_f32(*args, None, fake, 1, 2, 2, 3, 4, 32, 2, 0.5, None, 8, None) == 7     # unknown flag
+    assert lib.dsdpa_bwd_f32(*args, fake, fake, 1, 2, 2, 3, 4, 32, 2, 0.5, None, _native.FLAG_DETERMINISTIC, None) == 7
 
 
 def test_path_selector():

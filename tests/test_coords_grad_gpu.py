@@ -136,7 +136,7 @@ def test_dcoords_without_the_workspace_flag_matches_with_it():
     fws = torch.empty(max(lib.dsdpa_fwd_workspace_bytes(0, B, V, H, Himg, Wimg, D, P), 1), dtype=torch.uint8,
                       device="cuda")
     _native.check(lib.dsdpa_fwd_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out.data_ptr(),
-                                    lse.data_ptr(), fws.data_ptr(), B, V, H, Himg, Wimg, D, P, 0.3, None))
+                                    lse.data_ptr(), fws.data_ptr(), B, V, H, Himg, Wimg, D, P, 0.3, None, None))
     res = {}
     for flags in (0, _native.FLAG_COORDS_GRAD):
         nbytes = lib.dsdpa_bwd_workspace_bytes(0, B, V, H, Himg, Wimg, D, P, flags)
@@ -144,7 +144,7 @@ def test_dcoords_without_the_workspace_flag_matches_with_it():
         dq, dk, dv, dc = (torch.full_like(t, float("nan")) for t in (q, k, v, c))
         _native.check(lib.dsdpa_bwd_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out.data_ptr(),
                                         lse.data_ptr(), do.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-                                        dc.data_ptr(), ws.data_ptr(), B, V, H, Himg, Wimg, D, P, 0.3, flags, None))
+                                        dc.data_ptr(), ws.data_ptr(), B, V, H, Himg, Wimg, D, P, 0.3, None, flags, None))
         torch.cuda.synchronize()
         res[flags] = (nbytes, dq.cpu(), dc.cpu())
     assert res[_native.FLAG_COORDS_GRAD][0] > res[0][0]

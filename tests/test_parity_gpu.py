@@ -164,7 +164,7 @@ def test_lse_through_c_abi():
                      dtype=torch.uint8)
     assert ws.numel() > 0
     rc = lib.dsdpa_fwd_f32(qg.data_ptr(), kg.data_ptr(), vg.data_ptr(), cg.data_ptr(), out.data_ptr(),
-                           lse.data_ptr(), ws.data_ptr(), 2, 3, 2, 6, 4, 32, 23, 0.2,
+                           lse.data_ptr(), ws.data_ptr(), 2, 3, 2, 6, 4, 32, 23, 0.2, None,
                            torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
@@ -211,6 +211,91 @@ def test_reentrant_backward_and_noncontiguous_inputs():
     assert rel(out, ro) < 1e-4
     for got, again, ref in zip((qg.grad, kg.grad, vg.grad), g1, (rdq, rdk, rdv)):
         assert rel(got, ref) < 1e-3 and rel(again, ref) < 1e-3
+
+
+# ------------------------------------------------------------------ strided q, k, v
+# The reference's forward takes the strides of q, k, v (ops/triton.py:396-405). Here q, k, v with a contiguous
+# head dimension are read in place: the two layouts a model produces without a copy -- a projection output
+# (B, V, L, H, D) permuted to (B, V, H, L, D), and the three slices of a fused (B, V, L, 3, H, D) projection.
+STRIDED = [
+    # seed B  V  H  Himg Wimg D    P   layout
+    (61, 2, 3, 2, 6, 4, 32, 23, "permuted"),      # planes in LDS
+    (62, 1, 2, 3, 5, 7, 64, 9, "fused-qkv"),
+    (63, 1, 2, 2, 40, 40, 64, 6, "permuted"),     # planes too large for LDS: gather kernels
+    (64, 1, 2, 2, 24, 20, 32, 64, "fused-qkv"),   # 64 samples per view: chunks per view, window mode
+]
+
+
+def _strided_inputs(seed, B, V, H, L, D, layout, dtype):
+    g = torch.Generator().manual_seed(seed)
+    if layout == "permuted":
+        base = [torch.randn(B, V, L, H, D, generator=g).to(dtype).cuda() for _ in range(3)]
+        return [t.permute(0, 1, 3, 2, 4) for t in base]
+    qkv = torch.randn(B, V, L, 3, H, D, generator=g).to(dtype).cuda()
+    return [qkv[:, :, :, i].permute(0, 1, 3, 2, 4) for i in range(3)]
+
+
+@pytest.mark.parametrize("path", sorted(PATHS))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("case", STRIDED, ids=[f"t{c[0]}" for c in STRIDED])
+def test_strided_inputs_read_in_place(case, dtype, path):
+    seed, B, V, H, Himg, Wimg, D, P, layout = case
+    say(f"[case] strided seed={seed} B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} {layout} {dtype} path={path}")
+    L = Himg * Wimg
+    q, k, v = _strided_inputs(seed, B, V, H, L, D, layout, dtype)
+    assert not q.is_contiguous() and q.stride(-1) == 1
+    g = torch.Generator().manual_seed(seed + 100)
+    c = (torch.rand(B, V, L, V, P, 2, generator=g) * 1.2 - 0.1).cuda()
+    if P >= 64:
+        c = (0.5 + 0.05 * torch.randn(B, V, L, V, P, 2, generator=g)).cuda()
+    do = torch.randn(B, V, H, L, D, generator=g).to(dtype).cuda()
+    qg, kg, vg = (t.detach().requires_grad_(True) for t in (q, k, v))
+    scale = 1.0 / math.sqrt(D)
+    prev = _native.set_path(PATHS[path])
+    try:
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        before = torch.cuda.memory_allocated()
+        out = deform_sdpa_triton(qg, kg, vg, c, Wimg, Himg, scale)
+        torch.cuda.synchronize()
+        fwd_extra = torch.cuda.max_memory_allocated() - before
+        out.backward(do)
+        torch.cuda.synchronize()
+    finally:
+        _native.set_path(prev)
+    # no copy of q, k, v was made: the forward allocated out, lse and its workspace, nothing tensor-sized beyond
+    lib = _native.load()
+    code = _native.DSDPA_F32 if dtype == torch.float32 else _native.DSDPA_BF16
+    ws = lib.dsdpa_fwd_workspace_bytes(code, B, V, H, Himg, Wimg, D, P)
+    tensor_bytes = q.numel() * q.element_size()
+    assert fwd_extra < tensor_bytes + q.numel() // D * 4 + ws + tensor_bytes // 2 + 4096, (fwd_extra, tensor_bytes, ws)
+    assert out.is_contiguous() and qg.grad.shape == q.shape
+    ro, _, rdq, rdk, rdv = oracle_all(q.cpu(), k.cpu(), v.cpu(), c.cpu(), do.cpu(), Wimg, Himg, scale)
+    assert rel(out, ro) < TOL_FWD[dtype]
+    assert rel(qg.grad, rdq) < TOL_BWD[dtype]
+    assert rel(kg.grad, rdk) < TOL_BWD[dtype]
+    assert rel(vg.grad, rdv) < TOL_BWD[dtype]
+
+
+def test_unreadable_layouts_are_copied():
+    """A head dimension that is not contiguous, or rows that are not 16-byte aligned, cannot be read in place: the
+    operator copies (the reference would read them through its strides; same results)."""
+    say("[case] strided layouts that need a copy")
+    g = torch.Generator().manual_seed(65)
+    B, V, H, Himg, Wimg, D, P = 1, 2, 2, 4, 5, 32, 6
+    L = Himg * Wimg
+    wide = torch.randn(B, V, H, L, 2 * D, generator=g).cuda()
+    q = wide[..., ::2]                                      # head dimension strided
+    k = torch.randn(B, V, H, L, D + 2, generator=g).cuda()[..., 2:]     # rows start 8 bytes off a 16-byte boundary
+    v = torch.randn(B, V, H, L, D, generator=g).cuda()
+    c = torch.rand(B, V, L, V, P, 2, generator=g).cuda()
+    do = torch.randn(B, V, H, L, D, generator=g).cuda()
+    qg, kg, vg = (t.detach().requires_grad_(True) for t in (q, k, v))
+    out = deform_sdpa_triton(qg, kg, vg, c, Wimg, Himg, 0.3)
+    out.backward(do)
+    torch.cuda.synchronize()
+    ro, _, rdq, rdk, rdv = oracle_all(q.cpu(), k.cpu(), v.cpu(), c.cpu(), do.cpu(), Wimg, Himg, 0.3)
+    assert rel(out, ro) < 1e-4 and rel(qg.grad, rdq) < 1e-3 and rel(kg.grad, rdk) < 1e-3 and rel(vg.grad, rdv) < 1e-3
 
 
 # ------------------------------------------------------------------ the five named workloads

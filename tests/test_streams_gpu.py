@@ -50,10 +50,10 @@ def c_abi_backward(q, k, v, c, do, Himg, Wimg, flags, stream=None):
     dq, dk, dv = (torch.full_like(t, float("nan")) for t in (q, k, v))
     _native.check(getattr(lib, "dsdpa_fwd_" + sfx)(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out.data_ptr(), lse.data_ptr(), fws.data_ptr(),
-        B, V, H, Himg, Wimg, D, P, 0.3, sp))
+        B, V, H, Himg, Wimg, D, P, 0.3, None, sp))
     _native.check(getattr(lib, "dsdpa_bwd_" + sfx)(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out.data_ptr(), lse.data_ptr(), do.data_ptr(),
-        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), None, ws.data_ptr(), B, V, H, Himg, Wimg, D, P, 0.3, flags, sp))
+        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), None, ws.data_ptr(), B, V, H, Himg, Wimg, D, P, 0.3, None, flags, sp))
     return out, dq, dk, dv, (fws, ws, lse)
 
 

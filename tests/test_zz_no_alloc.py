@@ -34,12 +34,12 @@ def _both(lib, shape, dtype, seed):
     lse_b = lse_a.clone()
     _native.check(getattr(lib, "dsdpa_fwd_" + SFX[dtype])(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out_a.data_ptr(), lse_a.data_ptr(), ws.data_ptr(),
-        B, V, H, Himg, Wimg, D, P, 0.25, st))
+        B, V, H, Himg, Wimg, D, P, 0.25, None, st))
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
     _native.check(lib.dsdpa_fwd_noalloc(
         CODE[dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out_b.data_ptr(), lse_b.data_ptr(),
-        B, V, H, Himg, Wimg, D, P, 0.25, st))
+        B, V, H, Himg, Wimg, D, P, 0.25, None, st))
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
     return need, (out_a, lse_a), (out_b, lse_b)
@@ -74,7 +74,7 @@ def test_noalloc_forward_without_workspace_and_refusal():
     out = torch.full_like(q, 7.0)
     lse = torch.zeros(B, V, H, Himg * Wimg, device="cuda")
     rc = lib.dsdpa_fwd_noalloc(_native.DSDPA_F32, q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(),
-                               out.data_ptr(), lse.data_ptr(), *shape, 0.25, None)
+                               out.data_ptr(), lse.data_ptr(), *shape, 0.25, None, None)
     torch.cuda.synchronize()
     assert rc == _native.ERR_SCRATCH
     assert (out == 7.0).all()
