@@ -29,6 +29,16 @@ constexpr int kCellWaves = 4;
 
 __device__ __forceinline__ int cell_of(const Taps &tp, int Wimg) { return (tp.y0 + 1) * (Wimg + 1) + (tp.x0 + 1); }
 
+// Fractional position of a sample inside its cell: the bilinear weights are (1-fx)(1-fy), fx(1-fy), (1-fx)fy, fx*fy.
+// The binning pass stores it beside the sample id (same order), so that the dk/dv kernel reads it in list order
+// instead of gathering the coordinate pair again (a random 8-byte read per entry, per head).
+__device__ __forceinline__ float2 cell_fraction(float2 xy, const Dims &dm)
+{
+    const float x = ((xy.x * 2.0f - 1.0f) + 1.0f) * ((float)(dm.Wimg - 1) * 0.5f);
+    const float y = ((xy.y * 2.0f - 1.0f) + 1.0f) * ((float)(dm.Himg - 1) * 0.5f);
+    return make_float2(x - floorf(x), y - floorf(y));
+}
+
 __device__ __forceinline__ bool taps_any(const Taps &tp)
 {
     return (tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f);
@@ -36,11 +46,12 @@ __device__ __forceinline__ bool taps_any(const Taps &tp)
 
 // One thread per coordinate pair, in memory order (b, s1, l, s2, p).
 // mode 0: count[(b*V+s2)*NC + cell] += 1
-// mode 1: sorted[(b*V+s2)*M + cursor[(b*V+s2)*NC + cell]++] = (s1*L + l)*P + p
+// mode 1: sorted[(b*V+s2)*M + cursor[(b*V+s2)*NC + cell]++] = (s1*L + l)*P + p, and frac[same] = its (fx, fy)
 template <int MODE>
 __global__ __launch_bounds__(kBinThreads) void bin_samples_kernel(const float *__restrict__ coords_, Dims dm,
                                                                   int NC, unsigned *__restrict__ counters,
-                                                                  unsigned *__restrict__ sorted)
+                                                                  unsigned *__restrict__ sorted,
+                                                                  float2 *__restrict__ frac)
 {
     const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
     const long long i = (long long)blockIdx.x * kBinThreads + threadIdx.x;
@@ -62,6 +73,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_samples_kernel(const float *_
         const unsigned pos = atomicAdd(ctr, 1u);
         const size_t M = (size_t)dm.V * dm.L * dm.P;
         sorted[grp * M + pos] = (unsigned)ql * (unsigned)dm.P + (unsigned)p;
+        frac[grp * M + pos] = cell_fraction(xy, dm);
     }
 }
 
@@ -78,7 +90,7 @@ constexpr int kBinLdsThreads = 1024;
 template <int MODE>
 __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
     const float *__restrict__ coords_, Dims dm, int NC, int lchunk, int nlc,
-    unsigned *__restrict__ counters, unsigned *__restrict__ sorted)
+    unsigned *__restrict__ counters, unsigned *__restrict__ sorted, float2 *__restrict__ frac)
 {
     extern __shared__ unsigned s_hist[];                 // [V][NC]; mode 1 adds [V][NC] bases
     unsigned *s_base = s_hist + (size_t)dm.V * NC;
@@ -119,6 +131,7 @@ __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
             const int hidx = s2 * NC + cell_of(tp, dm.Wimg);
             const unsigned pos = s_base[hidx] + atomicAdd(&s_hist[hidx], 1u);
             sorted[((size_t)b * dm.V + s2) * M + pos] = ((unsigned)s1 * dm.L + l) * (unsigned)dm.P + (unsigned)p;
+            frac[((size_t)b * dm.V + s2) * M + pos] = cell_fraction(xy, dm);
         }
     }
 }
@@ -263,11 +276,11 @@ struct CellGrid {
 };
 
 template <typename S, int D, int DC>
-__global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 4) : (S::kBytes == 2 ? 3 : 2)) void bwd_dkdv_cell_kernel(
+__global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >= 64 ? 5 : 4) : (S::kBytes == 2 ? 3 : 2)) void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float2 *__restrict__ stats_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
-    const uint2 *__restrict__ items, const unsigned *__restrict__ nitems,
+    const float2 *__restrict__ frac, const uint2 *__restrict__ items, const unsigned *__restrict__ nitems,
     float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC, CellGrid cg)
 {
     constexpr int G = D / DC;
@@ -277,6 +290,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 
     __shared__ unsigned s_row[kCellWaves][kWave];           // byte offset of the entry's query row in dout (and its (lse, delta))
     __shared__ unsigned s_qrow[kCellWaves][kWave];          // ... in q (which may be strided)
     __shared__ float2 s_f[S::kBytes == 2 ? kCellWaves : 1][kWave];          // 16-bit storage: (fx, fy) of the entry
+    __shared__ __attribute__((aligned(16))) float s_flush[kCellWaves][4 * D];                 // the flush: four rows of dk, then of dv
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const unsigned work = (unsigned)xcd_logical_block(blockIdx.x, gridDim.x) * kCellWaves + wave;
@@ -384,25 +398,32 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 
     const unsigned view_rows = (unsigned)dm.H * (unsigned)dm.L;
     const float2 *coords = reinterpret_cast<const float2 *>(coords_);
 
-    // Walk the list 64 entries at a time. Sample ids are fetched one chunk ahead
-    // (the coordinate load depends on them).
+    // Walk the list 64 entries at a time. Sample ids, and the samples' positions in the cell when the binning
+    // pass left them beside the ids (frac; null after the lists were reordered), are fetched one chunk ahead.
+    const float2 *fracl = frac ? frac + grp * M : nullptr;
     auto load_id = [&](unsigned cstart) -> unsigned {
         return cstart < hi ? list[min(cstart + (unsigned)lane, hi - 1u)] : 0u;
     };
+    auto load_frac = [&](unsigned cstart) -> float2 {
+        return (fracl && cstart < hi) ? fracl[min(cstart + (unsigned)lane, hi - 1u)] : make_float2(0.f, 0.f);
+    };
     unsigned id_nxt = load_id(lo);
+    float2 ff_nxt = load_frac(lo);
     for (unsigned c0 = lo; c0 < hi; c0 += kWave) {
         const unsigned id = id_nxt;
+        float2 ff = ff_nxt;
         id_nxt = load_id(c0 + kWave);
+        ff_nxt = load_frac(c0 + kWave);
         // one list entry per lane: weights and query row
         const unsigned ql = dm.divP.div(id), p = id - ql * (unsigned)dm.P;     // ql = s1*L + l
         const unsigned s1 = dm.divL.div(ql), l = ql - s1 * (unsigned)dm.L;
-        const size_t ci = (((size_t)b * dm.V * dm.L + ql) * dm.V + s2) * (size_t)dm.P + p;
-        const float2 xy = coords[ci];
+        if (!fracl) {
+            const size_t ci = (((size_t)b * dm.V * dm.L + ql) * dm.V + s2) * (size_t)dm.P + p;
+            ff = cell_fraction(coords[ci], dm);
+        }
         // Plain bilinear weights, not masked: every sample of this list lies in this cell, whose taps
         // outside the image were loaded as zeros above and are skipped by the flush below.
-        const float x = ((xy.x * 2.0f - 1.0f) + 1.0f) * ((float)(dm.Wimg - 1) * 0.5f);
-        const float y = ((xy.y * 2.0f - 1.0f) + 1.0f) * ((float)(dm.Himg - 1) * 0.5f);
-        const float fx = x - floorf(x), fy = y - floorf(y);
+        const float fx = ff.x, fy = ff.y;
         const float gx = 1.0f - fx, gy = 1.0f - fy;
         // entries past the end of the list repeat its last sample with zero weights: they add nothing
         const bool live = c0 + (unsigned)lane < hi;
@@ -502,20 +523,9 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 
 #pragma unroll
         for (int d = 0; d < DC; ++d) { aK[tpi][d] = mK[d][tpi]; aV[tpi][d] = mV[d][tpi]; }
     }
-    // sum the NS slots, then one flush per pixel of the cell
-#pragma unroll
-    for (int off = G; off < kWave; off <<= 1) {
-#pragma unroll
-        for (int tpi = 0; tpi < 4; ++tpi) {
-#pragma unroll
-            for (int d = 0; d < DC; ++d) {
-                aK[tpi][d] += __shfl_xor(aK[tpi][d], off, kWave);
-                aV[tpi][d] += __shfl_xor(aV[tpi][d], off, kWave);
-            }
-        }
-    }
     if constexpr (!kPacked) {
-        // moments -> pixels: w00 = 1 - fx - fy + fx*fy, w01 = fx - fx*fy, w10 = fy - fx*fy, w11 = fx*fy
+        // moments -> pixels (linear, so it can be done on the slots' partial sums):
+        // w00 = 1 - fx - fy + fx*fy, w01 = fx - fx*fy, w10 = fy - fx*fy, w11 = fx*fy
 #pragma unroll
         for (int d = 0; d < DC; ++d) {
             aK[0][d] = (aK[0][d] - aK[1][d]) - (aK[2][d] - aK[3][d]);
@@ -526,22 +536,78 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 ? 5 : 
             aV[2][d] -= aV[3][d];
         }
     }
-    if (slot == 0) {
-        float *dkb = dk_acc + plane_base + lane_elem, *dvb = dv_acc + plane_base + lane_elem;
+    // Sum the NS slots. Slots that differ in lane bits below 16 are summed by butterflies (every lane ends
+    // up with the sum); the last two steps (lane bits 16 and 32) are reduce-scatters on the lane-swap
+    // instructions: a step adds the two halves and leaves each half with one half of the taps, so that in
+    // the end lane bit 16 and lane bit 32 select the tap a lane holds (G <= 16), or bit 32 the tap pair
+    // (G = 32), and all 64 lanes carry sums that go to memory.
+#pragma unroll
+    for (int off = G; off < 16; off <<= 1) {
 #pragma unroll
         for (int tpi = 0; tpi < 4; ++tpi) {
-            if (tv[tpi]) {
 #pragma unroll
-                for (int d = 0; d < DC; ++d) {
-                    float *pk = dkb + (size_t)tpix[tpi] * D + d, *pv = dvb + (size_t)tpix[tpi] * D + d;
-                    if (colour < 0) {
-                        atomicAdd(pk, aK[tpi][d]);
-                        atomicAdd(pv, aV[tpi][d]);
-                    } else {
-                        *pk += aK[tpi][d];
-                        *pv += aV[tpi][d];
-                    }
-                }
+            for (int d = 0; d < DC; ++d) {
+                aK[tpi][d] += __shfl_xor(aK[tpi][d], off, kWave);
+                aV[tpi][d] += __shfl_xor(aV[tpi][d], off, kWave);
+            }
+        }
+    }
+    static_assert(G <= 32, "at least two slots");
+    constexpr int kTapsHeld = G <= 16 ? 1 : 2;             // taps a lane holds after the reduce-scatters
+    float hK[kTapsHeld][DC], hV[kTapsHeld][DC];
+    if constexpr (G <= 16) {
+#pragma unroll
+        for (int d = 0; d < DC; ++d) {
+            // bit 16: rows {0, 1} | {2, 3}; then bit 32: first | second of the pair
+            const float k0 = swap_add_16(aK[0][d], aK[2][d]), k1 = swap_add_16(aK[1][d], aK[3][d]);
+            const float v0 = swap_add_16(aV[0][d], aV[2][d]), v1 = swap_add_16(aV[1][d], aV[3][d]);
+            hK[0][d] = swap_add_32(k0, k1);
+            hV[0][d] = swap_add_32(v0, v1);
+        }
+    } else {
+#pragma unroll
+        for (int d = 0; d < DC; ++d) {
+            hK[0][d] = swap_add_32(aK[0][d], aK[2][d]);
+            hK[1][d] = swap_add_32(aK[1][d], aK[3][d]);
+            hV[0][d] = swap_add_32(aV[0][d], aV[2][d]);
+            hV[1][d] = swap_add_32(aV[1][d], aV[3][d]);
+        }
+    }
+    // tap of hK[i] / hV[i] in this lane
+    const int held0 = G <= 16 ? ((lane >> 4) & 1) * 2 + (lane >> 5) : (lane >> 5) * 2;
+    // Through LDS into memory order: the four rows of dk (then of dv) as 4*D consecutive floats, which the
+    // wave then adds to memory 64 consecutive floats per instruction (one or two cache lines a request,
+    // where a lane adding its own DC consecutive floats would touch 64 / G lines with every instruction).
+    const bool writer = (lane & 15) < G;                     // (lanes that differ below bit 16 hold copies)
+    float *fl = s_flush[wave];
+    constexpr int kLog2D = __builtin_ctz(D);
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        wave_lds_sync();
+        if (writer) {
+#pragma unroll
+            for (int i = 0; i < kTapsHeld; ++i) {
+                float *dst = fl + (held0 + i) * D + lane_elem;
+#pragma unroll
+                for (int d = 0; d < DC; d += 4)
+                    *reinterpret_cast<float4 *>(dst + d) = which == 0
+                        ? make_float4(hK[i][d], hK[i][d + 1], hK[i][d + 2], hK[i][d + 3])
+                        : make_float4(hV[i][d], hV[i][d + 1], hV[i][d + 2], hV[i][d + 3]);
+            }
+        }
+        wave_lds_sync();
+        float *acc = (which == 0 ? dk_acc : dv_acc) + plane_base;
+#pragma unroll
+        for (int idx0 = 0; idx0 < 4 * D; idx0 += kWave) {
+            const int idx = idx0 + lane;
+            const int r = idx >> kLog2D, dd = idx & (D - 1);
+            const bool ok = ((r & 2) ? vy1 : vy0) && ((r & 1) ? vx1 : vx0);
+            const int pix = (y0 + (r >> 1)) * dm.Wimg + x0 + (r & 1);
+            const float val = fl[idx];
+            if (ok) {
+                float *pa = acc + (size_t)pix * D + dd;
+                if (colour < 0) atomicAdd(pa, val);
+                else *pa += val;
             }
         }
     }

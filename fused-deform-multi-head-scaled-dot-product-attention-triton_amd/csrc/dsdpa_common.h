@@ -383,6 +383,22 @@ __device__ __forceinline__ uint32_t wave_min_u16x2(uint32_t x)
     });
 }
 
+// Reduce-scatter steps on the lane-swap instructions of gfx950. swap_add_32(x, y): lanes 0..31 get x summed
+// over the wave's two halves (x[l] + x[l + 32]), lanes 32..63 get y summed the same way
+// (v_permlane32_swap: rows 2, 3 of the first operand change places with rows 0, 1 of the second; a row is
+// 16 lanes). swap_add_16(x, y): lanes with bit 16 clear get x[l] + x[l ^ 16], lanes with it set get y summed
+// the same way (v_permlane16_swap: odd rows of the first operand change places with even rows of the second).
+__device__ __forceinline__ float swap_add_32(float x, float y)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float swap_add_16(float x, float y)
+{
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Orders this wave's LDS writes before its later LDS reads (and the reverse):
 // waits for the wave's outstanding LDS traffic and stops the compiler from
 // moving LDS accesses across. No workgroup barrier is involved.

@@ -143,6 +143,7 @@ inline DescLayout desc_layout(size_t B, size_t V, size_t Himg, size_t Wimg, size
 //   counters B*V*NC u32                      per (batch, key view) cell counts, then fill cursors
 //   start    B*V*(NC+1) u32                  exclusive scan of the counts
 //   sorted   B*V*(V*L*P) u32                 sample ids ordered by cell
+//   frac     B*V*(V*L*P) x 8 bytes           (fx, fy) of the same samples, same order
 //   items    B*V*wmax x 8 bytes              work list of the dk/dv kernel: (cell, piece) per item
 //   nitems   B*V u32                         items per (batch, key view)
 //   acc      2*n floats                      fp32 dk/dv accumulators (16-bit storage only)
@@ -159,7 +160,7 @@ int sort_cell_lists(void *temp, size_t temp_bytes, const unsigned *ids_in, unsig
                     hipStream_t st);
 
 struct WorkspaceLayout {
-    size_t delta, counters, start, sorted, items, nitems, acc, desc, sorted2, seg, sorttmp, sorttmp_bytes, total;
+    size_t delta, counters, start, sorted, frac, items, nitems, acc, desc, sorted2, seg, sorttmp, sorttmp_bytes, total;
     DescLayout dl;
     size_t counters_bytes;
     int NC;
@@ -191,6 +192,7 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     w.counters = off; w.counters_bytes = round256(B * V * (size_t)w.NC * 4); off += w.counters_bytes;
     w.start = off; off += round256(B * V * ((size_t)w.NC + 1) * 4);
     w.sorted = off; off += round256(B * V * (V * Himg * Wimg * P) * 4);
+    w.frac = off; off += round256(B * V * (V * Himg * Wimg * P) * 8);
     work_list_geometry(V, Himg * Wimg, P, (size_t)w.NC, &w.piece, &w.wmax);
     w.items = off; off += round256(B * V * (size_t)w.wmax * 8);
     w.nitems = off; off += round256(B * V * 4);

@@ -380,6 +380,7 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
     unsigned *counters = (unsigned *)(ws + wl.counters);
     unsigned *start = (unsigned *)(ws + wl.start);
     unsigned *sorted = (unsigned *)(ws + wl.sorted);
+    float2 *frac = (float2 *)(ws + wl.frac);
     const size_t hist_bytes = (size_t)dm.V * wl.NC * sizeof(unsigned);
     // each of the three launches carries its own pair of events: the timer's slot 3 adds up their busy time
     ScopedKernelTimer t_count(3, st), t_scan(3, st), t_fill(3, st);
@@ -400,13 +401,13 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
         if (int rc = allow_full_lds(k1, lds_set[1])) return rc;
         DSDPA_LAUNCH(k0, dim3((unsigned)blocks), dim3(kBinLdsThreads), hist_bytes, st,
                               t_count.start(), t_count.stop(),
-                           coords, dm, wl.NC, lchunk, nlc, counters, sorted);
+                           coords, dm, wl.NC, lchunk, nlc, counters, sorted, frac);
         DSDPA_LAUNCH(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st,
                               t_scan.start(), t_scan.stop(), counters, start, wl.NC, wl.piece, wl.wmax,
                               (uint2 *)(ws + wl.items), (unsigned *)(ws + wl.nitems));
         DSDPA_LAUNCH(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
                               t_fill.start(), t_fill.stop(),
-                           coords, dm, wl.NC, lchunk, nlc, counters, sorted);
+                           coords, dm, wl.NC, lchunk, nlc, counters, sorted, frac);
         return check_launch();
     }
     const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
@@ -414,13 +415,13 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
     if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
     DSDPA_LAUNCH(bin_samples_kernel<0>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
                           t_count.start(), t_count.stop(),
-                       coords, dm, wl.NC, counters, sorted);
+                       coords, dm, wl.NC, counters, sorted, frac);
     DSDPA_LAUNCH(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st,
                           t_scan.start(), t_scan.stop(), counters, start, wl.NC, wl.piece, wl.wmax,
                               (uint2 *)(ws + wl.items), (unsigned *)(ws + wl.nitems));
     DSDPA_LAUNCH(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
                           t_fill.start(), t_fill.stop(),
-                       coords, dm, wl.NC, counters, sorted);
+                       coords, dm, wl.NC, counters, sorted, frac);
     return check_launch();
 }
 
@@ -428,7 +429,7 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
 template <typename S, int D>
 int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const float *coords,
                          const float2 *stats, const void *dout, const unsigned *start, const unsigned *sorted,
-                         const uint2 *items, const unsigned *nitems, unsigned piece, unsigned wmax,
+                         const float2 *frac, const uint2 *items, const unsigned *nitems, unsigned piece, unsigned wmax,
                          float *dk_acc, float *dv_acc, const Dims &dm, int NC, bool deterministic, hipStream_t st)
 {
     constexpr int DC = CellChunk<S, D>::value;
@@ -455,7 +456,7 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
         const bool first = colour <= 0, last = colour < 0 || colour == 3;
         DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
                               first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
-                              stats, dout, start, sorted, items, nitems, dk_acc, dv_acc, dm, NC, cg);
+                              stats, dout, start, sorted, frac, items, nitems, dk_acc, dv_acc, dm, NC, cg);
     }
     return check_launch();
 }
@@ -536,26 +537,22 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const float4 *desc_g = (const float4 *)(ws + wl.desc + wl.dl.g);
     const unsigned *start = (const unsigned *)(ws + wl.start);
     const unsigned *sorted = (const unsigned *)(ws + (deterministic ? wl.sorted2 : wl.sorted));
+    // (the reordered lists of the deterministic backward have no positions beside them: coordinates are read again)
+    const float2 *frac = deterministic ? nullptr : (const float2 *)(ws + wl.frac);
     // fp32 storage: dk and dv are their own accumulators; 16-bit: fp32 accumulators in the workspace
     float *dk_acc = S::kBytes == 4 ? (float *)dk : (float *)(ws + wl.acc);
     float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
     // Two sides that do not read what the other writes: tap table -> dq on the caller's stream, and clears ->
     // (lse, delta) pairs -> binning (-> list ordering) -> dk/dv on the side lane. Forked before anything is
     // enqueued; joined after the dk/dv kernel (before the casts of 16-bit storage, which need both).
-    // Shapes on the gather dq kernel (planes too large for LDS) run the binning BEFORE the fork instead: that
-    // kernel's many small workgroups fill every CU, and the binning workgroups (1024 threads, up to 135 KB of
-    // LDS) would wait beside it until it ends -- and the dk/dv kernel with them. Binning first (0.15 ms at
-    // 64x64, P = 64), the dq and the dk/dv kernel then share the GPU from the start.
+    // Only for shapes on the staged dq kernel, whose one 16-wave workgroup per CU leaves half the wave slots
+    // free. The gather dq kernel (planes too large for LDS) fills every CU with small workgroups: beside it the
+    // binning workgroups (1024 threads, up to 135 KB of LDS) wait until it ends, and with the binning done
+    // first the dq and dk/dv kernels only take turns (measured at 64x64, D = 128: 14.2 ms against 14.5 for the
+    // step, each kernel stretched to the sum of both) -- those shapes run the backward on the caller's stream.
     hipStream_t bst = st;
-    SideLane *side = cell_binned && !(flags & DSDPA_FLAG_SINGLE_STREAM) ? side_lane() : nullptr;
+    SideLane *side = cell_binned && staged && !(flags & DSDPA_FLAG_SINGLE_STREAM) ? side_lane() : nullptr;
     const size_t ncounters = cell_binned ? wl.counters_bytes / 4 : 0;
-    const bool bin_first = side && !staged;
-    if (bin_first) {
-        const ZeroJob zero_counters{{(float *)(ws + wl.counters), nullptr, nullptr, nullptr}, {ncounters, 0, 0, 0}};
-        if ((rc = zero_fill(zero_counters, st)) != DSDPA_OK) return rc;
-        if ((rc = launch_binning(coords, dm, wl, ws, st)) != DSDPA_OK) return rc;
-        if (deterministic && (rc = launch_list_ordering(dm, wl, ws, st)) != DSDPA_OK) return rc;
-    }
     SideJoin joiner;
     if (side && hipEventRecord(side->fork, st) == hipSuccess &&
         hipStreamWaitEvent(side->stream, side->fork, 0) == hipSuccess) {
@@ -565,11 +562,10 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
         joiner.pending = true;
     }
     const bool side_on = bst != st;
-    const bool binned = bin_first;                      // the cell lists are already made (or on their way on `st`)
     const size_t ndc = dcoords ? (size_t)dm.B * dm.V * dm.L * dm.N * 2 : 0;
     // what has to start at zero: on one stream everything in one job, which the tap-table launch (when
     // there is one) takes along; with the side lane the dk/dv side clears its own buffers there
-    const ZeroJob zero_all{{dk_acc, dv_acc, (float *)(ws + wl.counters), dcoords}, {n, n, binned ? 0 : ncounters, ndc}};
+    const ZeroJob zero_all{{dk_acc, dv_acc, (float *)(ws + wl.counters), dcoords}, {n, n, ncounters, ndc}};
     const ZeroJob zero_main{{dcoords, nullptr, nullptr, nullptr}, {ndc, 0, 0, 0}};
     const ZeroJob &zero = side_on ? zero_main : zero_all;
     if (staged) rc = launch_plane_descriptors(coords, dm, ws + wl.desc, wl.dl, cg_table, zero, 4, st);
@@ -577,15 +573,15 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     if (rc != DSDPA_OK) return rc;
     if (side_on) {
         // the dk/dv side: its clears, and the (lse, delta) pairs that the dq kernel otherwise writes on the way
-        const ZeroJob zero_side{{dk_acc, dv_acc, (float *)(ws + wl.counters), nullptr}, {n, n, binned ? 0 : ncounters, 0}};
+        const ZeroJob zero_side{{dk_acc, dv_acc, (float *)(ws + wl.counters), nullptr}, {n, n, ncounters, 0}};
         if ((rc = zero_fill(zero_side, bst)) != DSDPA_OK) return rc;
         const size_t lanes = (size_t)dm.rows * 4;
         hipLaunchKernelGGL((delta_kernel<S>), dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, bst, out, dout, lse,
                            stats, (size_t)dm.rows, D);
         if ((rc = check_launch()) != DSDPA_OK) return rc;
     }
-    if (cell_binned && !binned && (rc = launch_binning(coords, dm, wl, ws, bst)) != DSDPA_OK) return rc;
-    if (deterministic && !binned && (rc = launch_list_ordering(dm, wl, ws, bst)) != DSDPA_OK) return rc;
+    if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, bst)) != DSDPA_OK) return rc;
+    if (deterministic && (rc = launch_list_ordering(dm, wl, ws, bst)) != DSDPA_OK) return rc;
     float2 *dq_stats = side_on ? nullptr : stats;       // the dq kernel writes them only when dk/dv runs behind it
 #define DSDPA_BWD_CASE(DD)                                                                                      \
     case DD:                                                                                                    \
@@ -597,7 +593,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
                         : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dq_stats, dcoords,   \
                                                       dm, st);                                                  \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
-                rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, stats, dout, start, sorted,                   \
+                rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, stats, dout, start, sorted, frac,             \
                                                  (const uint2 *)(ws + wl.items),                                \
                                                  (const unsigned *)(ws + wl.nitems), wl.piece, wl.wmax, dk_acc, \
                                                  dv_acc, dm, wl.NC, deterministic, bst);                        \

@@ -143,8 +143,8 @@ enum { DSDPA_FLAG_DETERMINISTIC = 1, DSDPA_FLAG_COORDS_GRAD = 2, DSDPA_FLAG_SING
  * `workspace` must hold dsdpa_bwd_workspace_bytes(...) bytes (256-byte aligned):
  * the per-row delta = dout.out (one float per query row, the reference's `delta`,
  * ops/triton.py:430), the per-(batch, key view) ordering of the samples by
- * bilinear cell (one u32 per coordinate pair plus the cell offsets; it depends on
- * coords only and is shared by all heads) and, for bf16/fp16, the fp32 dk/dv
+ * bilinear cell (one u32 and the position inside the cell, 8 bytes, per coordinate pair, plus the cell
+ * offsets; it depends on coords only and is shared by all heads) and, for bf16/fp16, the fp32 dk/dv
  * accumulators that are rounded to the storage type at the end (fp32: dk and dv
  * are themselves the accumulators), and the same per-coordinate table as the forward's. Without
  * DSDPA_FLAG_DETERMINISTIC the accumulation order into dk/dv is not deterministic (float atomics,

@@ -51,6 +51,7 @@ def test_workspace_bytes():
     def expect(B, V, H, Himg, Wimg, D, P, storage16):
         rows, NC = B * V * H * Himg * Wimg, (Himg + 1) * (Wimg + 1)
         total = r256(rows * 8) + r256(B * V * NC * 4) + r256(B * V * (NC + 1) * 4) + r256(B * V * V * Himg * Wimg * P * 4)
+        total += r256(B * V * V * Himg * Wimg * P * 8)          # positions beside the ids
         # work list of the dk/dv kernel: items of at most `piece` list entries, (cell, piece) = 8 bytes each
         M = V * Himg * Wimg * P
         piece = (max(1024, 8 * M // NC) + 63) // 64 * 64
