@@ -25,7 +25,11 @@
 namespace dsdpa {
 
 constexpr int kBinThreads = 256;
-constexpr int kCellWaves = 4;
+// Waves per workgroup of the dk/dv kernel. One: items differ in length by orders of magnitude (a heavy
+// list's piece beside lists of a few entries), and a workgroup keeps its LDS and its place on the CU until
+// its longest wave ends -- with four waves a workgroup the SIMDs held 2.1 waves on average where the
+// registers allow 3 (64x64, 64 samples per view, clustered: 4.88 ms with four, 4.13 ms with one).
+constexpr int kCellWaves = 1;
 
 __device__ __forceinline__ int cell_of(const Taps &tp, int Wimg) { return (tp.y0 + 1) * (Wimg + 1) + (tp.x0 + 1); }
 
@@ -140,27 +144,28 @@ __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
 // start[grp*(NC+1) + c] (with the total at c = NC) and resets counters to the
 // same starts, so that the fill pass can use them as cursors.
 //
-// It also makes the dk/dv kernel's work list of this (b, s2): one item (cell, piece) per run of at most
-// `piece` consecutive entries of a non-empty cell list, in cell order -- items[grp*wmax + i], i < nitems[grp].
-// Empty cells get no item (clustered coordinates leave most of the grid empty), and a list much longer than
-// the average is cut into pieces that different waves take, so that the longest list no longer sets the
-// kernel's duration. wmax >= NC + M/piece bounds the number of items (M = entries of all lists).
+// It also makes the dk/dv kernel's work list of this (b, s2): one item (cell, first entry, end) per run of at
+// most `piece` consecutive entries of a non-empty list, in list order -- items[grp*wmax + i]; the slots after
+// the last item are marked empty (first = end). Empty lists get no item (clustered coordinates leave most
+// of the grid empty), and a list much longer than the average is cut into pieces that different waves take,
+// so that the longest list no longer sets the kernel's duration. wmax >= NC + M/piece bounds the number of
+// items (M = entries of all lists). An item carries all a wave needs to start on it: one read, where the
+// list's bounds would be a second, dependent one.
 static __global__ __launch_bounds__(1024) void bin_scan_kernel(unsigned *__restrict__ counters,
-                                                        unsigned *__restrict__ start, int NC, unsigned piece,
-                                                        unsigned wmax, uint2 *__restrict__ items,
-                                                        unsigned *__restrict__ nitems)
+                                                        unsigned *__restrict__ start, int NC,
+                                                        unsigned piece, unsigned wmax, uint4 *__restrict__ items)
 {
     __shared__ unsigned s_part[1024], s_pcs[1024];
     __shared__ unsigned s_carry, s_pcarry;
     unsigned *cnt = counters + (size_t)blockIdx.x * NC;
     unsigned *st = start + (size_t)blockIdx.x * (NC + 1);
-    uint2 *it = items + (size_t)blockIdx.x * wmax;
+    uint4 *it = items + (size_t)blockIdx.x * wmax;
     if (threadIdx.x == 0) { s_carry = 0; s_pcarry = 0; }
     __syncthreads();
     for (int base = 0; base < NC; base += 1024) {
         const int c = base + threadIdx.x;
         const unsigned v = c < NC ? cnt[c] : 0u;
-        const unsigned np = (v + piece - 1) / piece;               // pieces of this cell's list
+        const unsigned np = (v + piece - 1) / piece;               // pieces of this list
         s_part[threadIdx.x] = v;
         s_pcs[threadIdx.x] = np;
         __syncthreads();
@@ -178,17 +183,16 @@ static __global__ __launch_bounds__(1024) void bin_scan_kernel(unsigned *__restr
         if (c < NC) {
             st[c] = excl;
             cnt[c] = excl;
+            const unsigned cell = (unsigned)c;
             for (unsigned i = 0; i < np; ++i)
-                if (pexcl + i < wmax) it[pexcl + i] = make_uint2((unsigned)c, i);
+                if (pexcl + i < wmax) it[pexcl + i] = make_uint4(cell, excl + i * piece, min(excl + v, excl + (i + 1) * piece), 0u);
         }
         __syncthreads();
         if (threadIdx.x == 1023) { s_carry += s_part[1023]; s_pcarry += s_pcs[1023]; }
         __syncthreads();
     }
-    if (threadIdx.x == 0) {
-        st[NC] = s_carry;
-        nitems[blockIdx.x] = min(s_pcarry, wmax);
-    }
+    if (threadIdx.x == 0) st[NC] = s_carry;
+    for (unsigned i = min(s_pcarry, wmax) + threadIdx.x; i < wmax; i += 1024) it[i] = make_uint4(0u, 0u, 0u, 0u);
 }
 
 // Deterministic backward: begin / end of every cell list as positions in the flat id array
@@ -267,11 +271,10 @@ __device__ __forceinline__ void widen_words(const uint32_t (&w)[DC * S::kBytes /
 // two of them share a pixel, so the flush is a plain read-add-write, and the four launches, one
 // after the other, add every pixel's four contributions in a fixed order.
 // colour < 0 also switches the decode to the work list made by bin_scan_kernel: work index -> (b, h, s2, item),
-// `ncells` then being the list's capacity wmax per (b, s2); items beyond the list's length leave at once.
+// `ncells` then being the list's capacity wmax per (b, s2); empty slots leave at once.
 struct CellGrid {
     int colour, oy, ox, step, ncx, ncells;
     unsigned nwork;                         // B*H*V*ncells < 2^31
-    unsigned piece;                         // entries per work item (work-list mode)
     FastDiv div_cells, div_ncx, div_v, div_h;
 };
 
@@ -280,7 +283,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float2 *__restrict__ stats_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
-    const float2 *__restrict__ frac, const uint2 *__restrict__ items, const unsigned *__restrict__ nitems,
+    const float2 *__restrict__ frac, const uint4 *__restrict__ items,
     float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC, CellGrid cg)
 {
     constexpr int G = D / DC;
@@ -307,14 +310,12 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >
     int cy, cx, cell;
     unsigned lo, hi;
     if (colour < 0) {
-        if ((unsigned)ci >= nitems[grp]) return;
-        const uint2 item = items[grp * (size_t)cg.ncells + ci];
+        const uint4 item = items[grp * (size_t)cg.ncells + ci];              // (cell, first entry, end)
         cell = (int)item.x;
         cy = (int)cg.div_ncx.div(item.x);                      // div_ncx: by Wimg + 1 in this mode
         cx = cell - cy * (dm.Wimg + 1);
-        const unsigned l0 = start[grp * (NC + 1) + cell], l1 = start[grp * (NC + 1) + cell + 1];
-        lo = l0 + item.y * cg.piece;
-        hi = min(l1, lo + cg.piece);
+        lo = item.y;
+        hi = item.z;
     } else {
         const int cyi = (int)cg.div_ncx.div((unsigned)ci);
         cy = cyi * cg.step + cg.oy;

@@ -144,8 +144,7 @@ inline DescLayout desc_layout(size_t B, size_t V, size_t Himg, size_t Wimg, size
 //   start    B*V*(NC+1) u32                  exclusive scan of the counts
 //   sorted   B*V*(V*L*P) u32                 sample ids ordered by cell
 //   frac     B*V*(V*L*P) x 8 bytes           (fx, fy) of the same samples, same order
-//   items    B*V*wmax x 8 bytes              work list of the dk/dv kernel: (cell, piece) per item
-//   nitems   B*V u32                         items per (batch, key view)
+//   items    B*V*wmax x 16 bytes             work list of the dk/dv kernel: (cell, first entry, end) per item
 //   acc      2*n floats                      fp32 dk/dv accumulators (16-bit storage only)
 //   desc     20 bytes per coordinate pair    descriptor table (only when the plane kernels apply); 36 with
 //                                            the coordinate gradient
@@ -160,22 +159,23 @@ int sort_cell_lists(void *temp, size_t temp_bytes, const unsigned *ids_in, unsig
                     hipStream_t st);
 
 struct WorkspaceLayout {
-    size_t delta, counters, start, sorted, frac, items, nitems, acc, desc, sorted2, seg, sorttmp, sorttmp_bytes, total;
+    size_t delta, counters, start, sorted, frac, items, acc, desc, sorted2, seg, sorttmp, sorttmp_bytes, total;
     DescLayout dl;
     size_t counters_bytes;
     int NC;
     unsigned piece, wmax;       // work list of the dk/dv kernel: entries per item, items per (batch, key view)
 };
 
-// Work list of the dk/dv kernel: a cell list is cut into items of at most `piece` entries, eight times the
-// average list length over the whole cell grid (at least 1024, a multiple of 64): lists near the average
-// stay whole, the heavy ones of clustered coordinates are shared by several waves. NC + M/piece bounds the
+// Work list of the dk/dv kernel: a cell list is cut into items of at most `piece` entries, four times the
+// average list length over the whole cell grid (at least 512, a multiple of 64): lists near the average
+// stay whole, the heavy ones of clustered coordinates are shared by several waves (64x64, 64 samples per
+// view, clustered: 1024 entries a piece, 4.13 ms for the kernel; 2048: 4.35 ms, the last pieces running alone). NC + M/piece bounds the
 // number of items per (batch, key view), M = V*L*P being all its entries.
 inline void work_list_geometry(size_t V, size_t L, size_t P, size_t NC, unsigned *piece, unsigned *wmax)
 {
     const size_t M = V * L * P;
-    size_t pc = 8 * M / NC;
-    if (pc < 1024) pc = 1024;
+    size_t pc = 4 * M / NC;
+    if (pc < 512) pc = 512;
     pc = (pc + 63) / 64 * 64;
     if (pc > 0x40000000u) pc = 0x40000000u;
     *piece = (unsigned)pc;
@@ -194,8 +194,7 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     w.sorted = off; off += round256(B * V * (V * Himg * Wimg * P) * 4);
     w.frac = off; off += round256(B * V * (V * Himg * Wimg * P) * 8);
     work_list_geometry(V, Himg * Wimg, P, (size_t)w.NC, &w.piece, &w.wmax);
-    w.items = off; off += round256(B * V * (size_t)w.wmax * 8);
-    w.nitems = off; off += round256(B * V * 4);
+    w.items = off; off += round256(B * V * (size_t)w.wmax * 16);
     w.acc = off; if (storage16) off += round256(2 * rows * D * 4);
     // with the coordinate gradient the staged dq kernel needs more LDS; where it no longer fits, dq takes the
     // gather kernel and no table is needed

@@ -404,7 +404,7 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
                            coords, dm, wl.NC, lchunk, nlc, counters, sorted, frac);
         DSDPA_LAUNCH(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st,
                               t_scan.start(), t_scan.stop(), counters, start, wl.NC, wl.piece, wl.wmax,
-                              (uint2 *)(ws + wl.items), (unsigned *)(ws + wl.nitems));
+                              (uint4 *)(ws + wl.items));
         DSDPA_LAUNCH(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
                               t_fill.start(), t_fill.stop(),
                            coords, dm, wl.NC, lchunk, nlc, counters, sorted, frac);
@@ -418,7 +418,7 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
                        coords, dm, wl.NC, counters, sorted, frac);
     DSDPA_LAUNCH(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st,
                           t_scan.start(), t_scan.stop(), counters, start, wl.NC, wl.piece, wl.wmax,
-                              (uint2 *)(ws + wl.items), (unsigned *)(ws + wl.nitems));
+                              (uint4 *)(ws + wl.items));
     DSDPA_LAUNCH(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
                           t_fill.start(), t_fill.stop(),
                        coords, dm, wl.NC, counters, sorted, frac);
@@ -429,7 +429,7 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
 template <typename S, int D>
 int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const float *coords,
                          const float2 *stats, const void *dout, const unsigned *start, const unsigned *sorted,
-                         const float2 *frac, const uint2 *items, const unsigned *nitems, unsigned piece, unsigned wmax,
+                         const float2 *frac, const uint4 *items, unsigned wmax,
                          float *dk_acc, float *dv_acc, const Dims &dm, int NC, bool deterministic, hipStream_t st)
 {
     constexpr int DC = CellChunk<S, D>::value;
@@ -443,7 +443,6 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
         cg.step = colour < 0 ? 1 : 2;
         cg.ncx = (cw - cg.ox + cg.step - 1) / cg.step;
         cg.ncells = cg.ncx * ((ch - cg.oy + cg.step - 1) / cg.step);
-        cg.piece = piece;
         if (colour < 0) cg.ncells = (int)wmax;          // work-list mode: one wave per item slot
         const long long nwork = (long long)dm.B * dm.H * dm.V * cg.ncells;
         if (nwork >= 0x7fffffffll - kCellWaves) return DSDPA_ERR_TOO_LARGE;
@@ -456,7 +455,7 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
         const bool first = colour <= 0, last = colour < 0 || colour == 3;
         DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
                               first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
-                              stats, dout, start, sorted, frac, items, nitems, dk_acc, dv_acc, dm, NC, cg);
+                              stats, dout, start, sorted, frac, items, dk_acc, dv_acc, dm, NC, cg);
     }
     return check_launch();
 }
@@ -594,8 +593,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
                                                       dm, st);                                                  \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
                 rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, stats, dout, start, sorted, frac,             \
-                                                 (const uint2 *)(ws + wl.items),                                \
-                                                 (const unsigned *)(ws + wl.nitems), wl.piece, wl.wmax, dk_acc, \
+                                                 (const uint4 *)(ws + wl.items), wl.wmax, dk_acc,               \
                                                  dv_acc, dm, wl.NC, deterministic, bst);                        \
             else if (rc == DSDPA_OK)                                                                            \
                 rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, stats, dout, dk_acc, dv_acc, dm, st);         \

@@ -52,10 +52,10 @@ def test_workspace_bytes():
         rows, NC = B * V * H * Himg * Wimg, (Himg + 1) * (Wimg + 1)
         total = r256(rows * 8) + r256(B * V * NC * 4) + r256(B * V * (NC + 1) * 4) + r256(B * V * V * Himg * Wimg * P * 4)
         total += r256(B * V * V * Himg * Wimg * P * 8)          # positions beside the ids
-        # work list of the dk/dv kernel: items of at most `piece` list entries, (cell, piece) = 8 bytes each
+        # work list of the dk/dv kernel: items of at most `piece` list entries, (cell, first entry, end) in 16 bytes each
         M = V * Himg * Wimg * P
-        piece = (max(1024, 8 * M // NC) + 63) // 64 * 64
-        total += r256(B * V * (NC + M // piece + 1) * 8) + r256(B * V * 4)
+        piece = (max(512, 4 * M // NC) + 63) // 64 * 64
+        total += r256(B * V * (NC + M // piece + 1) * 16)
         total += r256(2 * rows * D * 4) if storage16 else 0
         return total + table(B, V, Himg, Wimg, D, P, storage16)
 
