@@ -92,6 +92,26 @@ inline SideLane *side_lane()
     return &s;
 }
 
+// Compute units of the current device (asked once per device; 256 when the runtime will not say).
+inline int device_cus()
+{
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> cus[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        n = 256;
+    }
+    cus[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
 inline int check_launch()
 {
     hipError_t e = hipGetLastError();

@@ -35,7 +35,7 @@
 
 namespace dsdpa {
 
-constexpr int kPlaneWaves = 16;
+constexpr int kPlaneWaves = 16;          // at most; see plane_waves for the number a launch uses
 
 // LDS addresses as plain 32-bit numbers: the tap addresses are sums and XORs of byte offsets, and a
 // pointer made from the finished number costs no instruction (adding offsets to a generic pointer to
@@ -61,7 +61,7 @@ __device__ __forceinline__ void stage_plane(unsigned char *lds, const char *src,
     constexpr int kRow = D * S::kBytes;
     constexpr int kChunksPerRow = kRow / 16;
     const int n16 = L * kChunksPerRow;
-    for (int i = threadIdx.x; i < n16; i += kPlaneWaves * kWave) {
+    for (int i = threadIdx.x; i < n16; i += (int)blockDim.x) {
         const int p = i / kChunksPerRow, q = p + 1, c = i % kChunksPerRow;
         const uint4 t = *reinterpret_cast<const uint4 *>(src + (size_t)p * px_bytes + c * 16);
         *reinterpret_cast<uint4 *>(lds + (size_t)q * 2 * kRow + ((q & 1) ^ which) * kRow + c * 16) = t;
@@ -73,7 +73,7 @@ __device__ __forceinline__ void zero_plane_pads(unsigned char *lds, int L)
 {
     constexpr int kRow = D * S::kBytes;
     constexpr int kChunks = 2 * kRow / 16;
-    for (int i = threadIdx.x; i < 2 * kChunks; i += kPlaneWaves * kWave) {
+    for (int i = threadIdx.x; i < 2 * kChunks; i += (int)blockDim.x) {
         const int pad = i / kChunks, c = i % kChunks;
         *reinterpret_cast<uint4 *>(lds + (size_t)(pad ? L + 1 : 0) * 2 * kRow + c * 16) = make_uint4(0, 0, 0, 0);
     }
@@ -93,6 +93,25 @@ __device__ __forceinline__ int paired_position(bool valid, int cls, int lane, un
     const int r = __popcll((cls ? m1 : m0) & below);
     const int pos_valid = r < np ? 2 * r + (cls ? 1 : 0) : np + r;
     return valid ? pos_valid : n0 + n1 + __popcll(mi & below);
+}
+
+// Waves per workgroup of a staged launch. The planes in LDS allow one workgroup per CU, so a launch runs in
+// rounds of `cus` workgroups, and a round lasts about as long as its workgroups have waves (the kernels are
+// bound by instruction issue) plus the staging of the planes (about two waves' worth). 16 waves is the most
+// rows per staged plane; fewer waves can mean fewer idle CUs in the last round: 2 x 8 x 16 planes of 14x14
+// pixels and 8 views make 416 workgroups of 16 waves, 1.6 rounds of 256, but 512 of 13 waves, two full
+// rounds of shorter workgroups. Picks the count with the lowest rounds * (waves + 2).
+inline int plane_waves(long long planes, int rows_per_plane, int rows_per_wave, int cus)
+{
+    int best = kPlaneWaves;
+    long long best_cost = -1;
+    for (int w = kPlaneWaves; w >= 4; --w) {
+        const long long rows = (long long)w * rows_per_wave;
+        const long long blocks = planes * ((rows_per_plane + rows - 1) / rows);
+        const long long cost = ((blocks + cus - 1) / cus) * (w + 2);
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = w; }
+    }
+    return best;
 }
 
 struct PlaneBlock {
@@ -240,7 +259,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
     int2 *s_e =
         reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kPlaneDescPlaces * 16) + wave * kPlaneDescPlaces;
 
-    const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * NS);
+    const PlaneBlock pb = decode_plane_block(dm, (int)(blockDim.x >> 6) * NS);   // (workgroups of up to kPlaneWaves waves)
     const int nq = dm.V * dm.L;
     const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
     const float qscale = dm.sm_scale * kLog2e;
@@ -381,7 +400,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
         reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kPlaneDescPlaces * 16) + wave * kPlaneDescPlaces;
     float2 *s_g = reinterpret_cast<float2 *>(smem + img_bytes + kPlaneDescBytes) + wave * kPlaneDescPlaces;   // CG only
 
-    const PlaneBlock pb = decode_plane_block(dm, kPlaneWaves * NS);
+    const PlaneBlock pb = decode_plane_block(dm, (int)(blockDim.x >> 6) * NS);   // (workgroups of up to kPlaneWaves waves)
     const int nq = dm.V * dm.L;
     const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
     const float qscale = dm.sm_scale * kLog2e;
