@@ -278,12 +278,18 @@ struct CellGrid {
     FastDiv div_cells, div_ncx, div_v, div_h;
 };
 
-template <typename S, int D, int DC>
-__global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >= 64 ? 5 : 4) : (S::kBytes == 2 ? 3 : 2)) void bwd_dkdv_cell_kernel(
+// HANDED: the dq kernel has left (p, sm_scale * ds) of every sample in `handed_` (per query row of this head,
+// in the order of the row's coordinates): an entry then costs a gather of that pair and the two rank-1 updates --
+// no taps in registers, no dot products, no exponential. Only with the work list (colour < 0) and with the
+// positions beside the ids (frac).
+template <typename S, int D, int DC, bool HANDED>
+__global__ __launch_bounds__(kCellWaves *kWave, HANDED ? (DC <= 4 ? 5 : 4)
+                                                       : DC <= 4 ? (S::kBytes == 2 && D >= 64 ? 5 : 4) : (S::kBytes == 2 ? 3 : 2))
+void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float2 *__restrict__ stats_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
-    const float2 *__restrict__ frac, const uint4 *__restrict__ items,
+    const float2 *__restrict__ frac, const uint4 *__restrict__ items, const float2 *__restrict__ handed_,
     float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC, CellGrid cg)
 {
     constexpr int G = D / DC;
@@ -293,6 +299,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >
     __shared__ unsigned s_row[kCellWaves][kWave];           // byte offset of the entry's query row in dout (and its (lse, delta))
     __shared__ unsigned s_qrow[kCellWaves][kWave];          // ... in q (which may be strided)
     __shared__ float2 s_f[S::kBytes == 2 ? kCellWaves : 1][kWave];          // 16-bit storage: (fx, fy) of the entry
+    __shared__ float2 s_pd[HANDED ? kCellWaves : 1][kWave];                  // HANDED: (p, sm_scale * ds) of the entry
     __shared__ __attribute__((aligned(16))) float s_flush[kCellWaves][4 * D];                 // the flush: four rows of dk, then of dv
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
@@ -351,7 +358,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >
     const float row_sx = (lane & 1) ? 1.0f : (kPacked ? -1.0f : 0.0f), row_ox = (lane & 1) ? 0.0f : 1.0f;
     const float row_sy = (lane & 2) ? 1.0f : (kPacked ? -1.0f : 0.0f), row_oy = (lane & 2) ? 0.0f : 1.0f;
 #pragma unroll
-    for (int tpi = 0; tpi < 4; ++tpi) {
+    for (int tpi = 0; tpi < (HANDED ? 0 : 4); ++tpi) {
         if constexpr (kPacked) {
 #pragma unroll
             for (int i = 0; i < DC / 2; ++i) { ktp[tpi][i] = 0u; vtp[tpi][i] = 0u; }
@@ -371,7 +378,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >
     // so that a sample's blend costs 3 multiply-adds per element instead of 4, and the sums are kept as the
     // matching moments (sum c, sum c*fx, sum c*fy, sum c*fx*fy times the query row), turned back into the
     // four pixels' sums after the loop. (Taps outside the image were loaded as zero rows.)
-    if constexpr (!kPacked) {
+    if constexpr (!kPacked && !HANDED) {
 #pragma unroll
         for (int d = 0; d < DC; ++d) {
             kt[3][d] = (kt[3][d] - kt[2][d]) - (kt[1][d] - kt[0][d]);
@@ -408,12 +415,34 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >
     auto load_frac = [&](unsigned cstart) -> float2 {
         return (fracl && cstart < hi) ? fracl[min(cstart + (unsigned)lane, hi - 1u)] : make_float2(0.f, 0.f);
     };
+    // HANDED: the entry's pair, gathered one chunk ahead (so the ids are fetched two chunks ahead). Rows of this
+    // wave's (b, h) are a uniform base plus a 32-bit byte offset (the host checks V*H*L*N*8 < 2^32).
+    const char *handed_bh = (const char *)(handed_ + ((size_t)b * dm.V * dm.H + h) * dm.L * (size_t)dm.N);
+    auto load_pair = [&](unsigned sid) -> float2 {
+        const unsigned qlx = dm.divP.div(sid), px = sid - qlx * (unsigned)dm.P;
+        const unsigned s1x = dm.divL.div(qlx), lx = qlx - s1x * (unsigned)dm.L;
+        const unsigned off = ((s1x * (unsigned)dm.H * (unsigned)dm.L + lx) * (unsigned)dm.N + (unsigned)s2 * (unsigned)dm.P + px) * 8u;
+        return *reinterpret_cast<const float2 *>(handed_bh + off);
+    };
     unsigned id_nxt = load_id(lo);
     float2 ff_nxt = load_frac(lo);
+    unsigned id_nxt2 = 0u;
+    float2 pd_nxt = make_float2(0.f, 0.f);
+    if constexpr (HANDED) {
+        id_nxt2 = load_id(lo + kWave);
+        pd_nxt = load_pair(id_nxt);
+    }
     for (unsigned c0 = lo; c0 < hi; c0 += kWave) {
         const unsigned id = id_nxt;
         float2 ff = ff_nxt;
-        id_nxt = load_id(c0 + kWave);
+        const float2 pdv = pd_nxt;
+        if constexpr (HANDED) {
+            id_nxt = id_nxt2;
+            id_nxt2 = load_id(c0 + 2 * kWave);
+            pd_nxt = load_pair(id_nxt);
+        } else {
+            id_nxt = load_id(c0 + kWave);
+        }
         ff_nxt = load_frac(c0 + kWave);
         // one list entry per lane: weights and query row
         const unsigned ql = dm.divP.div(id), p = id - ql * (unsigned)dm.P;     // ql = s1*L + l
@@ -429,7 +458,11 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >
         // entries past the end of the list repeat its last sample with zero weights: they add nothing
         const bool live = c0 + (unsigned)lane < hi;
         wave_lds_sync();
-        if constexpr (kPacked) {
+        if constexpr (HANDED) {
+            s_pd[wave][lane] = live ? pdv : make_float2(0.f, 0.f);      // a dead entry adds nothing
+            if constexpr (kPacked) s_f[wave][lane] = make_float2(fx, fy);
+            else s_w[wave][lane] = make_float4(fx, fy, 0.f, 0.f);
+        } else if constexpr (kPacked) {
             s_w[wave][lane] = live ? make_float4(gx * gy, fx * gy, gx * fy, fx * fy) : make_float4(0.f, 0.f, 0.f, 0.f);
             s_f[wave][lane] = make_float2(fx, live ? fy : __int_as_float(0x7fc00000));     // NaN marks a dead entry
         } else {
@@ -448,13 +481,33 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >
             const unsigned roff = r + lane_byte, soff = r >> kRowToPairShift;
             load_words<kRowWords>(q_bh + (s_qrow[wave][j0 + slot] + lane_byte), f.qw);
             load_words<kRowWords>(do_bh + roff, f.dw);
-            f.ld = *(const float2 *)(stats_bh + soff);
+            if constexpr (!HANDED) f.ld = *(const float2 *)(stats_bh + soff);
         };
         auto consume = [&](int j0, const RowFetch<kRowWords> &f) {
-            const float4 w = s_w[wave][j0 + slot];
             float qf[DC], dof[DC];
             widen_words<S, DC>(f.qw, qf);
             widen_words<S, DC>(f.dw, dof);
+            if constexpr (HANDED) {
+                const float2 pv = s_pd[wave][j0 + slot];
+                float fxs, fys;
+                if constexpr (kPacked) {
+                    const float2 ff2 = s_f[wave][j0 + slot];
+                    fxs = ff2.x;
+                    fys = ff2.y;
+                } else {
+                    const float4 w4 = s_w[wave][j0 + slot];
+                    fxs = w4.x;
+                    fys = w4.y;
+                }
+                const float cl = fmaf(fxs, row_sx, row_ox) * fmaf(fys, row_sy, row_oy);
+                const float ck = cl * pv.y, cv = cl * pv.x;
+#pragma unroll
+                for (int d = 0; d < DC; ++d) {
+                    mK[d] = block_outer_fma(ck, qf[d], mK[d]);
+                    mV[d] = block_outer_fma(cv, dof[d], mV[d]);
+                }
+            } else {
+            const float4 w = s_w[wave][j0 + slot];
             const float lse = f.ld.x, delta = f.ld.y;
             float dot = 0.f, dp = 0.f;
             if constexpr (kPacked) {
@@ -499,6 +552,7 @@ __global__ __launch_bounds__(kCellWaves *kWave, DC <= 4 ? (S::kBytes == 2 && D >
             for (int d = 0; d < DC; ++d) {
                 mK[d] = block_outer_fma(ck, qf[d], mK[d]);
                 mV[d] = block_outer_fma(cv, dof[d], mV[d]);
+            }
             }
         };
         // Trips go in pairs, and every request is unconditional: entries past the end of the list (up to the

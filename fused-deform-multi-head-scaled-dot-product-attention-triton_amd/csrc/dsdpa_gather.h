@@ -617,7 +617,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
     const void *__restrict__ dout_, void *__restrict__ dq_, float2 *__restrict__ stats_,
-    float *__restrict__ dcoords_, Dims dm)
+    float *__restrict__ dcoords_, float2 *__restrict__ handed_, Dims dm)
 {
     constexpr int G = D / DC;
     constexpr int NS = kWave / G;
@@ -627,6 +627,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     __shared__ uint4 s_e[kGatherWaves][kWave];
     __shared__ float4 s_gx[CG ? kGatherWaves : 1][kWave];
     __shared__ float4 s_gy[CG ? kGatherWaves : 1][kWave];
+    __shared__ float2 s_hand[CG ? 1 : kGatherWaves][kWave];                      // (p, sm_scale * ds) of the chunk's samples
     static_assert(!(CG && WIN), "the window mode has no coordinate gradient");
     constexpr int kTab = WIN ? kGatherWaves : 1, kTabUnits = WIN ? kWinUnits : 1;
     __shared__ __attribute__((aligned(16))) float s_dotk[kTab][4 * kTabUnits];     // window mode: q.K per pixel
@@ -661,6 +662,9 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     const float qscale = dm.sm_scale * kLog2e;
     const float lse = lse_[rc.row];
     if (stats_ && lane == 0) stats_[rc.row] = make_float2(lse, delta);     // null: a launch of its own does it
+    // handed_ (may be null; never with CG): per sample, in the order of the coordinates of this head's rows,
+    // (p, sm_scale * ds) for the dk/dv kernel, which then need not recompute them from the taps
+    float2 *handed_row = handed_ ? handed_ + (size_t)rc.row * dm.N : nullptr;
 
     float dqa[DC];
 #pragma unroll
@@ -716,6 +720,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                 const float dp = fmaf(w0, tT[te.x], fmaf(w1, tT[te.y], fmaf(w2, tT[te.z], w3 * tT[te.w])));
                 const float p = live ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
                 const float ds = p * (dp - delta);
+                if (handed_row && live) handed_row[nc] = make_float2(p, ds * dm.sm_scale);
                 if (w0 != 0.f) atomicAdd(&tA[te.x], (double)(ds * w0));
                 if (w1 != 0.f) atomicAdd(&tA[te.y], (double)(ds * w1));
                 if (w2 != 0.f) atomicAdd(&tA[te.z], (double)(ds * w2));
@@ -849,8 +854,18 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                 dp = group_sum<G>(dp);
                 float p = (j < cnt) ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
                 float ds = p * (dp - delta);
+                if constexpr (!CG) s_hand[wave][j] = make_float2(p, ds * dm.sm_scale);   // (all lanes of the slot: same value, same place)
 #pragma unroll
                 for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
+            }
+        }
+        if constexpr (!CG) {
+            // the chunk's pairs, one sample per lane, in one coalesced store (plain stores and loads: streaming
+            // ones keep the pairs out of L2, where the dk/dv kernel finds them: 2.44 -> 2.64 ms at 64x64, D = 128)
+            if (handed_row) {
+                wave_lds_sync();
+                if (live) handed_row[c0 + lane] = s_hand[wave][lane];
+                wave_lds_sync();
             }
         }
     }

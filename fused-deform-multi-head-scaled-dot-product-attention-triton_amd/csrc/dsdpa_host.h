@@ -165,6 +165,8 @@ inline DescLayout desc_layout(size_t B, size_t V, size_t Himg, size_t Wimg, size
 //   sorted   B*V*(V*L*P) u32                 sample ids ordered by cell
 //   frac     B*V*(V*L*P) x 8 bytes           (fx, fy) of the same samples, same order
 //   items    B*V*wmax x 16 bytes             work list of the dk/dv kernel: (cell, first entry, end) per item
+//   handed   rows*V*P x 8 bytes              (p, sm_scale*ds) per query*sample, dq kernel -> dk/dv kernel (shapes
+//                                            on the gather kernels only)
 //   acc      2*n floats                      fp32 dk/dv accumulators (16-bit storage only)
 //   desc     20 bytes per coordinate pair    descriptor table (only when the plane kernels apply); 36 with
 //                                            the coordinate gradient
@@ -179,7 +181,7 @@ int sort_cell_lists(void *temp, size_t temp_bytes, const unsigned *ids_in, unsig
                     hipStream_t st);
 
 struct WorkspaceLayout {
-    size_t delta, counters, start, sorted, frac, items, acc, desc, sorted2, seg, sorttmp, sorttmp_bytes, total;
+    size_t delta, counters, start, sorted, frac, items, handed, handed_bytes, acc, desc, sorted2, seg, sorttmp, sorttmp_bytes, total;
     DescLayout dl;
     size_t counters_bytes;
     int NC;
@@ -215,6 +217,15 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     w.frac = off; off += round256(B * V * (V * Himg * Wimg * P) * 8);
     work_list_geometry(V, Himg * Wimg, P, (size_t)w.NC, &w.piece, &w.wmax);
     w.items = off; off += round256(B * V * (size_t)w.wmax * 16);
+    // (p, sm_scale * ds) per query*sample, handed from the dq kernel to the dk/dv kernel: on shapes whose planes do
+    // not fit in LDS (the backward then runs dq before dk/dv on one stream), not for the deterministic backward
+    // (its four colour launches recompute), and only while a (batch item)'s pairs can be addressed with 32 bits
+    w.handed = off;
+    w.handed_bytes = 0;
+    if (!deterministic && !plane_path_fits(Himg * Wimg, D, storage16 ? 2 : 4) &&
+        V * H * Himg * Wimg * (V * P) * 8 < ((size_t)1 << 32))
+        w.handed_bytes = round256(rows * (V * P) * 8);
+    off += w.handed_bytes;
     w.acc = off; if (storage16) off += round256(2 * rows * D * 4);
     // with the coordinate gradient the staged dq kernel needs more LDS; where it no longer fits, dq takes the
     // gather kernel and no table is needed

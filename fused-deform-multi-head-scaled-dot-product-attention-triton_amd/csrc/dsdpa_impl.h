@@ -178,7 +178,7 @@ int launch_bwd_gather(const void *q, const void *k, const void *v, const float *
 template <typename S, int D>
 int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const float *coords, const void *out,
                          const float *lse, const void *dout, void *dq, float2 *stats, float *dcoords,
-                         const Dims &dm, hipStream_t st)
+                         float2 *handed, const Dims &dm, hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
@@ -186,15 +186,15 @@ int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const floa
     if (dcoords)
         DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, true, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
-                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, dm);
+                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm);
     else if (gather_window_mode(dm.P))
         DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, false, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
-                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, dm);
+                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm);
     else
         DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, false, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
-                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, dm);
+                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm);
     return check_launch();
 }
 
@@ -431,7 +431,7 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
 template <typename S, int D>
 int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const float *coords,
                          const float2 *stats, const void *dout, const unsigned *start, const unsigned *sorted,
-                         const float2 *frac, const uint4 *items, unsigned wmax,
+                         const float2 *frac, const uint4 *items, unsigned wmax, const float2 *handed,
                          float *dk_acc, float *dv_acc, const Dims &dm, int NC, bool deterministic, hipStream_t st)
 {
     constexpr int DC = CellChunk<S, D>::value;
@@ -455,9 +455,14 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
         cg.div_h = FastDiv::make((unsigned)dm.H);
         const unsigned blocks = (unsigned)((nwork + kCellWaves - 1) / kCellWaves);
         const bool first = colour <= 0, last = colour < 0 || colour == 3;
-        DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
-                              first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
-                              stats, dout, start, sorted, frac, items, dk_acc, dv_acc, dm, NC, cg);
+        if (handed && colour < 0 && frac)
+            DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC, true>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
+                                  first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
+                                  stats, dout, start, sorted, frac, items, handed, dk_acc, dv_acc, dm, NC, cg);
+        else
+            DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC, false>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
+                                  first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
+                                  stats, dout, start, sorted, frac, items, handed, dk_acc, dv_acc, dm, NC, cg);
     }
     return check_launch();
 }
@@ -540,6 +545,10 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const unsigned *sorted = (const unsigned *)(ws + (deterministic ? wl.sorted2 : wl.sorted));
     // (the reordered lists of the deterministic backward have no positions beside them: coordinates are read again)
     const float2 *frac = deterministic ? nullptr : (const float2 *)(ws + wl.frac);
+    // (p, sm_scale * ds) per query*sample from the dq kernel to the dk/dv kernel, where the layout has room for it
+    // (shapes on the gather dq kernel, which then runs before dk/dv on the same stream); the dq kernel with the
+    // coordinate gradient does not write it
+    float2 *handed = (wl.handed_bytes && cell_binned && !dcoords) ? (float2 *)(ws + wl.handed) : nullptr;
     // fp32 storage: dk and dv are their own accumulators; 16-bit: fp32 accumulators in the workspace
     float *dk_acc = S::kBytes == 4 ? (float *)dk : (float *)(ws + wl.acc);
     float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
@@ -592,10 +601,10 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
             rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, dq_stats,     \
                                                      desc_g, dcoords, dm, st)                                   \
                         : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dq_stats, dcoords,   \
-                                                      dm, st);                                                  \
+                                                      handed, dm, st);                                          \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
                 rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, stats, dout, start, sorted, frac,             \
-                                                 (const uint4 *)(ws + wl.items), wl.wmax, dk_acc,               \
+                                                 (const uint4 *)(ws + wl.items), wl.wmax, handed, dk_acc,       \
                                                  dv_acc, dm, wl.NC, deterministic, bst);                        \
             else if (rc == DSDPA_OK)                                                                            \
                 rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, stats, dout, dk_acc, dv_acc, dm, st);         \

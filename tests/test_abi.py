@@ -56,6 +56,9 @@ def test_workspace_bytes():
         M = V * Himg * Wimg * P
         piece = (max(512, 4 * M // NC) + 63) // 64 * 64
         total += r256(B * V * (NC + M // piece + 1) * 16)
+        # (p, ds) per query*sample, dq kernel -> dk/dv kernel, on shapes whose planes do not fit in LDS
+        if table(B, V, Himg, Wimg, D, P, storage16) == 0 and V * H * Himg * Wimg * V * P * 8 < 1 << 32:
+            total += r256(rows * V * P * 8)
         total += r256(2 * rows * D * 4) if storage16 else 0
         return total + table(B, V, Himg, Wimg, D, P, storage16)
 
