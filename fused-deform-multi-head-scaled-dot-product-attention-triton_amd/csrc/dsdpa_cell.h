@@ -283,7 +283,7 @@ struct CellGrid {
 // no taps in registers, no dot products, no exponential. Only with the work list (colour < 0) and with the
 // positions beside the ids (frac).
 template <typename S, int D, int DC, bool HANDED>
-__global__ __launch_bounds__(kCellWaves *kWave, HANDED ? (DC <= 4 ? 5 : 4)
+__global__ __launch_bounds__(kCellWaves *kWave, HANDED ? (DC <= 4 ? 5 : (S::kBytes == 2 ? 3 : 4))
                                                        : DC <= 4 ? (S::kBytes == 2 && D >= 64 ? 5 : 4) : (S::kBytes == 2 ? 3 : 2))
 void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
@@ -299,7 +299,6 @@ void bwd_dkdv_cell_kernel(
     __shared__ unsigned s_row[kCellWaves][kWave];           // byte offset of the entry's query row in dout (and its (lse, delta))
     __shared__ unsigned s_qrow[kCellWaves][kWave];          // ... in q (which may be strided)
     __shared__ float2 s_f[S::kBytes == 2 ? kCellWaves : 1][kWave];          // 16-bit storage: (fx, fy) of the entry
-    __shared__ float2 s_pd[HANDED ? kCellWaves : 1][kWave];                  // HANDED: (p, sm_scale * ds) of the entry
     __shared__ __attribute__((aligned(16))) float s_flush[kCellWaves][4 * D];                 // the flush: four rows of dk, then of dv
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
@@ -459,9 +458,8 @@ void bwd_dkdv_cell_kernel(
         const bool live = c0 + (unsigned)lane < hi;
         wave_lds_sync();
         if constexpr (HANDED) {
-            s_pd[wave][lane] = live ? pdv : make_float2(0.f, 0.f);      // a dead entry adds nothing
-            if constexpr (kPacked) s_f[wave][lane] = make_float2(fx, fy);
-            else s_w[wave][lane] = make_float4(fx, fy, 0.f, 0.f);
+            // (fx, fy, p, sm_scale * ds); a dead entry adds nothing
+            s_w[wave][lane] = make_float4(fx, fy, live ? pdv.x : 0.f, live ? pdv.y : 0.f);
         } else if constexpr (kPacked) {
             s_w[wave][lane] = live ? make_float4(gx * gy, fx * gy, gx * fy, fx * fy) : make_float4(0.f, 0.f, 0.f, 0.f);
             s_f[wave][lane] = make_float2(fx, live ? fy : __int_as_float(0x7fc00000));     // NaN marks a dead entry
@@ -488,19 +486,9 @@ void bwd_dkdv_cell_kernel(
             widen_words<S, DC>(f.qw, qf);
             widen_words<S, DC>(f.dw, dof);
             if constexpr (HANDED) {
-                const float2 pv = s_pd[wave][j0 + slot];
-                float fxs, fys;
-                if constexpr (kPacked) {
-                    const float2 ff2 = s_f[wave][j0 + slot];
-                    fxs = ff2.x;
-                    fys = ff2.y;
-                } else {
-                    const float4 w4 = s_w[wave][j0 + slot];
-                    fxs = w4.x;
-                    fys = w4.y;
-                }
-                const float cl = fmaf(fxs, row_sx, row_ox) * fmaf(fys, row_sy, row_oy);
-                const float ck = cl * pv.y, cv = cl * pv.x;
+                const float4 w4 = s_w[wave][j0 + slot];                 // (fx, fy, p, sm_scale * ds)
+                const float cl = fmaf(w4.x, row_sx, row_ox) * fmaf(w4.y, row_sy, row_oy);
+                const float ck = cl * w4.w, cv = cl * w4.z;
 #pragma unroll
                 for (int d = 0; d < DC; ++d) {
                     mK[d] = block_outer_fma(ck, qf[d], mK[d]);
@@ -560,6 +548,54 @@ void bwd_dkdv_cell_kernel(
         // request of a block wraps to entry 0 and is never used. (A request under a branch makes the compiler
         // wait for all outstanding loads at the join, which undoes the overlap.)
         static_assert(kWave % (2 * NS) == 0, "a block of 64 entries is a whole number of trip pairs");
+        if constexpr (HANDED && kPacked) {
+            // 16-bit storage with the pairs handed over: FOUR entries per slot and trip on the 4x4x4 block matrix
+            // instruction. k runs over the four entries, i over the four taps (lane 4b+i supplies the four
+            // entries' coefficients of tap i, high and low parts in two instructions), j over the block's lanes
+            // with their elements of the four query rows -- as stored, regrouped by two byte permutes per pair
+            // of rows. 4 * DC instructions do what 4 * 2 * DC rank-1 updates and as many bf16 -> fp32
+            // conversions did. The q rows of the next trip are requested when this trip's are used up, the
+            // dout rows likewise (one set of registers each).
+            constexpr int QT = 4 * NS;
+            static_assert(kWave % QT == 0, "a block of 64 entries is a whole number of four-entry trips");
+            uint32_t rq[4][kRowWords], rd[4][kRowWords];
+            auto issue_q = [&](int j0) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    load_words<kRowWords>(q_bh + (s_qrow[wave][j0 + 4 * slot + k] + lane_byte), rq[k]);
+            };
+            auto issue_d = [&](int j0) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    load_words<kRowWords>(do_bh + (s_row[wave][j0 + 4 * slot + k] + lane_byte), rd[k]);
+            };
+            issue_q(0);
+            issue_d(0);
+            for (int j0 = 0; j0 < cnt; j0 += QT) {
+                float ck[4], cv[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float4 e = s_w[wave][j0 + 4 * slot + k];      // (fx, fy, p, sm_scale * ds)
+                    const float cl = fmaf(e.x, row_sx, row_ox) * fmaf(e.y, row_sy, row_oy);
+                    ck[k] = cl * e.w;
+                    cv[k] = cl * e.z;
+                }
+                const uint4 sk = split_coefficients<S>(ck[0], ck[1], ck[2], ck[3]);
+                const uint4 sv = split_coefficients<S>(cv[0], cv[1], cv[2], cv[3]);
+                __builtin_amdgcn_sched_barrier(0);
+                block_blend4_pair<S, DC>(rq, __builtin_bit_cast(shortx4, make_uint2(sk.x, sk.y)),
+                                         __builtin_bit_cast(shortx4, make_uint2(sk.z, sk.w)), mK);
+                __builtin_amdgcn_sched_barrier(0);
+                issue_q((j0 + QT) & (kWave - 1));
+                __builtin_amdgcn_sched_barrier(0);
+                block_blend4_pair<S, DC>(rd, __builtin_bit_cast(shortx4, make_uint2(sv.x, sv.y)),
+                                         __builtin_bit_cast(shortx4, make_uint2(sv.z, sv.w)), mV);
+                __builtin_amdgcn_sched_barrier(0);
+                issue_d((j0 + QT) & (kWave - 1));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            continue;
+        }
         RowFetch<kRowWords> fa, fb;
         issue(0, fa);
         for (int j0 = 0; j0 < cnt; j0 += 2 * NS) {

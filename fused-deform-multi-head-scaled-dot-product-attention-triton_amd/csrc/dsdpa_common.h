@@ -354,6 +354,89 @@ __device__ __forceinline__ floatx4 block_outer_fma(float a, float x, floatx4 acc
     return __builtin_amdgcn_mfma_f32_4x4x1f32(a, x, acc, 0, 0, 0);
 }
 
+// 16-bit storage, at least four lanes per slot: the weighted sum of four rows on the 4x4x4 block matrix
+// instruction. For every block of four lanes it computes C[i][j] += sum_k A[i][k] * B[k][j]: k runs over the
+// four rows (pixels of a unit, or taps of a sample), j over the block's lanes, each with its own
+// elements of those rows, and the two rows of A that are used are the high and the low part of the four
+// coefficients (each a 16-bit float; together 16 bits of mantissa), so that acc[e][0] + acc[e][1] is the sum
+// with coefficients good to 2^-16. Lane 4b+i supplies row i of A: `coef` is this lane's row (the high parts
+// in lanes 4b, the low parts in lanes 4b+1, zero elsewhere). The rows come as packed pairs, which two byte
+// permutes per pair of rows turn into "four rows' values of one element".
+template <typename S, int DC>
+__device__ __forceinline__ void block_blend4(const uint32_t (&r)[4][DC / 2], shortx4 coef, floatx4 (&acc)[DC])
+{
+#pragma unroll
+    for (int i = 0; i < DC / 2; ++i) {
+        const uint32_t lo01 = __builtin_amdgcn_perm(r[1][i], r[0][i], 0x05040100u);
+        const uint32_t lo23 = __builtin_amdgcn_perm(r[3][i], r[2][i], 0x05040100u);
+        const uint32_t hi01 = __builtin_amdgcn_perm(r[1][i], r[0][i], 0x07060302u);
+        const uint32_t hi23 = __builtin_amdgcn_perm(r[3][i], r[2][i], 0x07060302u);
+        const uint2 be = make_uint2(lo01, lo23), bo = make_uint2(hi01, hi23);
+        if constexpr (S::kBf16) {
+            acc[2 * i] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(coef, __builtin_bit_cast(shortx4, be), acc[2 * i], 0, 0, 0);
+            acc[2 * i + 1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(coef, __builtin_bit_cast(shortx4, bo), acc[2 * i + 1], 0, 0, 0);
+        } else {
+            typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+            acc[2 * i] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, coef), __builtin_bit_cast(halfx4, be), acc[2 * i], 0, 0, 0);
+            acc[2 * i + 1] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, coef), __builtin_bit_cast(halfx4, bo), acc[2 * i + 1], 0, 0, 0);
+        }
+    }
+}
+
+// Four fp32 coefficients as the block matrix instruction's rows: .x, .y = the high parts (storage type, by
+// truncation for bf16 / rounding for fp16) as four packed 16-bit floats, .z, .w = the same of the remainders.
+template <typename S>
+__device__ __forceinline__ uint4 split_coefficients(float c0, float c1, float c2, float c3)
+{
+    if constexpr (S::kBf16) {
+        const uint32_t u0 = __float_as_uint(c0), u1 = __float_as_uint(c1), u2 = __float_as_uint(c2), u3 = __float_as_uint(c3);
+        const float l0 = c0 - __uint_as_float(u0 & 0xffff0000u), l1 = c1 - __uint_as_float(u1 & 0xffff0000u);
+        const float l2 = c2 - __uint_as_float(u2 & 0xffff0000u), l3 = c3 - __uint_as_float(u3 & 0xffff0000u);
+        return make_uint4(__builtin_amdgcn_perm(u1, u0, 0x07060302u), __builtin_amdgcn_perm(u3, u2, 0x07060302u),
+                          __builtin_amdgcn_perm(__float_as_uint(l1), __float_as_uint(l0), 0x07060302u),
+                          __builtin_amdgcn_perm(__float_as_uint(l3), __float_as_uint(l2), 0x07060302u));
+    } else {
+        union { uint32_t u; _Float16 h[2]; } a, b, c, d;
+        a.h[0] = (_Float16)c0; a.h[1] = (_Float16)c1; b.h[0] = (_Float16)c2; b.h[1] = (_Float16)c3;
+        c.h[0] = (_Float16)(c0 - (float)a.h[0]); c.h[1] = (_Float16)(c1 - (float)a.h[1]);
+        d.h[0] = (_Float16)(c2 - (float)b.h[0]); d.h[1] = (_Float16)(c3 - (float)b.h[1]);
+        return make_uint4(a.u, b.u, c.u, d.u);
+    }
+}
+
+__device__ __forceinline__ uint4 lane_offsets(const uint4 &e, unsigned lane_byte)
+{
+    return make_uint4(e.x + lane_byte, e.y + lane_byte, e.z + lane_byte, e.w + lane_byte);
+}
+
+// The same with two coefficient operands (the high and the low parts of four rows of coefficients, see
+// split_coefficients): acc[e][i] += sum_k (hi[i][k] + lo[i][k]) * r[k][e], all four rows i in use. The byte
+// permutes are done once for both.
+template <typename S, int DC>
+__device__ __forceinline__ void block_blend4_pair(const uint32_t (&r)[4][DC / 2], shortx4 hi, shortx4 lo, floatx4 (&acc)[DC])
+{
+#pragma unroll
+    for (int i = 0; i < DC / 2; ++i) {
+        const uint32_t lo01 = __builtin_amdgcn_perm(r[1][i], r[0][i], 0x05040100u);
+        const uint32_t lo23 = __builtin_amdgcn_perm(r[3][i], r[2][i], 0x05040100u);
+        const uint32_t hi01 = __builtin_amdgcn_perm(r[1][i], r[0][i], 0x07060302u);
+        const uint32_t hi23 = __builtin_amdgcn_perm(r[3][i], r[2][i], 0x07060302u);
+        const uint2 be = make_uint2(lo01, lo23), bo = make_uint2(hi01, hi23);
+        if constexpr (S::kBf16) {
+            acc[2 * i] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(hi, __builtin_bit_cast(shortx4, be), acc[2 * i], 0, 0, 0);
+            acc[2 * i + 1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(hi, __builtin_bit_cast(shortx4, bo), acc[2 * i + 1], 0, 0, 0);
+            acc[2 * i] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(lo, __builtin_bit_cast(shortx4, be), acc[2 * i], 0, 0, 0);
+            acc[2 * i + 1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(lo, __builtin_bit_cast(shortx4, bo), acc[2 * i + 1], 0, 0, 0);
+        } else {
+            typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+            acc[2 * i] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, hi), __builtin_bit_cast(halfx4, be), acc[2 * i], 0, 0, 0);
+            acc[2 * i + 1] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, hi), __builtin_bit_cast(halfx4, bo), acc[2 * i + 1], 0, 0, 0);
+            acc[2 * i] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, lo), __builtin_bit_cast(halfx4, be), acc[2 * i], 0, 0, 0);
+            acc[2 * i + 1] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, lo), __builtin_bit_cast(halfx4, bo), acc[2 * i + 1], 0, 0, 0);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ reductions over the whole wave
 // Every lane ends up with the result. Five steps stay in the vector ALU (DPP / swizzle), the last is a shuffle.
 template <typename T, typename Op>
