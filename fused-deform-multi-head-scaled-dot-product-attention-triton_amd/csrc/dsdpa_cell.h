@@ -48,12 +48,17 @@ __device__ __forceinline__ bool taps_any(const Taps &tp)
     return (tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f);
 }
 
+// Lists are kept per key = (group of query views s1 / vpg, cell), NK = groups * NC keys per (batch, key view).
+// With more than one group the dk/dv kernel works through a key view's lists one group of query views at a
+// time, so that the query rows it gathers (q and dout of that group only) stay in the XCD's L2.
+//
 // One thread per coordinate pair, in memory order (b, s1, l, s2, p).
-// mode 0: count[(b*V+s2)*NC + cell] += 1
-// mode 1: sorted[(b*V+s2)*M + cursor[(b*V+s2)*NC + cell]++] = (s1*L + l)*P + p, and frac[same] = its (fx, fy)
+// mode 0: count[(b*V+s2)*NK + key] += 1
+// mode 1: sorted[(b*V+s2)*M + cursor[(b*V+s2)*NK + key]++] = (s1*L + l)*P + p, and frac[same] = its (fx, fy)
 template <int MODE>
 __global__ __launch_bounds__(kBinThreads) void bin_samples_kernel(const float *__restrict__ coords_, Dims dm,
-                                                                  int NC, unsigned *__restrict__ counters,
+                                                                  int NC, int NK, int vpg,
+                                                                  unsigned *__restrict__ counters,
                                                                   unsigned *__restrict__ sorted,
                                                                   float2 *__restrict__ frac)
 {
@@ -70,7 +75,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_samples_kernel(const float *_
     const int ql = (int)(t % ((long long)dm.V * dm.L));   // s1*L + l
     const int b = (int)(t / ((long long)dm.V * dm.L));
     const size_t grp = (size_t)b * dm.V + s2;
-    unsigned *ctr = counters + grp * NC + cell_of(tp, dm.Wimg);
+    unsigned *ctr = counters + grp * NK + (ql / dm.L / vpg) * NC + cell_of(tp, dm.Wimg);
     if (MODE == 0) {
         atomicAdd(ctr, 1u);
     } else {
@@ -93,7 +98,7 @@ constexpr int kBinLdsThreads = 1024;
 
 template <int MODE>
 __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
-    const float *__restrict__ coords_, Dims dm, int NC, int lchunk, int nlc,
+    const float *__restrict__ coords_, Dims dm, int NC, int NK, int vpg, int lchunk, int nlc,
     unsigned *__restrict__ counters, unsigned *__restrict__ sorted, float2 *__restrict__ frac)
 {
     extern __shared__ unsigned s_hist[];                 // [V][NC]; mode 1 adds [V][NC] bases
@@ -113,16 +118,17 @@ __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
         if (taps_any(tp)) atomicAdd(&s_hist[((i / dm.P) % dm.V) * NC + cell_of(tp, dm.Wimg)], 1u);
     }
     __syncthreads();
-    unsigned *gctr = counters + (size_t)b * dm.V * NC;   // [s2][cell] of this batch item
+    // [s2][key] of this batch item, at this workgroup's group of query views
+    unsigned *gctr = counters + (size_t)b * dm.V * NK + (size_t)(s1 / vpg) * NC;
     if (MODE == 0) {
         for (int i = threadIdx.x; i < nhist; i += kBinLdsThreads) {
             const unsigned c = s_hist[i];
-            if (c) atomicAdd(gctr + i, c);
+            if (c) atomicAdd(gctr + (size_t)(i / NC) * NK + i % NC, c);
         }
     } else {
         for (int i = threadIdx.x; i < nhist; i += kBinLdsThreads) {
             const unsigned c = s_hist[i];
-            s_base[i] = c ? atomicAdd(gctr + i, c) : 0u;
+            s_base[i] = c ? atomicAdd(gctr + (size_t)(i / NC) * NK + i % NC, c) : 0u;
             s_hist[i] = 0u;
         }
         __syncthreads();
@@ -140,7 +146,7 @@ __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
     }
 }
 
-// One workgroup per (b, s2): exclusive scan of the NC cell counts. Writes
+// One workgroup per (b, s2): exclusive scan of the list lengths (NC here = the number of keys, group-major). Writes
 // start[grp*(NC+1) + c] (with the total at c = NC) and resets counters to the
 // same starts, so that the fill pass can use them as cursors.
 //
@@ -152,7 +158,7 @@ __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
 // items (M = entries of all lists). An item carries all a wave needs to start on it: one read, where the
 // list's bounds would be a second, dependent one.
 static __global__ __launch_bounds__(1024) void bin_scan_kernel(unsigned *__restrict__ counters,
-                                                        unsigned *__restrict__ start, int NC,
+                                                        unsigned *__restrict__ start, int NC, int grid_cells,
                                                         unsigned piece, unsigned wmax, uint4 *__restrict__ items)
 {
     __shared__ unsigned s_part[1024], s_pcs[1024];
@@ -183,7 +189,7 @@ static __global__ __launch_bounds__(1024) void bin_scan_kernel(unsigned *__restr
         if (c < NC) {
             st[c] = excl;
             cnt[c] = excl;
-            const unsigned cell = (unsigned)c;
+            const unsigned cell = (unsigned)(c % grid_cells);
             for (unsigned i = 0; i < np; ++i)
                 if (pexcl + i < wmax) it[pexcl + i] = make_uint4(cell, excl + i * piece, min(excl + v, excl + (i + 1) * piece), 0u);
         }
@@ -548,8 +554,9 @@ void bwd_dkdv_cell_kernel(
         // request of a block wraps to entry 0 and is never used. (A request under a branch makes the compiler
         // wait for all outstanding loads at the join, which undoes the overlap.)
         static_assert(kWave % (2 * NS) == 0, "a block of 64 entries is a whole number of trip pairs");
-        if constexpr (HANDED && kPacked) {
-            // 16-bit storage with the pairs handed over: FOUR entries per slot and trip on the 4x4x4 block matrix
+        if constexpr (HANDED && kPacked && DC >= 8) {
+            // 16-bit storage with the pairs handed over, eight elements per lane (at four the trips are too short
+            // for the requests to arrive in time: 1.14 -> 1.22 ms at 48x48, D = 64): FOUR entries per slot and trip on the 4x4x4 block matrix
             // instruction. k runs over the four entries, i over the four taps (lane 4b+i supplies the four
             // entries' coefficients of tap i, high and low parts in two instructions), j over the block's lanes
             // with their elements of the four query rows -- as stored, regrouped by two byte permutes per pair

@@ -184,7 +184,8 @@ struct WorkspaceLayout {
     size_t delta, counters, start, sorted, frac, items, handed, handed_bytes, acc, desc, sorted2, seg, sorttmp, sorttmp_bytes, total;
     DescLayout dl;
     size_t counters_bytes;
-    int NC;
+    int NC;                     // cells of the grid
+    int NK, vpg;                // lists per (batch, key view) = groups of query views * NC; query views per group
     unsigned piece, wmax;       // work list of the dk/dv kernel: entries per item, items per (batch, key view)
 };
 
@@ -203,6 +204,22 @@ inline void work_list_geometry(size_t V, size_t L, size_t P, size_t NC, unsigned
     *piece = (unsigned)pc;
     *wmax = (unsigned)(NC + M / pc + 1);
 }
+// Query views per group of the dk/dv lists (only where the dq kernel hands its pairs over: there the dk/dv kernel
+// waits for the query rows it gathers and for little else). The rows of one (batch, head), q and dout, are
+// 2*V*L*D*e bytes; where that is more than an XCD's 4 MB of L2, the entries -- which the cell order scatters over
+// all of it -- miss L2. Lists per (group of query views, cell), worked through group by group, keep the rows in
+// use to one group's: groups of at most 4 MB (64x64, D = 128, 16-bit, V = 4: 8 MB, two groups: 2.31 -> 2.07 ms;
+// four groups 2.23 ms -- every group multiplies the items, each with its set-up and flush), as long as the lists
+// stay long enough to pay for that (an average of 48 entries over the whole grid).
+inline int views_per_group(size_t V, size_t L, size_t D, size_t esize, size_t P, size_t NC, bool handed)
+{
+    const size_t rows_bytes = 2 * V * L * D * esize, M = V * L * P, cap = (size_t)4 << 20;
+    if (!handed || rows_bytes <= cap) return (int)V;
+    size_t groups = (rows_bytes + cap - 1) / cap;
+    if (groups > V) groups = V;
+    while (groups > 1 && M / (groups * NC) < 48) --groups;
+    return (int)((V + groups - 1) / groups);
+}
 inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Himg, size_t Wimg, size_t D, size_t P,
                                         bool storage16, bool deterministic, bool coords_grad)
 {
@@ -211,20 +228,22 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     w.NC = (int)((Himg + 1) * (Wimg + 1));
     size_t off = 0;
     w.delta = off; off += round256(rows * 8);           // (lse, delta) per row
-    w.counters = off; w.counters_bytes = round256(B * V * (size_t)w.NC * 4); off += w.counters_bytes;
-    w.start = off; off += round256(B * V * ((size_t)w.NC + 1) * 4);
+    const bool handed = !deterministic && !plane_path_fits(Himg * Wimg, D, storage16 ? 2 : 4) &&
+                        V * H * Himg * Wimg * (V * P) * 8 < ((size_t)1 << 32);
+    w.vpg = views_per_group(V, Himg * Wimg, D, storage16 ? 2 : 4, P, (size_t)w.NC, handed);
+    w.NK = w.NC * (int)((V + w.vpg - 1) / w.vpg);
+    w.counters = off; w.counters_bytes = round256(B * V * (size_t)w.NK * 4); off += w.counters_bytes;
+    w.start = off; off += round256(B * V * ((size_t)w.NK + 1) * 4);
     w.sorted = off; off += round256(B * V * (V * Himg * Wimg * P) * 4);
     w.frac = off; off += round256(B * V * (V * Himg * Wimg * P) * 8);
-    work_list_geometry(V, Himg * Wimg, P, (size_t)w.NC, &w.piece, &w.wmax);
+    work_list_geometry(V, Himg * Wimg, P, (size_t)w.NK, &w.piece, &w.wmax);
     w.items = off; off += round256(B * V * (size_t)w.wmax * 16);
     // (p, sm_scale * ds) per query*sample, handed from the dq kernel to the dk/dv kernel: on shapes whose planes do
     // not fit in LDS (the backward then runs dq before dk/dv on one stream), not for the deterministic backward
     // (its four colour launches recompute), and only while a (batch item)'s pairs can be addressed with 32 bits
     w.handed = off;
     w.handed_bytes = 0;
-    if (!deterministic && !plane_path_fits(Himg * Wimg, D, storage16 ? 2 : 4) &&
-        V * H * Himg * Wimg * (V * P) * 8 < ((size_t)1 << 32))
-        w.handed_bytes = round256(rows * (V * P) * 8);
+    if (handed) w.handed_bytes = round256(rows * (V * P) * 8);
     off += w.handed_bytes;
     w.acc = off; if (storage16) off += round256(2 * rows * D * 4);
     // with the coordinate gradient the staged dq kernel needs more LDS; where it no longer fits, dq takes the

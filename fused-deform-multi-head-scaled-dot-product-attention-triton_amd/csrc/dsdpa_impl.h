@@ -403,13 +403,13 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
         if (int rc = allow_full_lds(k1, lds_set[1])) return rc;
         DSDPA_LAUNCH(k0, dim3((unsigned)blocks), dim3(kBinLdsThreads), hist_bytes, st,
                               t_count.start(), t_count.stop(),
-                           coords, dm, wl.NC, lchunk, nlc, counters, sorted, frac);
+                           coords, dm, wl.NC, wl.NK, wl.vpg, lchunk, nlc, counters, sorted, frac);
         DSDPA_LAUNCH(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st,
-                              t_scan.start(), t_scan.stop(), counters, start, wl.NC, wl.piece, wl.wmax,
+                              t_scan.start(), t_scan.stop(), counters, start, wl.NK, wl.NC, wl.piece, wl.wmax,
                               (uint4 *)(ws + wl.items));
         DSDPA_LAUNCH(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
                               t_fill.start(), t_fill.stop(),
-                           coords, dm, wl.NC, lchunk, nlc, counters, sorted, frac);
+                           coords, dm, wl.NC, wl.NK, wl.vpg, lchunk, nlc, counters, sorted, frac);
         return check_launch();
     }
     const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
@@ -417,13 +417,13 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
     if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
     DSDPA_LAUNCH(bin_samples_kernel<0>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
                           t_count.start(), t_count.stop(),
-                       coords, dm, wl.NC, counters, sorted, frac);
+                       coords, dm, wl.NC, wl.NK, wl.vpg, counters, sorted, frac);
     DSDPA_LAUNCH(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st,
-                          t_scan.start(), t_scan.stop(), counters, start, wl.NC, wl.piece, wl.wmax,
+                          t_scan.start(), t_scan.stop(), counters, start, wl.NK, wl.NC, wl.piece, wl.wmax,
                               (uint4 *)(ws + wl.items));
     DSDPA_LAUNCH(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
                           t_fill.start(), t_fill.stop(),
-                       coords, dm, wl.NC, counters, sorted, frac);
+                       coords, dm, wl.NC, wl.NK, wl.vpg, counters, sorted, frac);
     return check_launch();
 }
 
@@ -605,7 +605,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
             if (rc == DSDPA_OK && cell_binned)                                                                  \
                 rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, stats, dout, start, sorted, frac,             \
                                                  (const uint4 *)(ws + wl.items), wl.wmax, handed, dk_acc,       \
-                                                 dv_acc, dm, wl.NC, deterministic, bst);                        \
+                                                 dv_acc, dm, wl.NK, deterministic, bst);                        \
             else if (rc == DSDPA_OK)                                                                            \
                 rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, stats, dout, dk_acc, dv_acc, dm, st);         \
             if (rc == DSDPA_OK) rc = joiner.join();                                                              \

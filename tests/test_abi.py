@@ -48,8 +48,22 @@ def test_workspace_bytes():
         m = B * V * L * V * P
         return r256(m * 16) + r256(m * 4)
 
+    def groups(V, H, L, D, e, P, NC, handed):
+        # lists per (group of query views, cell) where the pairs are handed over and the q and dout rows of one
+        # (batch, head) outgrow L2
+        rows_bytes, M, cap = 2 * V * L * D * e, V * L * P, 4 << 20
+        if not handed or rows_bytes <= cap:
+            return 1
+        g = min(V, (rows_bytes + cap - 1) // cap)
+        while g > 1 and M // (g * NC) < 48:
+            g -= 1
+        vpg = (V + g - 1) // g
+        return (V + vpg - 1) // vpg
+
     def expect(B, V, H, Himg, Wimg, D, P, storage16):
         rows, NC = B * V * H * Himg * Wimg, (Himg + 1) * (Wimg + 1)
+        handed = table(B, V, Himg, Wimg, D, P, storage16) == 0 and V * H * Himg * Wimg * V * P * 8 < 1 << 32
+        NC = NC * groups(V, H, Himg * Wimg, D, 2 if storage16 else 4, P, NC, handed)
         total = r256(rows * 8) + r256(B * V * NC * 4) + r256(B * V * (NC + 1) * 4) + r256(B * V * V * Himg * Wimg * P * 4)
         total += r256(B * V * V * Himg * Wimg * P * 8)          # positions beside the ids
         # work list of the dk/dv kernel: items of at most `piece` list entries, (cell, first entry, end) in 16 bytes each
