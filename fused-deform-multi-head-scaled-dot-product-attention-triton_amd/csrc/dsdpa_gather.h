@@ -86,11 +86,14 @@ __device__ __forceinline__ void stage_descriptors(const float2 *__restrict__ coo
 // rows of K and of V, read as contiguous runs, where the taps cost 4 per sample: about 120 against 256 for
 // 64 samples with a standard deviation of two pixels. Chosen per chunk, from the bounding box of its taps.
 //
-// The window is walked in UNITS of four pixels that are neighbours in a row (one 16-byte load per pixel
-// at constant offsets from the unit's first): its rows are padded to a whole number of units, and it is
-// moved left where that would cross the right edge of the image, so every pixel of every unit lies
-// inside the image. Tables are indexed by entry = (row - ymin) * 4 * nu + (column - xmin).
+// The window is laid out in UNITS of four pixels that are neighbours in a row: its rows are padded to a whole
+// number of units, and it is moved left where that would cross the right edge of the image, so every pixel
+// of every unit lies inside the image. Tables are indexed by entry = (row - ymin) * 4 * nu + (column - xmin).
+// Only the pixels that some tap of the chunk touches are worked on, four at a time ("quads", see
+// window_quads): of the 134 pixels of the padded box of such a chunk, 72 on average.
 constexpr int kWinUnits = 64;                  // units per window: the tables of a wave hold 256 pixels
+constexpr int kWinEntries = 4 * kWinUnits;
+constexpr int kWinDummy = kWinEntries;         // table entry of the padding pixels of the last quad (a place of its own)
 
 struct Window { int xmin, ymin, nu, nunits; };     // wave-uniform; nu = units per window row
 
@@ -133,27 +136,59 @@ __device__ __forceinline__ int4 window_entries(const Taps &tp, const Window &win
                      min(max(cy1 + cx1, 0), last));
 }
 
-// The unit this slot takes in the step that starts at unit u0 (held at the last unit beyond the window),
-// and the byte offset of its first pixel from plane (b, view 0, h).
-__device__ __forceinline__ unsigned window_unit(const Window &win, int u0, int slot, int Wimg, unsigned view_byte,
-                                                float rnu, unsigned px_bytes, int *unit)
+// The touched pixels of the window, compacted into quads. te: this lane's four table entries (every lane has
+// four, the clamped taps of weight 0 included, so that every entry a sample reads is among the touched).
+// Lane i looks after unit i: a bitmap in LDS tells which of its four pixels are touched, ballots rank them
+// (pixel k of all units before pixel k+1), and the lane writes each one's byte offset from plane (b, view 0, h)
+// to q_off[rank] and its table entry to q_ent[rank]. The last quad is padded with the window's first pixel
+// (inside the image) and the dummy entry. Returns the number of quads (wave-uniform).
+__device__ __forceinline__ int window_quads(const Window &win, const int4 &te, int lane, int Wimg, unsigned view_byte,
+                                            float rnu, unsigned px_bytes, unsigned *bm, unsigned *q_off,
+                                            unsigned *q_ent)
 {
-    const int u = min(u0 + slot, win.nunits - 1);
-    const int wy = (int)(((float)u + 0.5f) * rnu);             // u / nu: exact for these small numbers
-    const int wxu = u - wy * win.nu;
-    *unit = u;
-    return view_byte + (unsigned)((win.ymin + wy) * Wimg + win.xmin + 4 * wxu) * px_bytes;
+    if (lane < kWinEntries / 32) bm[lane] = 0u;
+    wave_lds_sync();
+    atomicOr(&bm[te.x >> 5], 1u << (te.x & 31));
+    atomicOr(&bm[te.y >> 5], 1u << (te.y & 31));
+    atomicOr(&bm[te.z >> 5], 1u << (te.z & 31));
+    atomicOr(&bm[te.w >> 5], 1u << (te.w & 31));
+    wave_lds_sync();
+    const unsigned nib = lane < win.nunits ? (bm[lane >> 3] >> ((lane & 7) * 4)) & 0xFu : 0u;
+    const int wy = (int)(((float)lane + 0.5f) * rnu);          // lane / nu: exact for these small numbers
+    const int wxu = lane - wy * win.nu;
+    const unsigned first = view_byte + (unsigned)((win.ymin + wy) * Wimg + win.xmin + 4 * wxu) * px_bytes;
+    int total = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const bool set = ((nib >> k) & 1u) != 0u;
+        const unsigned long long mask = __ballot(set);
+        const int rank = total + (int)__builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32),
+                                                                __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+        if (set) {
+            q_off[rank] = first + (unsigned)k * px_bytes;
+            q_ent[rank] = (unsigned)(4 * lane + k);
+        }
+        total += __popcll(mask);
+    }
+    const int nquads = (total + 3) >> 2;
+    if (lane < 4 * nquads - total) {
+        q_off[total + lane] = view_byte + (unsigned)(win.ymin * Wimg + win.xmin) * px_bytes;
+        q_ent[total + lane] = (unsigned)kWinDummy;
+    }
+    wave_lds_sync();
+    return nquads;
 }
 
-// q.K for the four pixels of this slot's unit, summed over the slot: t[4*unit + k].
+// x.row for the four pixels of this slot's quad (byte offsets o[k], this lane's part of the row included), summed
+// over the slot.
 template <typename S, int DC, int G>
-__device__ __forceinline__ void window_dots(const char *__restrict__ base, unsigned off, unsigned px_bytes,
+__device__ __forceinline__ void window_dots(const char *__restrict__ base, const unsigned (&o)[4],
                                             const float (&xf)[DC], const uint32_t *xp, float (&d)[4])
 {
     if constexpr (S::kBytes == 2) {
         uint32_t r[4][DC / 2];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) load_packed<S, DC>(base + off + k * px_bytes, r[k]);
+        for (int k = 0; k < 4; ++k) load_packed<S, DC>(base + o[k], r[k]);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             float acc = 0.f;
@@ -171,7 +206,7 @@ __device__ __forceinline__ void window_dots(const char *__restrict__ base, unsig
     } else {
         float r[4][DC];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) load_chunk<S, DC>(base + off + k * px_bytes, r[k]);
+        for (int k = 0; k < 4; ++k) load_chunk<S, DC>(base + o[k], r[k]);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             float acc = 0.f;
@@ -231,9 +266,12 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
     __shared__ float4 s_w[kGatherWaves][kWave];
     __shared__ uint4 s_e[kGatherWaves][kWave];
     constexpr int kTab = WIN ? kGatherWaves : 1, kTabUnits = WIN ? kWinUnits : 1;
-    __shared__ __attribute__((aligned(16))) float s_dot[kTab][4 * kTabUnits];      // window mode: q.K per pixel
-    __shared__ __attribute__((aligned(16))) double s_coef[kTab][4 * kTabUnits];    // window mode: coefficient of V per pixel
-    __shared__ uint4 s_blend[kTab][2 * kTabUnits];                                  // ... per unit, as the V pass reads them
+    __shared__ __attribute__((aligned(16))) float s_dot[kTab][4 * kTabUnits + 4];     // window mode: q.K per pixel (+ the dummy entry)
+    __shared__ __attribute__((aligned(16))) double s_coef[kTab][4 * kTabUnits + 4];   // window mode: coefficient of V per pixel
+    __shared__ uint4 s_blend[kTab][2 * kTabUnits];                                  // ... per quad, as the V pass reads them
+    __shared__ __attribute__((aligned(16))) unsigned s_qoff[kTab][4 * kTabUnits + 4]; // window mode: byte offsets of the quads' pixels
+    __shared__ __attribute__((aligned(16))) unsigned s_qent[kTab][4 * kTabUnits + 4]; // ... and their table entries
+    __shared__ unsigned s_bitmap[kTab][kWinEntries / 32];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
@@ -291,19 +329,30 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
                 uint4 *tC = s_blend[wave];
                 const float rnu = 1.0f / (float)win.nu;
                 const unsigned view_byte = (unsigned)s2c * (unsigned)rc.view_stride * S::kBytes;
-                // one q.K dot product per pixel of the window
-                for (int u0 = 0; u0 < win.nunits; u0 += NS) {
-                    int unit;
-                    const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
+                // one q.K dot product per touched pixel of the window
+                const int4 te = window_entries(tp, win, dm.Wimg, dm.Himg);
+                const unsigned *q_off = s_qoff[wave], *q_ent = s_qent[wave];
+                const int nquads = window_quads(win, te, lane, dm.Wimg, view_byte, rnu, kRow, s_bitmap[wave],
+                                                s_qoff[wave], s_qent[wave]);
+                for (int q0 = 0; q0 < nquads; q0 += NS) {
+                    const int qd = min(q0 + slot, nquads - 1);
+                    const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
+                    const uint4 ent = *reinterpret_cast<const uint4 *>(q_ent + 4 * qd);
+                    const unsigned o[4] = { off.x + lane_byte, off.y + lane_byte, off.z + lane_byte, off.w + lane_byte };
                     float d4[4];
-                    window_dots<S, DC, G>(kb, off, kRow, qf, qp, d4);
-                    if (g == 0) *reinterpret_cast<float4 *>(tS + 4 * unit) = make_float4(d4[0], d4[1], d4[2], d4[3]);
+                    window_dots<S, DC, G>(kb, o, qf, qp, d4);
+                    if (g == 0) {
+                        tS[ent.x] = d4[0];
+                        tS[ent.y] = d4[1];
+                        tS[ent.z] = d4[2];
+                        tS[ent.w] = d4[3];
+                    }
                 }
+                if (lane == 0) tA[kWinDummy] = 0.0;
                 for (int e = lane; e < 4 * win.nunits; e += kWave) tA[e] = 0.0;
                 wave_lds_sync();
                 // the samples, one per lane: logit from four of the pixel scalars, then the softmax bookkeeping
                 // of the chunk with ONE running maximum for all slots (they are brought to a common one first)
-                const int4 te = window_entries(tp, win, dm.Wimg, dm.Himg);
                 const float w0 = live ? tp.w[0] : 0.f, w1 = live ? tp.w[1] : 0.f;
                 const float w2 = live ? tp.w[2] : 0.f, w3 = live ? tp.w[3] : 0.f;
                 float logit = fmaf(w0, tS[te.x], fmaf(w1, tS[te.y], fmaf(w2, tS[te.z], w3 * tS[te.w])));
@@ -323,10 +372,11 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
                 if (w2 != 0.f) atomicAdd(&tA[te.z], (double)(p * w2));
                 if (w3 != 0.f) atomicAdd(&tA[te.w], (double)(p * w3));
                 wave_lds_sync();
-                // the coefficients of each unit in the form the V pass wants them (one unit per lane)
-                if (lane < win.nunits) {
-                    const float c0 = (float)tA[4 * lane], c1 = (float)tA[4 * lane + 1];
-                    const float c2 = (float)tA[4 * lane + 2], c3 = (float)tA[4 * lane + 3];
+                // the coefficients of each quad in the form the V pass wants them (one quad per lane)
+                if (lane < nquads) {
+                    const uint4 ent = *reinterpret_cast<const uint4 *>(q_ent + 4 * lane);
+                    const float c0 = (float)tA[ent.x], c1 = (float)tA[ent.y];
+                    const float c2 = (float)tA[ent.z], c3 = (float)tA[ent.w];
                     if constexpr (kBlock) {
                         tC[2 * lane] = split_coefficients<S>(c0, c1, c2, c3);      // rows 0, 1: high and low parts
                         tC[2 * lane + 1] = make_uint4(0u, 0u, 0u, 0u);             // rows 2, 3
@@ -335,33 +385,37 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
                     }
                 }
                 wave_lds_sync();
-                // one weighted sum of V rows per unit
+                // one weighted sum of V rows per quad
                 if constexpr (kBlock) {
                     floatx4 macc[DC];
 #pragma unroll
                     for (int d = 0; d < DC; ++d) macc[d] = floatx4{0.f, 0.f, 0.f, 0.f};
-                    for (int u0 = 0; u0 < win.nunits; u0 += NS) {
-                        int unit;
-                        const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
-                        uint2 cf = reinterpret_cast<const uint2 *>(tC)[4 * unit + (lane & 3)];
-                        if (u0 + slot >= win.nunits) cf = make_uint2(0u, 0u);
+                    for (int q0 = 0; q0 < nquads; q0 += NS) {
+                        const int qd = min(q0 + slot, nquads - 1);
+                        const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
+                        uint2 cf = reinterpret_cast<const uint2 *>(tC)[4 * qd + (lane & 3)];
+                        if (q0 + slot >= nquads) cf = make_uint2(0u, 0u);
                         uint32_t r[4][DC / 2];
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) load_packed<S, DC>(vb + off + k * kRow, r[k]);
+                        load_packed<S, DC>(vb + (off.x + lane_byte), r[0]);
+                        load_packed<S, DC>(vb + (off.y + lane_byte), r[1]);
+                        load_packed<S, DC>(vb + (off.z + lane_byte), r[2]);
+                        load_packed<S, DC>(vb + (off.w + lane_byte), r[3]);
                         block_blend4<S, DC>(r, __builtin_bit_cast(shortx4, cf), macc);
                     }
 #pragma unroll
                     for (int d = 0; d < DC; ++d) acc[d] += macc[d][0] + macc[d][1];
                 } else {
-                    for (int u0 = 0; u0 < win.nunits; u0 += NS) {
-                        int unit;
-                        const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
-                        uint4 cu = tC[2 * unit];
-                        if (u0 + slot >= win.nunits) cu = make_uint4(0u, 0u, 0u, 0u);
+                    for (int q0 = 0; q0 < nquads; q0 += NS) {
+                        const int qd = min(q0 + slot, nquads - 1);
+                        const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
+                        uint4 cu = tC[2 * qd];
+                        if (q0 + slot >= nquads) cu = make_uint4(0u, 0u, 0u, 0u);
                         const float cf[4] = { __uint_as_float(cu.x), __uint_as_float(cu.y), __uint_as_float(cu.z), __uint_as_float(cu.w) };
                         float r[4][DC];
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) load_chunk<S, DC>(vb + off + k * kRow, r[k]);
+                        load_chunk<S, DC>(vb + (off.x + lane_byte), r[0]);
+                        load_chunk<S, DC>(vb + (off.y + lane_byte), r[1]);
+                        load_chunk<S, DC>(vb + (off.z + lane_byte), r[2]);
+                        load_chunk<S, DC>(vb + (off.w + lane_byte), r[3]);
 #pragma unroll
                         for (int k = 0; k < 4; ++k) {
 #pragma unroll
@@ -575,10 +629,13 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
     __shared__ float2 s_hand[CG ? 1 : kGatherWaves][kWave];                      // (p, sm_scale * ds) of the chunk's samples
     static_assert(!(CG && WIN), "the window mode has no coordinate gradient");
     constexpr int kTab = WIN ? kGatherWaves : 1, kTabUnits = WIN ? kWinUnits : 1;
-    __shared__ __attribute__((aligned(16))) float s_dotk[kTab][4 * kTabUnits];     // window mode: q.K per pixel
-    __shared__ __attribute__((aligned(16))) float s_dotv[kTab][4 * kTabUnits];     // window mode: dout.V per pixel
-    __shared__ __attribute__((aligned(16))) double s_coef[kTab][4 * kTabUnits];    // window mode: coefficient of K per pixel
-    __shared__ uint4 s_blend[kTab][2 * kTabUnits];                                  // ... per unit, as the last pass reads them
+    __shared__ __attribute__((aligned(16))) float s_dotk[kTab][4 * kTabUnits + 4];    // window mode: q.K per pixel (+ the dummy entry)
+    __shared__ __attribute__((aligned(16))) float s_dotv[kTab][4 * kTabUnits + 4];    // window mode: dout.V per pixel
+    __shared__ __attribute__((aligned(16))) double s_coef[kTab][4 * kTabUnits + 4];   // window mode: coefficient of K per pixel
+    __shared__ uint4 s_blend[kTab][2 * kTabUnits];                                  // ... per quad, as the last pass reads them
+    __shared__ __attribute__((aligned(16))) unsigned s_qoff[kTab][4 * kTabUnits + 4]; // window mode: byte offsets of the quads' pixels
+    __shared__ __attribute__((aligned(16))) unsigned s_qent[kTab][4 * kTabUnits + 4]; // ... and their table entries
+    __shared__ unsigned s_bitmap[kTab][kWinEntries / 32];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
@@ -643,22 +700,28 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                 uint4 *tC = s_blend[wave];
                 const float rnu = 1.0f / (float)win.nu;
                 const unsigned view_byte = (unsigned)s2c * (unsigned)rc.view_stride * S::kBytes;
-                // q.K and dout.V per pixel of the window
-                for (int u0 = 0; u0 < win.nunits; u0 += NS) {
-                    int unit;
-                    const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
+                // q.K and dout.V per touched pixel of the window
+                const int4 te = window_entries(tp, win, dm.Wimg, dm.Himg);
+                const unsigned *q_off = s_qoff[wave], *q_ent = s_qent[wave];
+                const int nquads = window_quads(win, te, lane, dm.Wimg, view_byte, rnu, kRow, s_bitmap[wave],
+                                                s_qoff[wave], s_qent[wave]);
+                for (int q0 = 0; q0 < nquads; q0 += NS) {
+                    const int qd = min(q0 + slot, nquads - 1);
+                    const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
+                    const uint4 ent = *reinterpret_cast<const uint4 *>(q_ent + 4 * qd);
+                    const unsigned o[4] = { off.x + lane_byte, off.y + lane_byte, off.z + lane_byte, off.w + lane_byte };
                     float dk4[4], dv4[4];
-                    window_dots<S, DC, G>(kb, off, kRow, qf, qp, dk4);
-                    window_dots<S, DC, G>(vb, off, kRow, dof, dop, dv4);
+                    window_dots<S, DC, G>(kb, o, qf, qp, dk4);
+                    window_dots<S, DC, G>(vb, o, dof, dop, dv4);
                     if (g == 0) {
-                        *reinterpret_cast<float4 *>(tS + 4 * unit) = make_float4(dk4[0], dk4[1], dk4[2], dk4[3]);
-                        *reinterpret_cast<float4 *>(tT + 4 * unit) = make_float4(dv4[0], dv4[1], dv4[2], dv4[3]);
+                        tS[ent.x] = dk4[0]; tS[ent.y] = dk4[1]; tS[ent.z] = dk4[2]; tS[ent.w] = dk4[3];
+                        tT[ent.x] = dv4[0]; tT[ent.y] = dv4[1]; tT[ent.z] = dv4[2]; tT[ent.w] = dv4[3];
                     }
                 }
+                if (lane == 0) tA[kWinDummy] = 0.0;
                 for (int e = lane; e < 4 * win.nunits; e += kWave) tA[e] = 0.0;
                 wave_lds_sync();
                 // the samples, one per lane
-                const int4 te = window_entries(tp, win, dm.Wimg, dm.Himg);
                 const float w0 = live ? tp.w[0] : 0.f, w1 = live ? tp.w[1] : 0.f;
                 const float w2 = live ? tp.w[2] : 0.f, w3 = live ? tp.w[3] : 0.f;
                 const float dot = fmaf(w0, tS[te.x], fmaf(w1, tS[te.y], fmaf(w2, tS[te.z], w3 * tS[te.w])));
@@ -671,9 +734,10 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                 if (w2 != 0.f) atomicAdd(&tA[te.z], (double)(ds * w2));
                 if (w3 != 0.f) atomicAdd(&tA[te.w], (double)(ds * w3));
                 wave_lds_sync();
-                if (lane < win.nunits) {
-                    const float c0f = (float)tA[4 * lane], c1f = (float)tA[4 * lane + 1];
-                    const float c2f = (float)tA[4 * lane + 2], c3f = (float)tA[4 * lane + 3];
+                if (lane < nquads) {
+                    const uint4 ent = *reinterpret_cast<const uint4 *>(q_ent + 4 * lane);
+                    const float c0f = (float)tA[ent.x], c1f = (float)tA[ent.y];
+                    const float c2f = (float)tA[ent.z], c3f = (float)tA[ent.w];
                     if constexpr (kBlock) {
                         tC[2 * lane] = split_coefficients<S>(c0f, c1f, c2f, c3f);
                         tC[2 * lane + 1] = make_uint4(0u, 0u, 0u, 0u);
@@ -682,33 +746,37 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                     }
                 }
                 wave_lds_sync();
-                // dq += coefficient * K per pixel
+                // dq += coefficient * K per touched pixel
                 if constexpr (kBlock) {
                     floatx4 macc[DC];
 #pragma unroll
                     for (int d = 0; d < DC; ++d) macc[d] = floatx4{0.f, 0.f, 0.f, 0.f};
-                    for (int u0 = 0; u0 < win.nunits; u0 += NS) {
-                        int unit;
-                        const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
-                        uint2 cf = reinterpret_cast<const uint2 *>(tC)[4 * unit + (lane & 3)];
-                        if (u0 + slot >= win.nunits) cf = make_uint2(0u, 0u);
+                    for (int q0 = 0; q0 < nquads; q0 += NS) {
+                        const int qd = min(q0 + slot, nquads - 1);
+                        const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
+                        uint2 cf = reinterpret_cast<const uint2 *>(tC)[4 * qd + (lane & 3)];
+                        if (q0 + slot >= nquads) cf = make_uint2(0u, 0u);
                         uint32_t r[4][DC / 2];
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) load_packed<S, DC>(kb + off + k * kRow, r[k]);
+                        load_packed<S, DC>(kb + (off.x + lane_byte), r[0]);
+                        load_packed<S, DC>(kb + (off.y + lane_byte), r[1]);
+                        load_packed<S, DC>(kb + (off.z + lane_byte), r[2]);
+                        load_packed<S, DC>(kb + (off.w + lane_byte), r[3]);
                         block_blend4<S, DC>(r, __builtin_bit_cast(shortx4, cf), macc);
                     }
 #pragma unroll
                     for (int d = 0; d < DC; ++d) dqa[d] += macc[d][0] + macc[d][1];
                 } else {
-                    for (int u0 = 0; u0 < win.nunits; u0 += NS) {
-                        int unit;
-                        const unsigned off = window_unit(win, u0, slot, dm.Wimg, view_byte, rnu, kRow, &unit) + lane_byte;
-                        uint4 cu = tC[2 * unit];
-                        if (u0 + slot >= win.nunits) cu = make_uint4(0u, 0u, 0u, 0u);
+                    for (int q0 = 0; q0 < nquads; q0 += NS) {
+                        const int qd = min(q0 + slot, nquads - 1);
+                        const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
+                        uint4 cu = tC[2 * qd];
+                        if (q0 + slot >= nquads) cu = make_uint4(0u, 0u, 0u, 0u);
                         const float cf[4] = { __uint_as_float(cu.x), __uint_as_float(cu.y), __uint_as_float(cu.z), __uint_as_float(cu.w) };
                         float r[4][DC];
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) load_chunk<S, DC>(kb + off + k * kRow, r[k]);
+                        load_chunk<S, DC>(kb + (off.x + lane_byte), r[0]);
+                        load_chunk<S, DC>(kb + (off.y + lane_byte), r[1]);
+                        load_chunk<S, DC>(kb + (off.z + lane_byte), r[2]);
+                        load_chunk<S, DC>(kb + (off.w + lane_byte), r[3]);
 #pragma unroll
                         for (int k = 0; k < 4; ++k) {
 #pragma unroll
