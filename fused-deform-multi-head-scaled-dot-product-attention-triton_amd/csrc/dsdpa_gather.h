@@ -367,10 +367,11 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
                 const float psum = wave_sum(p);
                 if (slot == 0) lsum += psum;
                 // coefficient of every pixel: sum over the samples of p times the tap's bilinear weight
-                if (w0 != 0.f) atomicAdd(&tA[te.x], (double)(p * w0));
-                if (w1 != 0.f) atomicAdd(&tA[te.y], (double)(p * w1));
-                if (w2 != 0.f) atomicAdd(&tA[te.z], (double)(p * w2));
-                if (w3 != 0.f) atomicAdd(&tA[te.w], (double)(p * w3));
+                // (every lane adds all four: a tap of weight 0 or a lane beyond the chunk adds 0 to an entry of the tables)
+                atomicAdd(&tA[te.x], (double)(p * w0));
+                atomicAdd(&tA[te.y], (double)(p * w1));
+                atomicAdd(&tA[te.z], (double)(p * w2));
+                atomicAdd(&tA[te.w], (double)(p * w3));
                 wave_lds_sync();
                 // the coefficients of each quad in the form the V pass wants them (one quad per lane)
                 if (lane < nquads) {
@@ -729,10 +730,10 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
                 const float p = live ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
                 const float ds = p * (dp - delta);
                 if (handed_row && live) handed_row[nc] = make_float2(p, ds * dm.sm_scale);
-                if (w0 != 0.f) atomicAdd(&tA[te.x], (double)(ds * w0));
-                if (w1 != 0.f) atomicAdd(&tA[te.y], (double)(ds * w1));
-                if (w2 != 0.f) atomicAdd(&tA[te.z], (double)(ds * w2));
-                if (w3 != 0.f) atomicAdd(&tA[te.w], (double)(ds * w3));
+                atomicAdd(&tA[te.x], (double)(ds * w0));
+                atomicAdd(&tA[te.y], (double)(ds * w1));
+                atomicAdd(&tA[te.z], (double)(ds * w2));
+                atomicAdd(&tA[te.w], (double)(ds * w3));
                 wave_lds_sync();
                 if (lane < nquads) {
                     const uint4 ent = *reinterpret_cast<const uint4 *>(q_ent + 4 * lane);
