@@ -306,6 +306,9 @@ void bwd_dkdv_cell_kernel(
     __shared__ unsigned s_qrow[kCellWaves][kWave];          // ... in q (which may be strided)
     __shared__ float2 s_f[S::kBytes == 2 ? kCellWaves : 1][kWave];          // 16-bit storage: (fx, fy) of the entry
     __shared__ __attribute__((aligned(16))) float s_flush[kCellWaves][4 * D];                 // the flush: four rows of dk, then of dv
+    constexpr bool kQuad = HANDED && S::kBytes == 2 && DC >= 8;            // four-entry trips (below)
+    __shared__ float4 s_wq[kQuad ? kCellWaves : 1][2 * kWave];               // kQuad: two sets of entry tables, used in turn
+    __shared__ unsigned s_rowq[kQuad ? kCellWaves : 1][2 * kWave], s_qrowq[kQuad ? kCellWaves : 1][2 * kWave];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const unsigned work = (unsigned)xcd_logical_block(blockIdx.x, gridDim.x) * kCellWaves + wave;
@@ -429,15 +432,102 @@ void bwd_dkdv_cell_kernel(
         const unsigned off = ((s1x * (unsigned)dm.H * (unsigned)dm.L + lx) * (unsigned)dm.N + (unsigned)s2 * (unsigned)dm.P + px) * 8u;
         return *reinterpret_cast<const float2 *>(handed_bh + off);
     };
-    unsigned id_nxt = load_id(lo);
-    float2 ff_nxt = load_frac(lo);
+    if constexpr (kQuad) {
+        // 16-bit storage with the pairs handed over, eight elements per lane (at four the trips are too short for
+        // the requests to arrive in time: 1.14 -> 1.22 ms at 48x48, D = 64): FOUR entries per slot and trip on the
+        // 4x4x4 block matrix instruction. k runs over the four entries, i over the four taps (lane 4b+i supplies
+        // the four entries' coefficients of tap i, high and low parts in two instructions), j over the block's
+        // lanes with their elements of the four query rows -- as stored, regrouped by two byte permutes per pair
+        // of rows. 4 * DC instructions do what 4 * 2 * DC rank-1 updates and as many bf16 -> fp32 conversions did.
+        //
+        // Everything is requested ahead, across the 64-entry blocks too: the q rows of the next trip when this
+        // trip's are used up, the dout rows likewise (one set of registers each); the entry tables of the next
+        // block are made while this block is worked on (two sets in LDS, used in turn), from ids fetched three
+        // blocks ahead and pairs and positions fetched two blocks ahead, so that the last trip of a block can
+        // request the rows of the first trip of the next.
+        constexpr int QT = 4 * NS;
+        static_assert(kWave % QT == 0, "a block of 64 entries is a whole number of four-entry trips");
+        // (one array per table, the set chosen by an index: pointers picked at run time would be generic ones,
+        // whose loads count as memory loads and make every wait a wait for the rows in flight)
+        auto prepare = [&](unsigned cstart, int buf, unsigned sid, float2 ff, float2 pdv) {
+            const unsigned ql = dm.divP.div(sid);                                  // ql = s1*L + l
+            const unsigned s1 = dm.divL.div(ql), l = ql - s1 * (unsigned)dm.L;
+            const bool live = cstart + (unsigned)lane < hi;                        // a dead entry adds nothing
+            s_wq[wave][buf * kWave + lane] = make_float4(ff.x, ff.y, live ? pdv.x : 0.f, live ? pdv.y : 0.f);
+            s_rowq[wave][buf * kWave + lane] = (s1 * view_rows + l) * kRowBytes;
+            s_qrowq[wave][buf * kWave + lane] = (s1 * (unsigned)dm.q_sv + l * (unsigned)dm.q_sl) * S::kBytes;
+        };
+        uint32_t rq[4][kRowWords], rd[4][kRowWords];
+        auto issue_q = [&](int buf, int j0) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) load_words<kRowWords>(q_bh + (s_qrowq[wave][buf * kWave + j0 + 4 * slot + k] + lane_byte), rq[k]);
+        };
+        auto issue_d = [&](int buf, int j0) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) load_words<kRowWords>(do_bh + (s_rowq[wave][buf * kWave + j0 + 4 * slot + k] + lane_byte), rd[k]);
+        };
+        {
+            const unsigned id0 = load_id(lo);
+            prepare(lo, 0, id0, load_frac(lo), load_pair(id0));
+        }
+        unsigned id_a = load_id(lo + kWave);                                        // of the next block
+        float2 ff_a = load_frac(lo + kWave), pd_a = load_pair(id_a);
+        unsigned id_b = load_id(lo + 2 * kWave);                                    // of the block after it
+        wave_lds_sync();
+        issue_q(0, 0);
+        issue_d(0, 0);
+        int cur = 0;
+        for (unsigned c0 = lo; c0 < hi; c0 += kWave) {
+            const bool has_next = c0 + kWave < hi;
+            const float2 pd_b = load_pair(id_b), ff_b = load_frac(c0 + 2 * kWave);
+            const unsigned id_c = load_id(c0 + 3 * kWave);
+            __builtin_amdgcn_sched_barrier(0);                 // (requested here, not where they are used)
+            wave_lds_sync();
+            prepare(c0 + kWave, cur ^ 1, id_a, ff_a, pd_a);
+            wave_lds_sync();
+            const int cnt = (int)min((unsigned)kWave, hi - c0);
+            for (int j0 = 0; j0 < cnt; j0 += QT) {
+                float ck[4], cv[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float4 e = s_wq[wave][cur * kWave + j0 + 4 * slot + k];        // (fx, fy, p, sm_scale * ds)
+                    const float cl = fmaf(e.x, row_sx, row_ox) * fmaf(e.y, row_sy, row_oy);
+                    ck[k] = cl * e.w;
+                    cv[k] = cl * e.z;
+                }
+                const uint4 sk = split_coefficients<S>(ck[0], ck[1], ck[2], ck[3]);
+                const uint4 sv = split_coefficients<S>(cv[0], cv[1], cv[2], cv[3]);
+                // the next trip: of this block, or the first of the next block (none: this block's first, unused)
+                const bool over = j0 + QT >= kWave && has_next;
+                const int nbuf = over ? cur ^ 1 : cur, nj = (j0 + QT) & (kWave - 1);
+                __builtin_amdgcn_sched_barrier(0);
+                block_blend4_pair<S, DC>(rq, __builtin_bit_cast(shortx4, make_uint2(sk.x, sk.y)),
+                                         __builtin_bit_cast(shortx4, make_uint2(sk.z, sk.w)), mK);
+                __builtin_amdgcn_sched_barrier(0);
+                issue_q(nbuf, nj);
+                __builtin_amdgcn_sched_barrier(0);
+                block_blend4_pair<S, DC>(rd, __builtin_bit_cast(shortx4, make_uint2(sv.x, sv.y)),
+                                         __builtin_bit_cast(shortx4, make_uint2(sv.z, sv.w)), mV);
+                __builtin_amdgcn_sched_barrier(0);
+                issue_d(nbuf, nj);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            id_a = id_b;
+            ff_a = ff_b;
+            pd_a = pd_b;
+            id_b = id_c;
+            cur ^= 1;
+        }
+    }
+    unsigned id_nxt = kQuad ? 0u : load_id(lo);
+    float2 ff_nxt = kQuad ? make_float2(0.f, 0.f) : load_frac(lo);
     unsigned id_nxt2 = 0u;
     float2 pd_nxt = make_float2(0.f, 0.f);
-    if constexpr (HANDED) {
+    if constexpr (HANDED && !kQuad) {
         id_nxt2 = load_id(lo + kWave);
         pd_nxt = load_pair(id_nxt);
     }
-    for (unsigned c0 = lo; c0 < hi; c0 += kWave) {
+    for (unsigned c0 = lo; c0 < (kQuad ? lo : hi); c0 += kWave) {
         const unsigned id = id_nxt;
         float2 ff = ff_nxt;
         const float2 pdv = pd_nxt;
@@ -554,55 +644,6 @@ void bwd_dkdv_cell_kernel(
         // request of a block wraps to entry 0 and is never used. (A request under a branch makes the compiler
         // wait for all outstanding loads at the join, which undoes the overlap.)
         static_assert(kWave % (2 * NS) == 0, "a block of 64 entries is a whole number of trip pairs");
-        if constexpr (HANDED && kPacked && DC >= 8) {
-            // 16-bit storage with the pairs handed over, eight elements per lane (at four the trips are too short
-            // for the requests to arrive in time: 1.14 -> 1.22 ms at 48x48, D = 64): FOUR entries per slot and trip on the 4x4x4 block matrix
-            // instruction. k runs over the four entries, i over the four taps (lane 4b+i supplies the four
-            // entries' coefficients of tap i, high and low parts in two instructions), j over the block's lanes
-            // with their elements of the four query rows -- as stored, regrouped by two byte permutes per pair
-            // of rows. 4 * DC instructions do what 4 * 2 * DC rank-1 updates and as many bf16 -> fp32
-            // conversions did. The q rows of the next trip are requested when this trip's are used up, the
-            // dout rows likewise (one set of registers each).
-            constexpr int QT = 4 * NS;
-            static_assert(kWave % QT == 0, "a block of 64 entries is a whole number of four-entry trips");
-            uint32_t rq[4][kRowWords], rd[4][kRowWords];
-            auto issue_q = [&](int j0) {
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    load_words<kRowWords>(q_bh + (s_qrow[wave][j0 + 4 * slot + k] + lane_byte), rq[k]);
-            };
-            auto issue_d = [&](int j0) {
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    load_words<kRowWords>(do_bh + (s_row[wave][j0 + 4 * slot + k] + lane_byte), rd[k]);
-            };
-            issue_q(0);
-            issue_d(0);
-            for (int j0 = 0; j0 < cnt; j0 += QT) {
-                float ck[4], cv[4];
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const float4 e = s_w[wave][j0 + 4 * slot + k];      // (fx, fy, p, sm_scale * ds)
-                    const float cl = fmaf(e.x, row_sx, row_ox) * fmaf(e.y, row_sy, row_oy);
-                    ck[k] = cl * e.w;
-                    cv[k] = cl * e.z;
-                }
-                const uint4 sk = split_coefficients<S>(ck[0], ck[1], ck[2], ck[3]);
-                const uint4 sv = split_coefficients<S>(cv[0], cv[1], cv[2], cv[3]);
-                __builtin_amdgcn_sched_barrier(0);
-                block_blend4_pair<S, DC>(rq, __builtin_bit_cast(shortx4, make_uint2(sk.x, sk.y)),
-                                         __builtin_bit_cast(shortx4, make_uint2(sk.z, sk.w)), mK);
-                __builtin_amdgcn_sched_barrier(0);
-                issue_q((j0 + QT) & (kWave - 1));
-                __builtin_amdgcn_sched_barrier(0);
-                block_blend4_pair<S, DC>(rd, __builtin_bit_cast(shortx4, make_uint2(sv.x, sv.y)),
-                                         __builtin_bit_cast(shortx4, make_uint2(sv.z, sv.w)), mV);
-                __builtin_amdgcn_sched_barrier(0);
-                issue_d((j0 + QT) & (kWave - 1));
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            continue;
-        }
         RowFetch<kRowWords> fa, fb;
         issue(0, fa);
         for (int j0 = 0; j0 < cnt; j0 += 2 * NS) {
