@@ -341,9 +341,10 @@ __device__ __forceinline__ float group_sum(float x)
 
 // ------------------------------------------------------------------ 4x4 block matrix instructions
 // gfx950 has matrix instructions that treat a wave as 16 independent blocks of 4 lanes. Measured here, one of
-// them takes the issue port for about 1.3 times as long as one vector multiply-add and cannot overlap with
-// vector instructions of the same SIMD, but does the work of four: used as a wide multiply-add, not as a
-// GEMM (every sample has its own operands).
+// them takes 10-11 clocks of the SIMD where a vector multiply-add, a packed dot product or a byte permute takes
+// 4.6, and cannot overlap with vector instructions of the same SIMD, but does the work of four (4x4x1) or
+// sixteen (4x4x4) multiply-adds per lane: used as a wide multiply-add, not as a GEMM (every sample has its
+// own operands).
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 
