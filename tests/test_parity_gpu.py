@@ -110,11 +110,15 @@ WINDOWS = [
 ]
 
 
+# path: GATHER = forward in window mode, backward by the per-tap atomic kernel; AUTO = where the planes do not fit in
+# LDS (w32, w33, w35, w36 and the fp32 case of w31), forward and dq in window mode, dq handing (p, ds) to the
+# cell-binned dk/dv kernel (four-entry trips for 16-bit storage at D >= 128), else the staged kernels.
+@pytest.mark.parametrize("path", [_native.PATH_GATHER, _native.PATH_AUTO], ids=["gather", "auto"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
 @pytest.mark.parametrize("case", WINDOWS, ids=[f"w{c[0]}" for c in WINDOWS])
-def test_clustered_windows_vs_oracle(case, dtype):
+def test_clustered_windows_vs_oracle(case, dtype, path):
     seed, B, V, H, Himg, Wimg, D, P, sigma, lo, hi = case
-    say(f"[case] windows seed={seed} B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} sigma={sigma} {dtype}")
+    say(f"[case] windows seed={seed} B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} sigma={sigma} {dtype} path={path}")
     g = torch.Generator().manual_seed(seed)
     L = Himg * Wimg
     q, k, v = (torch.randn(B, V, H, L, D, generator=g).to(dtype) for _ in range(3))
@@ -123,7 +127,7 @@ def test_clustered_windows_vs_oracle(case, dtype):
     c[0, 0, 1, 0, 3, 0] = float("nan")                     # one NaN coordinate inside a cluster
     do = torch.randn(B, V, H, L, D, generator=g).to(dtype)
     scale = 1.0 / math.sqrt(D)
-    prev = _native.set_path(_native.PATH_GATHER)
+    prev = _native.set_path(path)
     try:
         out, dq, dk, dv = run_op(q, k, v, c, do, Wimg, Himg, scale)
     finally:
