@@ -107,6 +107,8 @@ WINDOWS = [
     (34, 1, 2, 1, 40, 3, 16, 64, 0.05, 0.2, 0.8),          # image narrower than one unit of a window row
     (35, 1, 1, 2, 12, 12, 256, 130, 0.3, 0.5, 0.5),        # wide spread: windows too large, every chunk gathers
     (36, 1, 2, 2, 33, 29, 64, 64, 0.004, 0.1, 0.9),        # very tight clusters: windows of one or two units
+    (37, 1, 4, 1, 48, 48, 256, 64, 0.03, 0.3, 0.7),        # q and dout rows of a (batch, head) beyond 4 MB: dk/dv lists
+                                                           # per group of query views (fp32: four groups, 16-bit: two)
 ]
 
 
