@@ -146,7 +146,9 @@ enum { DSDPA_FLAG_DETERMINISTIC = 1, DSDPA_FLAG_COORDS_GRAD = 2, DSDPA_FLAG_SING
  * bilinear cell (one u32 and the position inside the cell, 8 bytes, per coordinate pair, plus the cell
  * offsets; it depends on coords only and is shared by all heads) and, for bf16/fp16, the fp32 dk/dv
  * accumulators that are rounded to the storage type at the end (fp32: dk and dv
- * are themselves the accumulators), and the same per-coordinate table as the forward's. Without
+ * are themselves the accumulators), and the same per-coordinate table as the forward's -- or, on shapes
+ * whose K/V planes do not fit in LDS, 8 bytes per (query row, sample) in which the dq kernel leaves the
+ * softmax weight and its gradient for the dk/dv kernel. Without
  * DSDPA_FLAG_DETERMINISTIC the accumulation order into dk/dv is not deterministic (float atomics,
  * as in the reference, ops/triton.py:345-360).
  */
