@@ -287,12 +287,14 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float4 *
 {
     constexpr int DC = Chunk<S, D>::value;
     const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes;
-    const int waves = plane_waves((long long)dm.B * dm.H, dm.V * dm.L, kWave / (D / DC), device_cus());
-    const int rows_per_block = waves * (kWave / (D / DC));
+    int waves, row_blocks;
+    plane_config((long long)dm.B * dm.H, dm.V * dm.L, kWave / (D / DC), dm.P, device_cus(), DC <= 8 ? 2 : 1, &waves,
+                 &row_blocks);          // (16 elements per lane: two rows' state does not fit in the registers)
+    const int rows_per_block = row_blocks * waves * (kWave / (D / DC));
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
-    auto kern = fwd_slot_kernel<S, D, DC>;
-    static std::atomic<unsigned long long> lds_set{0};
-    if (int rc = allow_full_lds(kern, lds_set)) return rc;
+    auto kern = row_blocks == 2 ? fwd_slot_kernel<S, D, DC, 2> : fwd_slot_kernel<S, D, DC, 1>;
+    static std::atomic<unsigned long long> lds_set[2];
+    if (int rc = allow_full_lds(kern, lds_set[row_blocks - 1])) return rc;
     ScopedKernelTimer timer(0, st);
     DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(waves * kWave), smem, st,
                           timer.start(), timer.stop(), q, k, v, desc_w, desc_e, out, lse, dm);
@@ -307,7 +309,8 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
 {
     constexpr int DC = Chunk<S, D>::value;
     const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes + (dcoords ? kPlaneGradBytes : 0);
-    const int waves = plane_waves((long long)dm.B * dm.H, dm.V * dm.L, kWave / (D / DC), device_cus());
+    int waves, row_blocks;
+    plane_config((long long)dm.B * dm.H, dm.V * dm.L, kWave / (D / DC), dm.P, device_cus(), 1, &waves, &row_blocks);
     const int rows_per_block = waves * (kWave / (D / DC));
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
     auto kern = dcoords ? bwd_dq_slot_kernel<S, D, DC, true> : bwd_dq_slot_kernel<S, D, DC, false>;

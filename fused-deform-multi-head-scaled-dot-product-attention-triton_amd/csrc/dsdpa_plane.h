@@ -95,23 +95,28 @@ __device__ __forceinline__ int paired_position(bool valid, int cls, int lane, un
     return valid ? pos_valid : n0 + n1 + __popcll(mi & below);
 }
 
-// Waves per workgroup of a staged launch. The planes in LDS allow one workgroup per CU, so a launch runs in
-// rounds of `cus` workgroups, and a round lasts about as long as its workgroups have waves (the kernels are
-// bound by instruction issue) plus the staging of the planes (about two waves' worth). 16 waves is the most
-// rows per staged plane; fewer waves can mean fewer idle CUs in the last round: 2 x 8 x 16 planes of 14x14
-// pixels and 8 views make 416 workgroups of 16 waves, 1.6 rounds of 256, but 512 of 13 waves, two full
-// rounds of shorter workgroups. Picks the count with the lowest rounds * (waves + 2).
-inline int plane_waves(long long planes, int rows_per_plane, int rows_per_wave, int cus)
+// Waves per workgroup and query-row blocks per workgroup of a staged launch. The planes in LDS allow one workgroup
+// per CU, so a launch runs in rounds of `cus` workgroups, and a round lasts about as long as its workgroups have
+// waves times samples per view (the kernels are bound by instruction issue) plus the staging of the planes (about
+// two waves' worth at 32 samples per view: 64 in these units). 16 waves is the most rows per staged plane and
+// block; fewer waves can mean fewer idle CUs in the last round (2 x 8 x 16 planes of 14x14 pixels and 8 views
+// make 416 workgroups of 16 waves, 1.6 rounds of 256, but 512 of 13 waves, two full rounds of shorter
+// workgroups), and two row blocks per workgroup halve the staging of a launch of many rounds (few samples per
+// view: the reference's sweep). Picks the pair with the lowest rounds * (blocks * waves * P + 64).
+inline void plane_config(long long planes, int rows_per_plane, int rows_per_wave, int P, int cus, int max_blocks,
+                         int *waves, int *row_blocks)
 {
-    int best = kPlaneWaves;
     long long best_cost = -1;
-    for (int w = kPlaneWaves; w >= 4; --w) {
-        const long long rows = (long long)w * rows_per_wave;
-        const long long blocks = planes * ((rows_per_plane + rows - 1) / rows);
-        const long long cost = ((blocks + cus - 1) / cus) * (w + 2);
-        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = w; }
+    *waves = kPlaneWaves;
+    *row_blocks = 1;
+    for (int rb = 1; rb <= max_blocks; ++rb) {
+        for (int w = kPlaneWaves; w >= 4; --w) {
+            const long long rows = (long long)rb * w * rows_per_wave;
+            const long long blocks = planes * ((rows_per_plane + rows - 1) / rows);
+            const long long cost = ((blocks + cus - 1) / cus) * ((long long)rb * w * P + 64);
+            if (best_cost < 0 || cost < best_cost) { best_cost = cost; *waves = w; *row_blocks = rb; }
+        }
     }
-    return best;
 }
 
 struct PlaneBlock {
@@ -242,7 +247,10 @@ __device__ __forceinline__ int stage_slot_descriptors(const float4 *__restrict__
     return __float_as_int(gw.z);
 }
 
-template <typename S, int D, int DC>
+// ROWS: query-row blocks per workgroup. With two, a workgroup of W waves covers 2*W*NS rows: every staged plane is
+// worked on for the first W*NS rows and then for the second, so a launch of several rounds of workgroups stages
+// half as often (at 12 views x 12 samples per view the staging is a third of a workgroup's time).
+template <typename S, int D, int DC, int ROWS>
 __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float4 *__restrict__ desc_w, const uint32_t *__restrict__ desc_e, void *__restrict__ out_,
@@ -259,7 +267,8 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
     int2 *s_e =
         reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kPlaneDescPlaces * 16) + wave * kPlaneDescPlaces;
 
-    const PlaneBlock pb = decode_plane_block(dm, (int)(blockDim.x >> 6) * NS);   // (workgroups of up to kPlaneWaves waves)
+    const int rows_block = (int)(blockDim.x >> 6) * NS;                       // (workgroups of up to kPlaneWaves waves)
+    const PlaneBlock pb = decode_plane_block(dm, ROWS * rows_block);
     const int nq = dm.V * dm.L;
     const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
     const float qscale = dm.sm_scale * kLog2e;
@@ -267,24 +276,31 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
 
     zero_plane_pads<S, D>(smem, dm.L);
 
-    const int qidx = pb.qbase + wave * NS + slot;
-    const bool have = qidx < nq;
-    const unsigned qc = (unsigned)(have ? qidx : nq - 1);
-    const unsigned s1 = dm.divL.div(qc), l = qc - s1 * (unsigned)dm.L;
-    const size_t row = (((size_t)pb.b * dm.V + s1) * dm.H + pb.h) * dm.L + l;
-    const size_t crow = (((size_t)pb.b * dm.V + s1) * dm.L + l) * (size_t)dm.N;
-    float qf[DC], acc[DC];
-    uint32_t qp[kPacked ? DC / 2 : 1];
-    if constexpr (kPacked) {
-        load_packed<S, DC>((const char *)q_ + (dm.q_row(pb.b, (int)s1, pb.h, (int)l) + lane_elem) * S::kBytes, qp);
-    } else {
-        load_chunk<S, DC>((const char *)q_ + (dm.q_row(pb.b, (int)s1, pb.h, (int)l) + lane_elem) * S::kBytes, qf);
+    // per row block: this slot's row and its state
+    bool have_s[ROWS];
+    size_t row_s[ROWS], crow_s[ROWS];
+    float qf_s[ROWS][DC], acc_s[ROWS][DC], m_s[ROWS], lsum_s[ROWS];
+    uint32_t qp_s[ROWS][kPacked ? DC / 2 : 1];
 #pragma unroll
-        for (int d = 0; d < DC; ++d) qf[d] *= qscale;
+    for (int rb = 0; rb < ROWS; ++rb) {
+        const int qidx = pb.qbase + rb * rows_block + wave * NS + slot;
+        have_s[rb] = qidx < nq;
+        const unsigned qc = (unsigned)(have_s[rb] ? qidx : nq - 1);
+        const unsigned s1 = dm.divL.div(qc), l = qc - s1 * (unsigned)dm.L;
+        row_s[rb] = (((size_t)pb.b * dm.V + s1) * dm.H + pb.h) * dm.L + l;
+        crow_s[rb] = (((size_t)pb.b * dm.V + s1) * dm.L + l) * (size_t)dm.N;
+        if constexpr (kPacked) {
+            load_packed<S, DC>((const char *)q_ + (dm.q_row(pb.b, (int)s1, pb.h, (int)l) + lane_elem) * S::kBytes, qp_s[rb]);
+        } else {
+            load_chunk<S, DC>((const char *)q_ + (dm.q_row(pb.b, (int)s1, pb.h, (int)l) + lane_elem) * S::kBytes, qf_s[rb]);
+#pragma unroll
+            for (int d = 0; d < DC; ++d) qf_s[rb][d] *= qscale;
+        }
+        m_s[rb] = kNegBig;
+        lsum_s[rb] = 0.f;
+#pragma unroll
+        for (int d = 0; d < DC; ++d) acc_s[rb][d] = 0.f;
     }
-    float m = kNegBig, lsum = 0.f;
-#pragma unroll
-    for (int d = 0; d < DC; ++d) acc[d] = 0.f;
 
     for (int s2 = 0; s2 < dm.V; ++s2) {
         const size_t plane = dm.kv_plane(pb.b, s2, pb.h) * S::kBytes;
@@ -293,6 +309,13 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
         stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, px_bytes, 0);
         stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, px_bytes, 1);
         __syncthreads();
+#pragma unroll
+        for (int rb = 0; rb < ROWS; ++rb) {
+        const size_t crow = crow_s[rb];
+        const float (&qf)[DC] = qf_s[rb];
+        const uint32_t (&qp)[kPacked ? DC / 2 : 1] = qp_s[rb];
+        float (&acc)[DC] = acc_s[rb];
+        float &m = m_s[rb], &lsum = lsum_s[rb];
         for (int c0 = 0; c0 < dm.P; c0 += G) {
             stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g, slot, G, s_w,
                                          s_e);
@@ -365,14 +388,18 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
                 }
             }
         }
+        }
     }
 
-    if (have) {
-        const float inv = 1.0f / lsum;
 #pragma unroll
-        for (int d = 0; d < DC; ++d) acc[d] *= inv;
-        store_chunk<S, DC>((char *)out_ + (row * D + lane_elem) * S::kBytes, acc);
-        if (g == 0) lse_[row] = m + __log2f(lsum);
+    for (int rb = 0; rb < ROWS; ++rb) {
+        if (have_s[rb]) {
+            const float inv = 1.0f / lsum_s[rb];
+#pragma unroll
+            for (int d = 0; d < DC; ++d) acc_s[rb][d] *= inv;
+            store_chunk<S, DC>((char *)out_ + (row_s[rb] * D + lane_elem) * S::kBytes, acc_s[rb]);
+            if (g == 0) lse_[row_s[rb]] = m_s[rb] + __log2f(lsum_s[rb]);
+        }
     }
 }
 

@@ -96,6 +96,23 @@ def test_small_cases_vs_oracle(case, dtype, path):
     assert rel(dv, rdv) < TOL_BWD[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_staged_forward_two_row_blocks(dtype):
+    """Many planes, few samples per view: the staged forward then gives a workgroup two blocks of query rows per
+    staged plane (512 workgroups of one block would be two rounds on 256 CUs; 8 samples per view make the staging
+    weigh). Rows per (batch, head) = 1944 is no multiple of the 256 rows of a workgroup: the last one is part full."""
+    B, V, H, Himg, Wimg, D, P = 2, 6, 16, 18, 18, 32, 8
+    say(f"[case] two row blocks B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} {dtype}")
+    q, k, v, c, do = make_case(71, B, V, H, Himg, Wimg, D, P, -0.05, 1.05, dtype)
+    scale = 1.0 / math.sqrt(D)
+    out, dq, dk, dv = run_op(q, k, v, c, do, Wimg, Himg, scale)
+    ro, _, rdq, rdk, rdv = oracle_all(q, k, v, c, do, Wimg, Himg, scale)
+    assert rel(out, ro) < TOL_FWD[dtype]
+    assert rel(dq, rdq) < TOL_BWD[dtype]
+    assert rel(dk, rdk) < TOL_BWD[dtype]
+    assert rel(dv, rdv) < TOL_BWD[dtype]
+
+
 # Clustered coordinates with at least 64 samples per view: the gather kernels then cut chunks per key view and
 # work on the pixels of the window a chunk's samples fall into (fp32: multiply-adds; 16-bit storage: the 4x4x4
 # block matrix instruction), or gather tap by tap where the window is too large or the image too narrow.
