@@ -292,7 +292,10 @@ int launch_fwd_plane(const void *q, const void *k, const void *v, const float4 *
                  &row_blocks);          // (16 elements per lane: two rows' state does not fit in the registers)
     const int rows_per_block = row_blocks * waves * (kWave / (D / DC));
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
-    auto kern = row_blocks == 2 ? fwd_slot_kernel<S, D, DC, 2> : fwd_slot_kernel<S, D, DC, 1>;
+    auto kern = fwd_slot_kernel<S, D, DC, 1>;
+    if constexpr (DC <= 8) {
+        if (row_blocks == 2) kern = fwd_slot_kernel<S, D, DC, 2>;
+    }
     static std::atomic<unsigned long long> lds_set[2];
     if (int rc = allow_full_lds(kern, lds_set[row_blocks - 1])) return rc;
     ScopedKernelTimer timer(0, st);
@@ -310,12 +313,17 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
     constexpr int DC = Chunk<S, D>::value;
     const size_t smem = (size_t)plane_lds_bytes<S, D>(dm.L) + kPlaneDescBytes + (dcoords ? kPlaneGradBytes : 0);
     int waves, row_blocks;
-    plane_config((long long)dm.B * dm.H, dm.V * dm.L, kWave / (D / DC), dm.P, device_cus(), 1, &waves, &row_blocks);
-    const int rows_per_block = waves * (kWave / (D / DC));
+    // (two row blocks only without the coordinate gradient and up to 8 elements per lane: registers)
+    plane_config((long long)dm.B * dm.H, dm.V * dm.L, kWave / (D / DC), dm.P, device_cus(), (!dcoords && DC <= 8) ? 2 : 1,
+                 &waves, &row_blocks);
+    const int rows_per_block = row_blocks * waves * (kWave / (D / DC));
     const long long blocks = (long long)dm.B * dm.H * ((dm.V * dm.L + rows_per_block - 1) / rows_per_block);
-    auto kern = dcoords ? bwd_dq_slot_kernel<S, D, DC, true> : bwd_dq_slot_kernel<S, D, DC, false>;
-    static std::atomic<unsigned long long> lds_set[2];
-    if (int rc = allow_full_lds(kern, lds_set[dcoords ? 1 : 0])) return rc;
+    auto kern = dcoords ? bwd_dq_slot_kernel<S, D, DC, true, 1> : bwd_dq_slot_kernel<S, D, DC, false, 1>;
+    if constexpr (DC <= 8) {
+        if (row_blocks == 2) kern = bwd_dq_slot_kernel<S, D, DC, false, 2>;
+    }
+    static std::atomic<unsigned long long> lds_set[3];
+    if (int rc = allow_full_lds(kern, lds_set[dcoords ? 2 : row_blocks - 1])) return rc;
     ScopedKernelTimer timer(2, st);
     DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(waves * kWave), smem, st,
                           timer.start(), timer.stop(), q, k, v, desc_w, desc_e, out, lse, dout, dq, stats, desc_g,

@@ -408,7 +408,8 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
 // fx, fy from the table and reduced over the slot. The lane that fetched a sample's table entry keeps
 // the sample's result, and after the pass every lane adds its own sample's pair to dcoords (zeroed before
 // the launch) with float atomics -- one wave-wide pair of atomics per pass, not one per trip.
-template <typename S, int D, int DC, bool CG>
+// ROWS: query-row blocks per workgroup, as in the forward.
+template <typename S, int D, int DC, bool CG, int ROWS>
 __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float4 *__restrict__ desc_w, const uint32_t *__restrict__ desc_e, const void *__restrict__ out_,
@@ -427,7 +428,8 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
         reinterpret_cast<int2 *>(smem + img_bytes + kPlaneWaves * kPlaneDescPlaces * 16) + wave * kPlaneDescPlaces;
     float2 *s_g = reinterpret_cast<float2 *>(smem + img_bytes + kPlaneDescBytes) + wave * kPlaneDescPlaces;   // CG only
 
-    const PlaneBlock pb = decode_plane_block(dm, (int)(blockDim.x >> 6) * NS);   // (workgroups of up to kPlaneWaves waves)
+    const int rows_block = (int)(blockDim.x >> 6) * NS;                       // (workgroups of up to kPlaneWaves waves)
+    const PlaneBlock pb = decode_plane_block(dm, ROWS * rows_block);
     const int nq = dm.V * dm.L;
     const int g = lane % G, slot = lane / G, lane_elem = g * DC, lane_byte = lane_elem * S::kBytes;
     const float qscale = dm.sm_scale * kLog2e;
@@ -435,29 +437,33 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
 
     zero_plane_pads<S, D>(smem, dm.L);
 
-    const int qidx = pb.qbase + wave * NS + slot;
-    const bool have = qidx < nq;
-    const unsigned qc = (unsigned)(have ? qidx : nq - 1);
-    const unsigned s1 = dm.divL.div(qc), l = qc - s1 * (unsigned)dm.L;
-    const size_t row = (((size_t)pb.b * dm.V + s1) * dm.H + pb.h) * dm.L + l;
-    const size_t crow = (((size_t)pb.b * dm.V + s1) * dm.L + l) * (size_t)dm.N;
-    const size_t roff = (row * D + lane_elem) * S::kBytes;
-    float qf[DC], dof[DC], dqa[DC];
-    uint32_t dop[kPacked ? DC / 2 : 1];
-    float delta;
-    {
+    // per row block: this slot's row and its state
+    bool have_s[ROWS];
+    size_t crow_s[ROWS], roff_s[ROWS];
+    float qf_s[ROWS][DC], dof_s[ROWS][DC], dqa_s[ROWS][DC], delta_s[ROWS], lse_s[ROWS];
+    uint32_t dop_s[ROWS][kPacked ? DC / 2 : 1];
+#pragma unroll
+    for (int rb = 0; rb < ROWS; ++rb) {
+        const int qidx = pb.qbase + rb * rows_block + wave * NS + slot;
+        have_s[rb] = qidx < nq;
+        const unsigned qc = (unsigned)(have_s[rb] ? qidx : nq - 1);
+        const unsigned s1 = dm.divL.div(qc), l = qc - s1 * (unsigned)dm.L;
+        const size_t row = (((size_t)pb.b * dm.V + s1) * dm.H + pb.h) * dm.L + l;
+        crow_s[rb] = (((size_t)pb.b * dm.V + s1) * dm.L + l) * (size_t)dm.N;
+        const size_t roff = (row * D + lane_elem) * S::kBytes;
+        roff_s[rb] = roff;
         float of[DC];
-        load_chunk<S, DC>((const char *)q_ + (dm.q_row(pb.b, (int)s1, pb.h, (int)l) + lane_elem) * S::kBytes, qf);
-        load_chunk<S, DC>((const char *)dout_ + roff, dof);
-        if constexpr (kPacked) load_packed<S, DC>((const char *)dout_ + roff, dop);
+        load_chunk<S, DC>((const char *)q_ + (dm.q_row(pb.b, (int)s1, pb.h, (int)l) + lane_elem) * S::kBytes, qf_s[rb]);
+        load_chunk<S, DC>((const char *)dout_ + roff, dof_s[rb]);
+        if constexpr (kPacked) load_packed<S, DC>((const char *)dout_ + roff, dop_s[rb]);
         load_chunk<S, DC>((const char *)out_ + roff, of);
         float dl = 0.f;
 #pragma unroll
-        for (int d = 0; d < DC; ++d) { dl = fmaf(dof[d], of[d], dl); dqa[d] = 0.f; }
-        delta = group_sum<G>(dl);              // the reference's _bwd_preprocess, fused
+        for (int d = 0; d < DC; ++d) { dl = fmaf(dof_s[rb][d], of[d], dl); dqa_s[rb][d] = 0.f; }
+        delta_s[rb] = group_sum<G>(dl);              // the reference's _bwd_preprocess, fused
+        lse_s[rb] = lse_[row];
+        if (stats_ && have_s[rb] && g == 0) stats_[row] = make_float2(lse_s[rb], delta_s[rb]);     // null: a launch of its own does it
     }
-    const float lse = lse_[row];
-    if (stats_ && have && g == 0) stats_[row] = make_float2(lse, delta);     // null: a launch of its own does it
 
     for (int s2 = 0; s2 < dm.V; ++s2) {
         const size_t plane = dm.kv_plane(pb.b, s2, pb.h) * S::kBytes;
@@ -466,6 +472,15 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
         stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, px_bytes, 0);
         stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, px_bytes, 1);
         __syncthreads();
+#pragma unroll
+        for (int rb = 0; rb < ROWS; ++rb) {
+        const bool have = have_s[rb];
+        const size_t crow = crow_s[rb];
+        const float (&qf)[DC] = qf_s[rb];
+        const float (&dof)[DC] = dof_s[rb];
+        const uint32_t (&dop)[kPacked ? DC / 2 : 1] = dop_s[rb];
+        float (&dqa)[DC] = dqa_s[rb];
+        const float delta = delta_s[rb], lse = lse_s[rb];
         for (int c0 = 0; c0 < dm.P; c0 += G) {
             const int my_n = stage_slot_descriptors<S, D>(desc_w, desc_e, crow + (size_t)s2 * dm.P, dm.P, c0, g,
                                                           slot, G, s_w, s_e, CG ? desc_g : nullptr, s_g);
@@ -569,12 +584,16 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
                 atomicAdd(dst + 1, my_gy);
             }
         }
+        }
     }
 
-    if (have) {
 #pragma unroll
-        for (int d = 0; d < DC; ++d) dqa[d] *= dm.sm_scale;
-        store_chunk<S, DC>((char *)dq_ + roff, dqa);
+    for (int rb = 0; rb < ROWS; ++rb) {
+        if (have_s[rb]) {
+#pragma unroll
+            for (int d = 0; d < DC; ++d) dqa_s[rb][d] *= dm.sm_scale;
+            store_chunk<S, DC>((char *)dq_ + roff_s[rb], dqa_s[rb]);
+        }
     }
 }
 
