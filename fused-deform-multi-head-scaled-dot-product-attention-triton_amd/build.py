@@ -20,6 +20,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-munsafe-fp-atomics",                       # hardware float atomics (global_atomic_add_f32 / ds_add_f32)
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-mfma-vgpr-form",          # MFMA accumulators in VGPRs: no copies to and from AGPRs around the loops
     "-Wall", "-Wno-unused-function",
 ]
 

@@ -91,7 +91,8 @@ __device__ __forceinline__ void stage_descriptors(const float2 *__restrict__ coo
 // of every unit lies inside the image. Tables are indexed by entry = (row - ymin) * 4 * nu + (column - xmin).
 // Only the pixels that some tap of the chunk touches are worked on, four at a time ("quads", see
 // window_quads): of the 134 pixels of the padded box of such a chunk, 72 on average.
-constexpr int kWinUnits = 64;                  // units per window: the tables of a wave hold 256 pixels
+constexpr int kWinUnits = 48;                  // units per window: a window is taken only while 4 * units <= 3 * samples,
+                                               // so the tables of a wave hold 192 pixels
 constexpr int kWinEntries = 4 * kWinUnits;
 constexpr int kWinDummy = kWinEntries;         // table entry of the padding pixels of the last quad (a place of its own)
 
@@ -255,7 +256,7 @@ __device__ __forceinline__ void accumulate_taps(const char *__restrict__ base, c
 // mode above; chosen by the host for P >= 64, where a view's samples fill whole chunks. Without WIN the
 // chunks are 64 consecutive samples of the row, whatever views they belong to, and always gather.
 template <typename S, int D, int DC, bool WIN>
-__global__ __launch_bounds__(kGatherWaves *kWave) void fwd_gather_kernel(
+__global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void fwd_gather_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, void *__restrict__ out_, float *__restrict__ lse_, Dims dm)
 {
@@ -613,7 +614,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_gather_kernel(
 // per pixel of the window, each sample's logit and dp blended from those scalars, ds times the bilinear weights
 // scattered into one coefficient per pixel, dq += coefficient * K[pixel] per pixel.
 template <typename S, int D, int DC, bool CG, bool WIN>
-__global__ __launch_bounds__(kGatherWaves *kWave) void bwd_dq_gather_kernel(
+__global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void bwd_dq_gather_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
     const void *__restrict__ dout_, void *__restrict__ dq_, float2 *__restrict__ stats_,
