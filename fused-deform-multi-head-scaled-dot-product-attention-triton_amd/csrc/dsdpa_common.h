@@ -362,10 +362,15 @@ __device__ __forceinline__ floatx4 block_outer_fma(float a, float x, floatx4 acc
 // coefficients (each a 16-bit float; together 16 bits of mantissa), so that acc[e][0] + acc[e][1] is the sum
 // with coefficients good to 2^-16. Lane 4b+i supplies row i of A: `coef` is this lane's row (the high parts
 // in lanes 4b, the low parts in lanes 4b+1, zero elsewhere). The rows come as packed pairs, which two byte
-// permutes per pair of rows turn into "four rows' values of one element".
-template <typename S, int DC>
+// permutes per pair of rows turn into "four rows' values of one element". FIRST: acc is taken as 0 (the
+// instruction's inline constant; saves clearing 4 * DC registers before the first of a run of calls).
+template <typename S, int DC, bool FIRST = false>
 __device__ __forceinline__ void block_blend4(const uint32_t (&r)[4][DC / 2], shortx4 coef, floatx4 (&acc)[DC])
 {
+    if constexpr (FIRST) {
+#pragma unroll
+        for (int e = 0; e < DC; ++e) acc[e] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
 #pragma unroll
     for (int i = 0; i < DC / 2; ++i) {
         const uint32_t lo01 = __builtin_amdgcn_perm(r[1][i], r[0][i], 0x05040100u);

@@ -390,9 +390,8 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
                 // one weighted sum of V rows per quad
                 if constexpr (kBlock) {
                     floatx4 macc[DC];
-#pragma unroll
-                    for (int d = 0; d < DC; ++d) macc[d] = floatx4{0.f, 0.f, 0.f, 0.f};
-                    for (int q0 = 0; q0 < nquads; q0 += NS) {
+                    // (the first step starts the sums from the instruction's constant 0: there is always one)
+                    auto step = [&](int q0, auto first) {
                         const int qd = min(q0 + slot, nquads - 1);
                         const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
                         uint2 cf = reinterpret_cast<const uint2 *>(tC)[4 * qd + (lane & 3)];
@@ -402,8 +401,10 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
                         load_packed<S, DC>(vb + (off.y + lane_byte), r[1]);
                         load_packed<S, DC>(vb + (off.z + lane_byte), r[2]);
                         load_packed<S, DC>(vb + (off.w + lane_byte), r[3]);
-                        block_blend4<S, DC>(r, __builtin_bit_cast(shortx4, cf), macc);
-                    }
+                        block_blend4<S, DC, decltype(first)::value>(r, __builtin_bit_cast(shortx4, cf), macc);
+                    };
+                    step(0, std::true_type{});
+                    for (int q0 = NS; q0 < nquads; q0 += NS) step(q0, std::false_type{});
 #pragma unroll
                     for (int d = 0; d < DC; ++d) acc[d] += macc[d][0] + macc[d][1];
                 } else {
@@ -751,9 +752,8 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
                 // dq += coefficient * K per touched pixel
                 if constexpr (kBlock) {
                     floatx4 macc[DC];
-#pragma unroll
-                    for (int d = 0; d < DC; ++d) macc[d] = floatx4{0.f, 0.f, 0.f, 0.f};
-                    for (int q0 = 0; q0 < nquads; q0 += NS) {
+                    // (the first step starts the sums from the instruction's constant 0: there is always one)
+                    auto step = [&](int q0, auto first) {
                         const int qd = min(q0 + slot, nquads - 1);
                         const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
                         uint2 cf = reinterpret_cast<const uint2 *>(tC)[4 * qd + (lane & 3)];
@@ -763,8 +763,10 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
                         load_packed<S, DC>(kb + (off.y + lane_byte), r[1]);
                         load_packed<S, DC>(kb + (off.z + lane_byte), r[2]);
                         load_packed<S, DC>(kb + (off.w + lane_byte), r[3]);
-                        block_blend4<S, DC>(r, __builtin_bit_cast(shortx4, cf), macc);
-                    }
+                        block_blend4<S, DC, decltype(first)::value>(r, __builtin_bit_cast(shortx4, cf), macc);
+                    };
+                    step(0, std::true_type{});
+                    for (int q0 = NS; q0 < nquads; q0 += NS) step(q0, std::false_type{});
 #pragma unroll
                     for (int d = 0; d < DC; ++d) dqa[d] += macc[d][0] + macc[d][1];
                 } else {
