@@ -306,6 +306,8 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     const int view_chunks = (dm.P + kWave - 1) / kWave;
     const int nchunks = WIN ? dm.V * view_chunks : (dm.N + kWave - 1) / kWave;
     int next_view = 0, next_p0 = 0;                      // WIN: key view and first sample in it of the next chunk
+    // the coordinates of a chunk are requested a chunk ahead (they come from HBM, once each)
+    float2 xy_next = coords[rc.crow + min(lane, min(kWave, WIN ? dm.P : dm.N) - 1)];
     for (int ci = 0; ci < nchunks; ++ci) {
         const int s2c = next_view, p0 = next_p0;         // WIN: this chunk's
         const int c0 = WIN ? s2c * dm.P + p0 : ci * kWave;
@@ -317,7 +319,12 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
         // this lane's sample of the chunk
         const bool live = lane < cnt;
         const int nc = c0 + (live ? lane : cnt - 1);
-        const float2 xy = coords[rc.crow + nc];
+        const float2 xy = xy_next;
+        {
+            const int c0n = WIN ? next_view * dm.P + next_p0 : c0 + kWave;
+            const int cntn = WIN ? min(kWave, dm.P - next_p0) : min(kWave, dm.N - c0n);
+            xy_next = coords[rc.crow + min(c0n + min(lane, cntn - 1), dm.N - 1)];     // (after the last chunk: any valid one)
+        }
         const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
         if (window_ok) {                                 // (the chunk lies in one key view)
             const bool counted = live && ((tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f));
@@ -679,6 +686,8 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     const int view_chunks = (dm.P + kWave - 1) / kWave;
     const int nchunks = WIN ? dm.V * view_chunks : (dm.N + kWave - 1) / kWave;
     int next_view = 0, next_p0 = 0;                      // WIN: key view and first sample in it of the next chunk
+    // the coordinates of a chunk are requested a chunk ahead (they come from HBM, once each)
+    float2 xy_next = coords[rc.crow + min(lane, min(kWave, WIN ? dm.P : dm.N) - 1)];
     for (int ci = 0; ci < nchunks; ++ci) {
         const int s2c = next_view, p0 = next_p0;         // WIN: this chunk's
         const int c0 = WIN ? s2c * dm.P + p0 : ci * kWave;
@@ -690,7 +699,12 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
         // this lane's sample of the chunk
         const bool live = lane < cnt;
         const int nc = c0 + (live ? lane : cnt - 1);
-        const float2 xy0 = coords[rc.crow + nc];
+        const float2 xy0 = xy_next;
+        {
+            const int c0n = WIN ? next_view * dm.P + next_p0 : c0 + kWave;
+            const int cntn = WIN ? min(kWave, dm.P - next_p0) : min(kWave, dm.N - c0n);
+            xy_next = coords[rc.crow + min(c0n + min(lane, cntn - 1), dm.N - 1)];     // (after the last chunk: any valid one)
+        }
         const Taps tp = make_taps(xy0.x, xy0.y, dm.Wimg, dm.Himg);
         if constexpr (WIN) {
             const bool counted = live && ((tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f));
