@@ -301,6 +301,10 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     float m = kNegBig, lsum = 0.f, acc[DC];
 #pragma unroll
     for (int d = 0; d < DC; ++d) acc[d] = 0.f;
+    // WIN: m is kept the same in all slots from chunk to chunk, and the window chunks add their samples' weights
+    // per lane to lwin (same reference m), summed over the wave once, after the last chunk
+    float lwin = 0.f;
+    (void)lwin;
 
     const bool window_ok = WIN && dm.Wimg < 65536 && dm.Himg < 65536;
     const int view_chunks = (dm.P + kWave - 1) / kWave;
@@ -360,20 +364,19 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
                 for (int e = lane; e < 4 * win.nunits; e += kWave) tA[e] = 0.0;
                 wave_lds_sync();
                 // the samples, one per lane: logit from four of the pixel scalars, then the softmax bookkeeping
-                // of the chunk with ONE running maximum for all slots (they are brought to a common one first)
+                // of the chunk with the one running maximum that all slots share
                 const float w0 = live ? tp.w[0] : 0.f, w1 = live ? tp.w[1] : 0.f;
                 const float w2 = live ? tp.w[2] : 0.f, w3 = live ? tp.w[3] : 0.f;
                 float logit = fmaf(w0, tS[te.x], fmaf(w1, tS[te.y], fmaf(w2, tS[te.z], w3 * tS[te.w])));
                 if constexpr (kPacked) logit *= qscale;
-                const float m_new = fmaxf(wave_max(m), wave_max(live ? logit : kNegBig));
+                const float m_new = fmaxf(m, wave_max(live ? logit : kNegBig));
                 const float alpha = __builtin_amdgcn_exp2f(m - m_new);
                 m = m_new;
                 lsum *= alpha;
 #pragma unroll
                 for (int d = 0; d < DC; ++d) acc[d] *= alpha;
                 const float p = live ? __builtin_amdgcn_exp2f(logit - m_new) : 0.f;
-                const float psum = wave_sum(p);
-                if (slot == 0) lsum += psum;
+                lwin = fmaf(lwin, alpha, p);
                 // coefficient of every pixel: sum over the samples of p times the tap's bilinear weight
                 // (every lane adds all four: a tap of weight 0 or a lane beyond the chunk adds 0 to an entry of the tables)
                 atomicAdd(&tA[te.x], (double)(p * w0));
@@ -465,6 +468,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
         const float alpha = __builtin_amdgcn_exp2f(m - m_new);
         m = m_new;
         lsum *= alpha;
+        if constexpr (WIN) lwin *= alpha;
 #pragma unroll
         for (int d = 0; d < DC; ++d) acc[d] *= alpha;
 #pragma unroll
@@ -479,6 +483,19 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
                 accumulate_taps<S, DC>(vb, e, c, acc);
             }
         }
+        if constexpr (WIN) {                             // back to one running maximum for all slots
+            const float mu = wave_max(m);
+            const float a = __builtin_amdgcn_exp2f(m - mu);
+            m = mu;
+            lsum *= a;
+            lwin *= a;
+#pragma unroll
+            for (int d = 0; d < DC; ++d) acc[d] *= a;
+        }
+    }
+    if constexpr (WIN) {
+        const float lw = wave_sum(lwin);
+        if (slot == 0) lsum += lw;
     }
 
     // merge the NS slots (each has its own running max / sum / accumulator)
