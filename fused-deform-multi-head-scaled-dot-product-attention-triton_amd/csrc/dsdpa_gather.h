@@ -220,6 +220,39 @@ __device__ __forceinline__ void window_dots(const char *__restrict__ base, const
     for (int k = 0; k < 4; ++k) d[k] = group_sum<G>(d[k]);
 }
 
+// The same with EIGHT lanes per pixel (16-bit storage, rows of 16 lanes): lane g2 of a slot takes DC elements of
+// each half of the row (bytes o[k] + h * HALF, o[k] with the lane's offset inside a half included), so a step of the
+// wave covers eight quads instead of four with three lane sums per product instead of four, and a chunk's
+// pixels take about half as many steps. xp[h]: x's elements of the same two places.
+template <typename S, int DC, int HALF>
+__device__ __forceinline__ void window_dots_half(const char *__restrict__ base, const unsigned (&o)[4],
+                                                 const uint32_t (&xp)[2][DC / 2], float (&d)[4])
+{
+    uint32_t r[4][2][DC / 2];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        load_packed<S, DC>(base + o[k], r[k][0]);
+        load_packed<S, DC>(base + o[k] + HALF, r[k][1]);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float acc = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int i = 0; i < DC / 2; ++i) {
+                if constexpr (S::kBf16)
+                    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(dsdpa_bf16x2, xp[h][i]),
+                                                          __builtin_bit_cast(dsdpa_bf16x2, r[k][h][i]), acc, false);
+                else
+                    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(dsdpa_f16x2, xp[h][i]),
+                                                 __builtin_bit_cast(dsdpa_f16x2, r[k][h][i]), acc, false);
+            }
+        }
+        d[k] = group_sum<8>(acc);
+    }
+}
+
 // Bilinear blend of the four taps of one sample, this lane's DC elements. `e`: the taps' byte offsets from
 // the (uniform) base, this lane's part of the row included.
 template <typename S, int DC>
@@ -298,6 +331,15 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
         for (int d = 0; d < DC; ++d) qf[d] *= qscale;
     }
 
+    // window chunks with 16 lanes per row take their dot products with 8 lanes per pixel (window_dots_half); the
+    // q row is kept in LDS for that and read in that layout per chunk (no registers to spare for it between chunks)
+    constexpr bool kHalf = WIN && kPacked && G == 16;
+    constexpr unsigned kHalfBytes = D * S::kBytes / 2;
+    __shared__ uint4 s_xq[kHalf ? kGatherWaves : 1][kHalf ? D / 8 : 1];
+    if constexpr (kHalf) {
+        if (lane < D / 8) s_xq[wave][lane] = reinterpret_cast<const uint4 *>((const char *)q_ + rc.q_off * S::kBytes)[lane];
+    }
+
     float m = kNegBig, lsum = 0.f, acc[DC];
 #pragma unroll
     for (int d = 0; d < DC; ++d) acc[d] = 0.f;
@@ -346,18 +388,39 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
                 const unsigned *q_off = s_qoff[wave], *q_ent = s_qent[wave];
                 const int nquads = window_quads(win, te, lane, dm.Wimg, view_byte, rnu, kRow, s_bitmap[wave],
                                                 s_qoff[wave], s_qent[wave]);
-                for (int q0 = 0; q0 < nquads; q0 += NS) {
-                    const int qd = min(q0 + slot, nquads - 1);
-                    const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
-                    const uint4 ent = *reinterpret_cast<const uint4 *>(q_ent + 4 * qd);
-                    const unsigned o[4] = { off.x + lane_byte, off.y + lane_byte, off.z + lane_byte, off.w + lane_byte };
-                    float d4[4];
-                    window_dots<S, DC, G>(kb, o, qf, qp, d4);
-                    if (g == 0) {
-                        tS[ent.x] = d4[0];
-                        tS[ent.y] = d4[1];
-                        tS[ent.z] = d4[2];
-                        tS[ent.w] = d4[3];
+                if constexpr (kHalf) {
+                    const unsigned lb2 = (unsigned)(lane & 7) * DC * S::kBytes;
+                    uint32_t xq[2][DC / 2];
+                    load_packed<S, DC>((const char *)s_xq[wave] + lb2, xq[0]);
+                    load_packed<S, DC>((const char *)s_xq[wave] + lb2 + kHalfBytes, xq[1]);
+                    for (int q0 = 0; q0 < nquads; q0 += 2 * NS) {
+                        const int qd = min(q0 + (lane >> 3), nquads - 1);
+                        const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
+                        const uint4 ent = *reinterpret_cast<const uint4 *>(q_ent + 4 * qd);
+                        const unsigned o[4] = { off.x + lb2, off.y + lb2, off.z + lb2, off.w + lb2 };
+                        float d4[4];
+                        window_dots_half<S, DC, kHalfBytes>(kb, o, xq, d4);
+                        if ((lane & 7) == 0) {
+                            tS[ent.x] = d4[0];
+                            tS[ent.y] = d4[1];
+                            tS[ent.z] = d4[2];
+                            tS[ent.w] = d4[3];
+                        }
+                    }
+                } else {
+                    for (int q0 = 0; q0 < nquads; q0 += NS) {
+                        const int qd = min(q0 + slot, nquads - 1);
+                        const uint4 off = *reinterpret_cast<const uint4 *>(q_off + 4 * qd);
+                        const uint4 ent = *reinterpret_cast<const uint4 *>(q_ent + 4 * qd);
+                        const unsigned o[4] = { off.x + lane_byte, off.y + lane_byte, off.z + lane_byte, off.w + lane_byte };
+                        float d4[4];
+                        window_dots<S, DC, G>(kb, o, qf, qp, d4);
+                        if (g == 0) {
+                            tS[ent.x] = d4[0];
+                            tS[ent.y] = d4[1];
+                            tS[ent.z] = d4[2];
+                            tS[ent.w] = d4[3];
+                        }
                     }
                 }
                 if (lane == 0) tA[kWinDummy] = 0.0;
