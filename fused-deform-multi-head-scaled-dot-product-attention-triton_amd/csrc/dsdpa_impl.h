@@ -571,8 +571,11 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     // binning workgroups (1024 threads, up to 135 KB of LDS) wait until it ends, and with the binning done
     // first the dq and dk/dv kernels only take turns (measured at 64x64, D = 128: 14.2 ms against 14.5 for the
     // step, each kernel stretched to the sum of both) -- those shapes run the backward on the caller's stream.
+    // So do small problems: the fork and join cost about 0.05 ms of host time per call, which a backward of
+    // under two million query*samples (0.15 ms of kernels) does not win back.
     hipStream_t bst = st;
-    SideLane *side = cell_binned && staged && !(flags & DSDPA_FLAG_SINGLE_STREAM) ? side_lane() : nullptr;
+    const bool worth_forking = (long long)dm.rows * dm.N >= (2ll << 20);
+    SideLane *side = cell_binned && staged && worth_forking && !(flags & DSDPA_FLAG_SINGLE_STREAM) ? side_lane() : nullptr;
     const size_t ncounters = cell_binned ? wl.counters_bytes / 4 : 0;
     SideJoin joiner;
     if (side && hipEventRecord(side->fork, st) == hipSuccess &&

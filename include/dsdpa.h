@@ -122,7 +122,9 @@ enum { DSDPA_FLAG_DETERMINISTIC = 1, DSDPA_FLAG_COORDS_GRAD = 2, DSDPA_FLAG_SING
 /* DSDPA_FLAG_SINGLE_STREAM: enqueue every launch of the backward on `stream` itself. By default the dk/dv side
  * (clearing the accumulators, delta, the cell binning, the dk/dv kernel) runs on a second stream of the
  * library's beside the tap table and the dq kernel: neither side reads what the other writes, and the two
- * main kernels leave each other idle issue slots (C2: 7 % off the fwd+bwd step). Same results either way. */
+ * main kernels leave each other idle issue slots (C2: 7 % off the fwd+bwd step). Only on shapes whose K/V planes
+ * fit in LDS, and only from 2^21 query*samples (B*V*H*L * V*P) up: below that the fork and join cost more host
+ * time than the overlap saves. Same results either way. */
 /* DSDPA_FLAG_COORDS_GRAD: the workspace has room for the coordinate gradient's part of the per-coordinate
  * table (16 more bytes per coordinate pair where the staged kernels run), so that a backward given dcoords
  * stays on the staged dq kernel. Pass the same flags to dsdpa_bwd_workspace_bytes and to dsdpa_bwd_*;

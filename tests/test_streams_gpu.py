@@ -57,12 +57,15 @@ def c_abi_backward(q, k, v, c, do, Himg, Wimg, flags, stream=None):
     return out, dq, dk, dv, (fws, ws, lse)
 
 
+# The backward forks only from 2^21 query*samples (B*V*H*L * V*P) up and only on shapes whose planes fit in LDS:
+# s51, s53, s54 fork; s52 (gather dq) and s55 (small) run on the caller's stream whatever the flag.
 SHAPES = [
     # seed B V H Himg Wimg D   P  dtype
-    (51, 2, 3, 2, 6, 7, 32, 11, torch.float32),        # planes in LDS
+    (51, 2, 6, 3, 18, 18, 32, 32, torch.float32),      # planes in LDS
     (52, 1, 2, 2, 30, 30, 64, 5, torch.float32),       # gather dq
-    (53, 2, 2, 3, 9, 8, 64, 16, torch.bfloat16),       # fp32 accumulators in the workspace + casts
-    (54, 1, 4, 1, 5, 5, 128, 33, torch.float16),
+    (53, 2, 4, 8, 16, 16, 64, 32, torch.bfloat16),     # fp32 accumulators in the workspace + casts
+    (54, 2, 4, 32, 8, 8, 128, 33, torch.float16),
+    (55, 2, 3, 2, 6, 7, 32, 11, torch.float32),        # small
 ]
 
 
@@ -103,13 +106,14 @@ def test_caller_stream_is_ordered_before_and_after():
         assert abs(s_.item() - r_.double().sum().item()) <= 1e-4 * r_.double().abs().sum().item()
 
 
+@pytest.mark.parametrize("dims", [(2, 3, 4, 10, 9, 32, 13), (2, 4, 16, 12, 12, 32, 32)], ids=["small", "forking"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
-def test_captured_graph_replays_to_the_eager_result(dtype):
+def test_captured_graph_replays_to_the_eager_result(dtype, dims):
     """Forward + backward captured once in a HIP graph (torch.cuda.graph), replayed with new inputs copied into
     the static buffers, with eager work and synchronisations between the replays; every replay is compared
     with an eager call on the same inputs."""
-    say(f"[case] graph capture {dtype}")
-    B, V, H, Himg, Wimg, D, P = 2, 3, 4, 10, 9, 32, 13
+    say(f"[case] graph capture {dtype} {dims}")
+    B, V, H, Himg, Wimg, D, P = dims                   # the second: large enough for the backward to fork
     q, k, v, c, do = make(71, B, V, H, Himg, Wimg, D, P, dtype)
     sq, sk, sv = (t.clone().requires_grad_(True) for t in (q, k, v))
     sc, sdo = c.clone(), do.clone()
@@ -149,8 +153,8 @@ def test_two_host_threads_with_their_own_streams():
     one second stream per thread and device); both get the single-stream result."""
     import threading
     say("[case] two host threads")
-    cases = [make(91, 2, 3, 2, 9, 8, 32, 12), make(92, 1, 4, 3, 7, 11, 64, 9)]
-    dims = [(9, 8), (7, 11)]
+    cases = [make(91, 2, 4, 16, 12, 12, 32, 32), make(92, 2, 4, 16, 10, 13, 64, 32)]     # (both backwards fork)
+    dims = [(12, 12), (10, 13)]
     refs = [c_abi_backward(*cases[i], *dims[i], _native.FLAG_SINGLE_STREAM) for i in range(2)]
     torch.cuda.synchronize()
     results, errors = [None, None], []
