@@ -8,6 +8,7 @@ before use, and timing uses HIP events on the current stream (median of ``--rep`
 
     python sweep.py --b 2 --h 8 --d 32 --iw 18            # full sweep, prints a table per mode
     python sweep.py --quick                               # S, P in {2, 6, 12} only
+    python sweep.py --views 24 --samples 16 --path lds    # one point, on a named kernel path
 
 Besides the printed tables it leaves, in ``--save-path`` (default ``./results``), ``logs.txt`` with the ``[Mem]``
 lines and one latency CSV (and one peak-memory CSV) per mode and ``P_samples`` -- the files the reference's
@@ -24,6 +25,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 if HERE not in sys.path:
     sys.path.insert(0, HERE)
 
+from ops import _native                                         # noqa: E402
 from ops.torch import deform_sdpa_torch as ref_deform_sdpa      # noqa: E402
 from ops.triton import deform_sdpa_triton as fused_deform_sdpa  # noqa: E402
 
@@ -118,6 +120,11 @@ def main(argv=None):
     ap.add_argument("--sm-scale", type=float, default=0.5)
     ap.add_argument("--dtype", default="fp32", choices=["fp32", "bf16", "fp16"])
     ap.add_argument("--quick", action="store_true", help="S, P in {2, 6, 12} only")
+    ap.add_argument("--views", default=None, help="comma-separated S_views instead of the sweep's")
+    ap.add_argument("--samples", default=None, help="comma-separated P_samples instead of the sweep's")
+    ap.add_argument("--path", default="auto", choices=["auto", "lds", "gather"],
+                    help="kernel path of the fused provider: chosen by shape, K/V planes staged in LDS, or taps "
+                         "gathered through L1/L2")
     ap.add_argument("--no-torch", action="store_true", help="skip timing the eager provider")
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--rep", type=int, default=20)
@@ -127,6 +134,11 @@ def main(argv=None):
     dtype = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[args.dtype]
     S_LIST = [2, 6, 12] if args.quick else [2, 4, 6, 8, 10, 12]
     P_LIST = [2, 6, 12] if args.quick else [2, 4, 6, 8, 10, 12]
+    if args.views:
+        S_LIST = [int(x) for x in args.views.split(",")]
+    if args.samples:
+        P_LIST = [int(x) for x in args.samples.split(",")]
+    prev_path = _native.set_path({"auto": _native.PATH_AUTO, "lds": _native.PATH_LDS, "gather": _native.PATH_GATHER}[args.path])
     providers = ["fused"] if args.no_torch else ["fused", "torch"]
     dev = torch.device("cuda", torch.cuda.current_device())
     os.makedirs(args.save_path, exist_ok=True)
@@ -149,6 +161,7 @@ def main(argv=None):
                           f"H={args.iw} P={P} D={args.d} | peak={peak:.1f} MB", file=log, flush=True)
                 del q, k, v, coords
     log.close()
+    _native.set_path(prev_path)
     write_csv_tables(rows, args, providers, S_LIST, P_LIST)
     for mode in ("fwd", "bwd"):
         print(f"\nlatency (ms), mode={mode}, B={args.b} H={args.h} D={args.d} W={args.iw} dtype={args.dtype}")
