@@ -91,8 +91,9 @@ __device__ __forceinline__ void stage_descriptors(const float2 *__restrict__ coo
 // of every unit lies inside the image. Tables are indexed by entry = (row - ymin) * 4 * nu + (column - xmin).
 // Only the pixels that some tap of the chunk touches are worked on, four at a time ("quads", see
 // window_quads): of the 134 pixels of the padded box of such a chunk, 72 on average.
-constexpr int kWinUnits = 48;                  // units per window: a window is taken only while 4 * units <= 3 * samples,
-                                               // so the tables of a wave hold 192 pixels
+constexpr int kWinUnits = 56;                  // units per window: a window is taken only while 8 * units <= 7 * samples
+                                               // (the work goes with the touched pixels, the tables with the box):
+                                               // the tables of a wave hold 224 pixels
 constexpr int kWinEntries = 4 * kWinUnits;
 constexpr int kWinDummy = kWinEntries;         // table entry of the padding pixels of the last quad (a place of its own)
 
@@ -375,7 +376,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
         if (window_ok) {                                 // (the chunk lies in one key view)
             const bool counted = live && ((tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f));
             const Window win = chunk_window(tp, counted, dm.Wimg, dm.Himg);
-            if (win.nunits > 0 && win.nunits <= kWinUnits && 4 * win.nunits <= 3 * cnt) {
+            if (win.nunits > 0 && win.nunits <= kWinUnits && 8 * win.nunits <= 7 * cnt) {
                 const unsigned kRow = (unsigned)dm.kv_sl * S::kBytes;       // bytes between neighbouring pixels of K and V
                 constexpr bool kBlock = kPacked && G >= 4;         // V rows blended by the block matrix instruction
                 float *tS = s_dot[wave];
@@ -714,8 +715,8 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     static_assert(G >= 1 && G <= 16 && G * DC == D, "lane split");
     __shared__ float4 s_w[kGatherWaves][kWave];
     __shared__ uint4 s_e[kGatherWaves][kWave];
-    __shared__ float4 s_gx[CG ? kGatherWaves : 1][kWave];
-    __shared__ float4 s_gy[CG ? kGatherWaves : 1][kWave];
+    __shared__ float4 s_gx[CG ? kGatherWaves : 1][CG ? kWave : 1];
+    __shared__ float4 s_gy[CG ? kGatherWaves : 1][CG ? kWave : 1];
     __shared__ float2 s_hand[CG ? 1 : kGatherWaves][kWave];                      // (p, sm_scale * ds) of the chunk's samples
     static_assert(!(CG && WIN), "the window mode has no coordinate gradient");
     constexpr int kTab = WIN ? kGatherWaves : 1, kTabUnits = WIN ? kWinUnits : 1;
@@ -789,7 +790,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
         if constexpr (WIN) {
             const bool counted = live && ((tp.w[0] != 0.f) | (tp.w[1] != 0.f) | (tp.w[2] != 0.f) | (tp.w[3] != 0.f));
             const Window win = window_ok ? chunk_window(tp, counted, dm.Wimg, dm.Himg) : Window{0, 0, 0, 0};
-            if (win.nunits > 0 && win.nunits <= kWinUnits && 4 * win.nunits <= 3 * cnt) {
+            if (win.nunits > 0 && win.nunits <= kWinUnits && 8 * win.nunits <= 7 * cnt) {
                 const unsigned kRow = (unsigned)dm.kv_sl * S::kBytes;       // bytes between neighbouring pixels of K and V
                 constexpr bool kBlock = kPacked && G >= 4;
                 float *tS = s_dotk[wave], *tT = s_dotv[wave];
