@@ -280,7 +280,8 @@ __device__ __forceinline__ void widen_words(const uint32_t (&w)[DC * S::kBytes /
 // `ncells` then being the list's capacity wmax per (b, s2); empty slots leave at once.
 struct CellGrid {
     int colour, oy, ox, step, ncx, ncells;
-    unsigned nwork;                         // B*H*V*ncells < 2^31
+    int bh0;                                // first (batch, head) pair of this launch (b * H + h)
+    unsigned nwork;                         // pairs of this launch * V * ncells < 2^31
     FastDiv div_cells, div_ncx, div_v, div_h;
 };
 
@@ -317,8 +318,9 @@ void bwd_dkdv_cell_kernel(
     // plane-major: (b, h, s2, cell or work item)
     unsigned t = cg.div_cells.div(work);
     const int ci = (int)(work - t * (unsigned)cg.ncells);
-    const unsigned bh = cg.div_v.div(t);
-    const int s2 = (int)(t - bh * (unsigned)dm.V);
+    const unsigned bhl = cg.div_v.div(t);                      // pair within this launch
+    const int s2 = (int)(t - bhl * (unsigned)dm.V);
+    const unsigned bh = (unsigned)cg.bh0 + bhl;
     const int b = (int)cg.div_h.div(bh);
     const int h = (int)(bh - (unsigned)b * (unsigned)dm.H);
     const size_t grp = (size_t)b * dm.V + s2;
@@ -423,13 +425,13 @@ void bwd_dkdv_cell_kernel(
     auto load_frac = [&](unsigned cstart) -> float2 {
         return (fracl && cstart < hi) ? fracl[min(cstart + (unsigned)lane, hi - 1u)] : make_float2(0.f, 0.f);
     };
-    // HANDED: the entry's pair, gathered one chunk ahead (so the ids are fetched two chunks ahead). Rows of this
-    // wave's (b, h) are a uniform base plus a 32-bit byte offset (the host checks V*H*L*N*8 < 2^32).
-    const char *handed_bh = (const char *)(handed_ + ((size_t)b * dm.V * dm.H + h) * dm.L * (size_t)dm.N);
+    // HANDED: the entry's pair, gathered one chunk ahead (so the ids are fetched two chunks ahead). The pairs of
+    // this launch's (batch, head) pairs lie as [pair][s1][l][sample]; those of this wave's pair are a uniform base
+    // plus a 32-bit byte offset (the host checks V*L*N*8 < 2^32).
+    const char *handed_bh = (const char *)(handed_ + (size_t)bhl * dm.V * dm.L * (size_t)dm.N);
     auto load_pair = [&](unsigned sid) -> float2 {
-        const unsigned qlx = dm.divP.div(sid), px = sid - qlx * (unsigned)dm.P;
-        const unsigned s1x = dm.divL.div(qlx), lx = qlx - s1x * (unsigned)dm.L;
-        const unsigned off = ((s1x * (unsigned)dm.H * (unsigned)dm.L + lx) * (unsigned)dm.N + (unsigned)s2 * (unsigned)dm.P + px) * 8u;
+        const unsigned qlx = dm.divP.div(sid), px = sid - qlx * (unsigned)dm.P;       // qlx = s1*L + l
+        const unsigned off = (qlx * (unsigned)dm.N + (unsigned)s2 * (unsigned)dm.P + px) * 8u;
         return *reinterpret_cast<const float2 *>(handed_bh + off);
     };
     if constexpr (kQuad) {

@@ -707,7 +707,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
     const void *__restrict__ dout_, void *__restrict__ dq_, float2 *__restrict__ stats_,
-    float *__restrict__ dcoords_, float2 *__restrict__ handed_, Dims dm)
+    float *__restrict__ dcoords_, float2 *__restrict__ handed_, Dims dm, int work0, int work_end)
 {
     constexpr int G = D / DC;
     constexpr int NS = kWave / G;
@@ -729,8 +729,9 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     __shared__ unsigned s_bitmap[kTab][kWinEntries / 32];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
-    const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
-    if (work >= dm.rows) return;
+    // a launch covers the query rows [work0, work_end) of the (b, h, s1, l) order: a group of (batch, head) pairs
+    const int work = work0 + xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
+    if (work >= work_end) return;
     const RowCtx rc = decode_row(work, dm, D);
     const int g = lane % G, slot = lane / G, lane_elem = g * DC;
     const unsigned lane_byte = (unsigned)lane_elem * S::kBytes;
@@ -755,9 +756,10 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     const float qscale = dm.sm_scale * kLog2e;
     const float lse = lse_[rc.row];
     if (stats_ && lane == 0) stats_[rc.row] = make_float2(lse, delta);     // null: a launch of its own does it
-    // handed_ (may be null; never with CG): per sample, in the order of the coordinates of this head's rows,
-    // (p, sm_scale * ds) for the dk/dv kernel, which then need not recompute them from the taps
-    float2 *handed_row = handed_ ? handed_ + (size_t)rc.row * dm.N : nullptr;
+    // handed_ (may be null; never with CG): per sample, (p, sm_scale * ds) for the dk/dv kernel, which then need
+    // not recompute them from the taps: [pair (b, h) of this launch][s1][l][sample], i.e. in the order of the work
+    // items of this launch and, inside a row, of its coordinates
+    float2 *handed_row = handed_ ? handed_ + (size_t)(work - work0) * dm.N : nullptr;
 
     float dqa[DC];
 #pragma unroll

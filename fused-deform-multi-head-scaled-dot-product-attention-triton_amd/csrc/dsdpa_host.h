@@ -165,8 +165,9 @@ inline DescLayout desc_layout(size_t B, size_t V, size_t Himg, size_t Wimg, size
 //   sorted   B*V*(V*L*P) u32                 sample ids ordered by cell
 //   frac     B*V*(V*L*P) x 8 bytes           (fx, fy) of the same samples, same order
 //   items    B*V*wmax x 16 bytes             work list of the dk/dv kernel: (cell, first entry, end) per item
-//   handed   rows*V*P x 8 bytes              (p, sm_scale*ds) per query*sample, dq kernel -> dk/dv kernel (shapes
-//                                            on the gather kernels only)
+//   handed   bhg*V*L*(V*P) x 8 bytes         (p, sm_scale*ds) per query*sample of one GROUP of bhg (batch, head) pairs,
+//                                            dq kernel -> dk/dv kernel (shapes on the gather kernels only); at most
+//                                            kHandedCapBytes whatever the shape
 //   acc      2*n floats                      fp32 dk/dv accumulators (16-bit storage only)
 //   desc     20 bytes per coordinate pair    descriptor table (only when the plane kernels apply); 36 with
 //                                            the coordinate gradient
@@ -182,6 +183,7 @@ int sort_cell_lists(void *temp, size_t temp_bytes, const unsigned *ids_in, unsig
 
 struct WorkspaceLayout {
     size_t delta, counters, start, sorted, frac, items, handed, handed_bytes, acc, desc, sorted2, seg, sorttmp, sorttmp_bytes, total;
+    int bh_group;               // (batch, head) pairs whose pairs the handed buffer holds at a time; 0: nothing is handed over
     DescLayout dl;
     size_t counters_bytes;
     int NC;                     // cells of the grid
@@ -220,6 +222,28 @@ inline int views_per_group(size_t V, size_t L, size_t D, size_t esize, size_t P,
     while (groups > 1 && M / (groups * NC) < 48) --groups;
     return (int)((V + groups - 1) / groups);
 }
+// The dq kernel can hand (p, sm_scale * ds) of every query*sample over to the dk/dv kernel, which then neither
+// recomputes them nor needs the cell's taps. The whole backward's pairs would be rows * V*P * 8 bytes (0.54 GB
+// for 2 x 4 views x 8 heads x 64x64, 64 samples per view): more than the tensors, and more than the memory-side
+// cache holds. So the backward runs in GROUPS of (batch, head) pairs -- dq of a group, then dk/dv of the same
+// group, the cell lists being shared by all heads -- and the buffer holds one group's pairs: at most
+// kHandedCapBytes, which also stay in the memory-side cache between the two kernels. Returns the (batch, head)
+// pairs per group, 0 when nothing is handed over: shapes on the staged kernels (dq and dk/dv run side by side
+// there), the deterministic backward (its four colour launches recompute), the coordinate gradient (its dq
+// kernel does not write pairs), one pair's samples beyond the cap or beyond 32-bit byte offsets.
+constexpr size_t kHandedCapBytes = (size_t)128 << 20;
+inline int handed_group(size_t B, size_t V, size_t H, size_t L, size_t D, size_t P, size_t esize, bool deterministic,
+                        bool coords_grad)
+{
+    if (deterministic || coords_grad || plane_path_fits(L, D, esize)) return 0;
+    const size_t per_bh = V * L * (V * P) * 8;
+    if (per_bh >= ((size_t)1 << 32) || per_bh > kHandedCapBytes) return 0;
+    size_t g = kHandedCapBytes / per_bh;
+    if (g > B * H) g = B * H;
+    // groups of equal size (the last one may be smaller by less than one pair per group)
+    const size_t ngroups = (B * H + g - 1) / g;
+    return (int)((B * H + ngroups - 1) / ngroups);
+}
 inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Himg, size_t Wimg, size_t D, size_t P,
                                         bool storage16, bool deterministic, bool coords_grad)
 {
@@ -228,8 +252,8 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     w.NC = (int)((Himg + 1) * (Wimg + 1));
     size_t off = 0;
     w.delta = off; off += round256(rows * 8);           // (lse, delta) per row
-    const bool handed = !deterministic && !plane_path_fits(Himg * Wimg, D, storage16 ? 2 : 4) &&
-                        V * H * Himg * Wimg * (V * P) * 8 < ((size_t)1 << 32);
+    w.bh_group = handed_group(B, V, H, Himg * Wimg, D, P, storage16 ? 2 : 4, deterministic, coords_grad);
+    const bool handed = w.bh_group > 0;
     w.vpg = views_per_group(V, Himg * Wimg, D, storage16 ? 2 : 4, P, (size_t)w.NC, handed);
     w.NK = w.NC * (int)((V + w.vpg - 1) / w.vpg);
     w.counters = off; w.counters_bytes = round256(B * V * (size_t)w.NK * 4); off += w.counters_bytes;
@@ -238,12 +262,10 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     w.frac = off; off += round256(B * V * (V * Himg * Wimg * P) * 8);
     work_list_geometry(V, Himg * Wimg, P, (size_t)w.NK, &w.piece, &w.wmax);
     w.items = off; off += round256(B * V * (size_t)w.wmax * 16);
-    // (p, sm_scale * ds) per query*sample, handed from the dq kernel to the dk/dv kernel: on shapes whose planes do
-    // not fit in LDS (the backward then runs dq before dk/dv on one stream), not for the deterministic backward
-    // (its four colour launches recompute), and only while a (batch item)'s pairs can be addressed with 32 bits
+    // (p, sm_scale * ds) per query*sample of one group of (batch, head) pairs, handed from the dq kernel to the
+    // dk/dv kernel (see handed_group)
     w.handed = off;
-    w.handed_bytes = 0;
-    if (handed) w.handed_bytes = round256(rows * (V * P) * 8);
+    w.handed_bytes = round256((size_t)w.bh_group * V * Himg * Wimg * (V * P) * 8);
     off += w.handed_bytes;
     w.acc = off; if (storage16) off += round256(2 * rows * D * 4);
     // with the coordinate gradient the staged dq kernel needs more LDS; where it no longer fits, dq takes the

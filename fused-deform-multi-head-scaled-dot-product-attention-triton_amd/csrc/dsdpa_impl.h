@@ -175,26 +175,28 @@ int launch_bwd_gather(const void *q, const void *k, const void *v, const float *
     return check_launch();
 }
 
+// The query rows of the (batch, head) pairs [bh0, bh0 + nbh) (all of them: 0, B*H).
 template <typename S, int D>
 int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const float *coords, const void *out,
                          const float *lse, const void *dout, void *dq, float2 *stats, float *dcoords,
-                         float2 *handed, const Dims &dm, hipStream_t st)
+                         float2 *handed, const Dims &dm, int bh0, int nbh, hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
-    const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
+    const int work0 = bh0 * dm.V * dm.L, work_end = (bh0 + nbh) * dm.V * dm.L;      // (at most dm.rows)
+    const int blocks = (work_end - work0 + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(2, st);
     if (dcoords)
         DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, true, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
-                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm);
+                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm, work0, work_end);
     else if (gather_window_mode(dm.P))
         DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, false, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
-                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm);
+                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm, work0, work_end);
     else
         DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, false, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
-                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm);
+                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm, work0, work_end);
     return check_launch();
 }
 
@@ -443,7 +445,8 @@ template <typename S, int D>
 int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const float *coords,
                          const float2 *stats, const void *dout, const unsigned *start, const unsigned *sorted,
                          const float2 *frac, const uint4 *items, unsigned wmax, const float2 *handed,
-                         float *dk_acc, float *dv_acc, const Dims &dm, int NC, bool deterministic, hipStream_t st)
+                         float *dk_acc, float *dv_acc, const Dims &dm, int NC, bool deterministic, int bh0, int nbh,
+                         hipStream_t st)
 {
     constexpr int DC = CellChunk<S, D>::value;
     ScopedKernelTimer timer(1, st);
@@ -457,8 +460,9 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
         cg.ncx = (cw - cg.ox + cg.step - 1) / cg.step;
         cg.ncells = cg.ncx * ((ch - cg.oy + cg.step - 1) / cg.step);
         if (colour < 0) cg.ncells = (int)wmax;          // work-list mode: one wave per item slot
-        const long long nwork = (long long)dm.B * dm.H * dm.V * cg.ncells;
+        const long long nwork = (long long)nbh * dm.V * cg.ncells;       // the pairs [bh0, bh0 + nbh) of (batch, head)
         if (nwork >= 0x7fffffffll - kCellWaves) return DSDPA_ERR_TOO_LARGE;
+        cg.bh0 = bh0;
         cg.nwork = (unsigned)nwork;
         cg.div_cells = FastDiv::make((unsigned)cg.ncells);
         cg.div_ncx = FastDiv::make((unsigned)cg.ncx);
@@ -607,23 +611,30 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, bst)) != DSDPA_OK) return rc;
     if (deterministic && (rc = launch_list_ordering(dm, wl, ws, bst)) != DSDPA_OK) return rc;
     float2 *dq_stats = side_on ? nullptr : stats;       // the dq kernel writes them only when dk/dv runs behind it
+    // With the pairs handed over the two kernels go group by group of (batch, head) pairs: the buffer holds one
+    // group's pairs (workspace_layout), and the dk/dv kernel of a group finds them where the dq kernel of the same
+    // group has just left them. Otherwise one launch each covers all pairs.
+    const int nbh_all = dm.B * dm.H, bh_step = handed ? wl.bh_group : nbh_all;
 #define DSDPA_BWD_CASE(DD)                                                                                      \
     case DD:                                                                                                    \
         if (fused_atomics && !dcoords) {                                                                        \
             rc = launch_bwd_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dk_acc, dv_acc, dm, st);         \
-        } else {                                                                                                \
+            break;                                                                                              \
+        }                                                                                                       \
+        for (int bh0 = 0; bh0 < nbh_all && rc == DSDPA_OK; bh0 += bh_step) {                                    \
+            const int nbh = bh_step < nbh_all - bh0 ? bh_step : nbh_all - bh0;                                  \
             rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, dq_stats,     \
                                                      desc_g, dcoords, dm, st)                                   \
                         : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dq_stats, dcoords,   \
-                                                      handed, dm, st);                                          \
+                                                      handed, dm, bh0, nbh, st);                                \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
                 rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, stats, dout, start, sorted, frac,             \
                                                  (const uint4 *)(ws + wl.items), wl.wmax, handed, dk_acc,       \
-                                                 dv_acc, dm, wl.NK, deterministic, bst);                        \
+                                                 dv_acc, dm, wl.NK, deterministic, bh0, nbh, bst);              \
             else if (rc == DSDPA_OK)                                                                            \
                 rc = launch_bwd_dkdv_tile<S, DD>(q, k, v, coords, stats, dout, dk_acc, dv_acc, dm, st);         \
-            if (rc == DSDPA_OK) rc = joiner.join();                                                              \
         }                                                                                                       \
+        if (rc == DSDPA_OK) rc = joiner.join();                                                                 \
         break;
     switch (D) {
         DSDPA_BWD_CASE(16)

@@ -35,15 +35,23 @@ def oracle_on_slices(q, k, v, coords, dout, W, Himg, scale, slices, forward=True
         dq, dk, dv = oracle_bwd(*args, f(slice_bh(dout, b, h)), W, Himg, scale)
         return out, dq, dk, dv
 
-    with ThreadPoolExecutor(max_workers=max(1, len(slices))) as pool:
+    with ThreadPoolExecutor(max_workers=max(1, min(16, len(slices)))) as pool:
         return dict(zip(slices, pool.map(one, slices)))
 
 
-def spread_slices(B, H):
-    """Four (batch, head) pairs whose batch and head indices differ from each other wherever the shape allows."""
+def spread_slices(B, H, n=4):
+    """n (batch, head) pairs (all of them when n >= B*H) whose batch and head indices are spread over the shape: the
+    first and the last batch item and head are always among them."""
+    if n >= B * H:
+        return [(b, h) for b in range(B) for h in range(H)]
     cand = [(0, 1 % H), (B - 1, 0), (0, H - 1), (B - 1, H // 2)]
+    # further pairs: heads taken round with a stride coprime to H, batch items alternating
+    step = next(s for s in (3, 5, 7, 1) if H % s or s == 1)
+    cand += [((i + 1) % B, (2 + i * step) % H) for i in range(B * H)]
     out = []
     for c in cand:
         if c not in out:
             out.append(c)
+        if len(out) == n:
+            break
     return out

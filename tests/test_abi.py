@@ -60,9 +60,19 @@ def test_workspace_bytes():
         vpg = (V + g - 1) // g
         return (V + vpg - 1) // vpg
 
+    def handed_group(B, V, H, Himg, Wimg, D, P, storage16):
+        """(batch, head) pairs whose (p, ds) pairs the backward workspace holds at a time: on shapes whose planes
+        do not fit in LDS, as many as 128 MiB hold, in groups of equal size; 0 when one pair's do not fit"""
+        per_bh, cap = V * Himg * Wimg * V * P * 8, 128 << 20
+        if table(B, V, Himg, Wimg, D, P, storage16) != 0 or per_bh > cap:
+            return 0
+        g = min(B * H, cap // per_bh)
+        ngroups = (B * H + g - 1) // g
+        return (B * H + ngroups - 1) // ngroups
+
     def expect(B, V, H, Himg, Wimg, D, P, storage16):
         rows, NC = B * V * H * Himg * Wimg, (Himg + 1) * (Wimg + 1)
-        handed = table(B, V, Himg, Wimg, D, P, storage16) == 0 and V * H * Himg * Wimg * V * P * 8 < 1 << 32
+        handed = handed_group(B, V, H, Himg, Wimg, D, P, storage16) > 0
         NC = NC * groups(V, H, Himg * Wimg, D, 2 if storage16 else 4, P, NC, handed)
         total = r256(rows * 8) + r256(B * V * NC * 4) + r256(B * V * (NC + 1) * 4) + r256(B * V * V * Himg * Wimg * P * 4)
         total += r256(B * V * V * Himg * Wimg * P * 8)          # positions beside the ids
@@ -70,15 +80,22 @@ def test_workspace_bytes():
         M = V * Himg * Wimg * P
         piece = (max(512, 4 * M // NC) + 63) // 64 * 64
         total += r256(B * V * (NC + M // piece + 1) * 16)
-        # (p, ds) per query*sample, dq kernel -> dk/dv kernel, on shapes whose planes do not fit in LDS
-        if table(B, V, Himg, Wimg, D, P, storage16) == 0 and V * H * Himg * Wimg * V * P * 8 < 1 << 32:
-            total += r256(rows * V * P * 8)
+        # (p, ds) per query*sample of one group of (batch, head) pairs, dq kernel -> dk/dv kernel
+        total += r256(handed_group(B, V, H, Himg, Wimg, D, P, storage16) * V * Himg * Wimg * V * P * 8)
         total += r256(2 * rows * D * 4) if storage16 else 0
         return total + table(B, V, Himg, Wimg, D, P, storage16)
 
     assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32, 0) == expect(2, 6, 8, 18, 18, 32, 32, False)
     assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64, 32, 0) == expect(2, 6, 8, 48, 48, 64, 32, True)
     assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F16, 1, 2, 1, 3, 5, 16, 7, 0) == expect(1, 2, 1, 3, 5, 16, 7, True)
+    # the pairs handed from dq to dk/dv never take more than 128 MiB, whatever the shape: 64x64, 64 samples per
+    # view, 4 views, D = 128 (16 (batch, head) pairs of 32 MiB each) goes in groups of 4 ...
+    assert handed_group(2, 4, 8, 64, 64, 128, 64, True) == 4
+    c5 = lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 2, 4, 8, 64, 64, 128, 64, 0)
+    assert c5 == expect(2, 4, 8, 64, 64, 128, 64, True) and c5 < 2 * 2 * 4 * 8 * 4096 * 128 * 4 + (256 << 20)
+    # ... and a shape where one pair's alone would take more (96x96, 6 views) hands nothing over
+    assert handed_group(1, 6, 2, 96, 96, 64, 64, True) == 0
+    assert lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_BF16, 1, 6, 2, 96, 96, 64, 64, 0) == expect(1, 6, 2, 96, 96, 64, 64, True)
     assert lib.dsdpa_fwd_workspace_bytes(_native.DSDPA_F32, 2, 6, 8, 18, 18, 32, 32) == table(2, 6, 18, 18, 32, 32, False) > 0
     assert lib.dsdpa_fwd_workspace_bytes(_native.DSDPA_F16, 1, 2, 1, 3, 5, 16, 7) == table(1, 2, 3, 5, 16, 7, True) > 0
     assert lib.dsdpa_fwd_workspace_bytes(_native.DSDPA_BF16, 2, 6, 8, 48, 48, 64, 32) == 0      # planes too large for LDS
