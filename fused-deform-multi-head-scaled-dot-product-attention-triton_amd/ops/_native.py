@@ -81,13 +81,19 @@ def strides_arg(q, k, v):
     """The `strides` argument of the entry points for q, k, v given as (B, V, H, L, D) tensors: None when all three
     are contiguous, else a ctypes array of q's and k/v's element strides over (batch, view, head, pixel), or
     False when the kernels cannot read the tensors in place (the head dimension is not contiguous, k and v are
-    laid out differently, or a row start is not 16-byte aligned): the caller then copies."""
+    laid out differently, a row start is not 16-byte aligned, or the views and pixels of one (batch, head) lie
+    more than 2^30 elements apart): the caller then copies."""
     if q.is_contiguous() and k.is_contiguous() and v.is_contiguous():
         return None
     align = 16 // q.element_size()
+    V, L, D = q.shape[1], q.shape[3], q.shape[4]
     for t in (q, k, v):
         st = t.stride()
         if st[4] != 1 or t.data_ptr() % 16 or any(x % align or x < 0 for x in st[:4]) or st[3] < t.shape[4]:
+            return False
+        # the kernels address a pixel of one (batch, head) as view*sv + pixel*sl in 32 bits: a layout that reaches
+        # farther (the library would refuse it with DSDPA_ERR_TOO_LARGE) is copied as well
+        if (V - 1) * st[1] + (L - 1) * st[3] + D > (1 << 30) or st[1] > (1 << 30):
             return False
     if k.stride() != v.stride():
         return False

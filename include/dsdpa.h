@@ -149,8 +149,12 @@ enum { DSDPA_FLAG_DETERMINISTIC = 1, DSDPA_FLAG_COORDS_GRAD = 2, DSDPA_FLAG_SING
  * offsets; it depends on coords only and is shared by all heads) and, for bf16/fp16, the fp32 dk/dv
  * accumulators that are rounded to the storage type at the end (fp32: dk and dv
  * are themselves the accumulators), and the same per-coordinate table as the forward's -- or, on shapes
- * whose K/V planes do not fit in LDS, 8 bytes per (query row, sample) in which the dq kernel leaves the
- * softmax weight and its gradient for the dk/dv kernel. Without
+ * whose K/V planes do not fit in LDS, a buffer in which the dq kernel leaves the softmax weight and its
+ * gradient (8 bytes per (query row, sample)) for the dk/dv kernel: the backward runs in groups of (batch,
+ * head) pairs and the buffer holds one group's, at most 128 MiB whatever the shape. The workspace is therefore
+ * O(N) + O(coords) + a constant: the reference's own temporaries (dk32, dv32, delta, ops/triton.py:427-432)
+ * plus 12 to 32 bytes per coordinate pair, plus at most 128 MiB; nothing in it grows with (query rows) x
+ * (samples) or with samples x D. Without
  * DSDPA_FLAG_DETERMINISTIC the accumulation order into dk/dv is not deterministic (float atomics,
  * as in the reference, ops/triton.py:345-360).
  */

@@ -36,12 +36,22 @@ def _both(lib, shape, dtype, seed):
         q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out_a.data_ptr(), lse_a.data_ptr(), ws.data_ptr(),
         B, V, H, Himg, Wimg, D, P, 0.25, None, st))
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
-    _native.check(lib.dsdpa_fwd_noalloc(
-        CODE[dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out_b.data_ptr(), lse_b.data_ptr(),
-        B, V, H, Himg, Wimg, D, P, 0.25, None, st))
+
+    def call():
+        _native.check(lib.dsdpa_fwd_noalloc(
+            CODE[dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), out_b.data_ptr(), lse_b.data_ptr(),
+            B, V, H, Himg, Wimg, D, P, 0.25, None, st))
+        torch.cuda.synchronize()
+
+    # The first call on a device may load the code object and looks the built-in buffer's address up; from the
+    # second on, a call must leave the DRIVER's free memory as it found it (torch's own counters would not see a
+    # hipMalloc made inside the library) -- and torch's allocator must not have been asked for anything either.
+    call()
+    out_b.fill_(float("nan")), lse_b.fill_(float("nan"))
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    free_before, reserved_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
+    call()
+    assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_reserved() == reserved_before
     return need, (out_a, lse_a), (out_b, lse_b)
 
 
