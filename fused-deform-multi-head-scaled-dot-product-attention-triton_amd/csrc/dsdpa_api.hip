@@ -49,19 +49,19 @@ extern "C" {
 int dsdpa_fwd_f32(const float *q, const float *k, const float *v, const float *coords, float *out, float *lse, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides, void *stream)
 {
-    return fwd_impl<F32>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
+    return fwd_impl<F32>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream, true);
 }
 
 int dsdpa_fwd_bf16(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides, void *stream)
 {
-    return fwd_impl<BF16>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
+    return fwd_impl<BF16>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream, true);
 }
 
 int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse, void *workspace,
                   int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale, const long long *strides, void *stream)
 {
-    return fwd_impl<F16>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
+    return fwd_impl<F16>(q, k, v, coords, out, lse, workspace, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream, true);
 }
 
 int dsdpa_bwd_f32(const float *q, const float *k, const float *v, const float *coords, const float *out,
@@ -95,17 +95,22 @@ int dsdpa_fwd_noalloc(int dtype, const void *q, const void *k, const void *v, co
     if (dtype != DSDPA_F32 && dtype != DSDPA_BF16 && dtype != DSDPA_F16) return DSDPA_ERR_DTYPE;
     if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || P < 1) return DSDPA_ERR_BAD_SHAPE;
     if (!(D == 16 || D == 32 || D == 64 || D == 128 || D == 256)) return DSDPA_ERR_HEAD_DIM;
-    const size_t need = desc_layout(B, V, Himg, Wimg, D, P, dtype != DSDPA_F32 ? 2 : 4).bytes;
+    const size_t esize = dtype != DSDPA_F32 ? 2 : 4;
+    size_t need = desc_layout(B, V, Himg, Wimg, D, P, esize).bytes;
     if (need > (size_t)DSDPA_NOALLOC_SCRATCH_BYTES) return DSDPA_ERR_SCRATCH;
+    // (the dense-box forward's transposed V is an optional speed-up: taken when it fits, never a reason to refuse)
+    const size_t dense_need = dense_layout(B, V, H, Himg, Wimg, D, P, esize).bytes;
+    const bool dense_ok = dense_need != 0 && dense_need <= (size_t)DSDPA_NOALLOC_SCRATCH_BYTES;
+    if (dense_ok) need = dense_need;
     void *ws = nullptr;
     if (need) {
         ws = scratch_on_current_device();
         if (!ws) return DSDPA_ERR_HIP;
     }
     switch (dtype) {
-    case DSDPA_F32: return fwd_impl<F32>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
-    case DSDPA_BF16: return fwd_impl<BF16>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
-    default: return fwd_impl<F16>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream);
+    case DSDPA_F32: return fwd_impl<F32>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream, dense_ok);
+    case DSDPA_BF16: return fwd_impl<BF16>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream, dense_ok);
+    default: return fwd_impl<F16>(q, k, v, coords, out, lse, ws, B, V, H, Himg, Wimg, D, P, sm_scale, strides, stream, dense_ok);
     }
 }
 
@@ -113,7 +118,8 @@ size_t dsdpa_fwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int W
 {
     if (dtype != DSDPA_F32 && dtype != DSDPA_BF16 && dtype != DSDPA_F16) return 0;
     if (B < 1 || V < 1 || H < 1 || Himg < 1 || Wimg < 1 || D < 1 || P < 1) return 0;
-    return desc_layout(B, V, Himg, Wimg, D, P, dtype != DSDPA_F32 ? 2 : 4).bytes;
+    const size_t esize = dtype != DSDPA_F32 ? 2 : 4;
+    return desc_layout(B, V, Himg, Wimg, D, P, esize).bytes + dense_layout(B, V, H, Himg, Wimg, D, P, esize).bytes;
 }
 
 size_t dsdpa_bwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P, unsigned flags)

@@ -3,7 +3,7 @@
 
 namespace dsdpa {
 template int fwd_impl<F32>(const void *, const void *, const void *, const float *, void *, float *, void *, int, int, int, int,
-                           int, int, int, float, const long long *, void *);
+                           int, int, int, float, const long long *, void *, bool);
 template int bwd_impl<F32>(const void *, const void *, const void *, const float *, const void *, const float *,
                            const void *, void *, void *, void *, float *, void *, int, int, int, int, int, int, int, float,
                            const long long *, unsigned, void *);

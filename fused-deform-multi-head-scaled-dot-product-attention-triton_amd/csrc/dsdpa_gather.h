@@ -292,7 +292,8 @@ __device__ __forceinline__ void accumulate_taps(const char *__restrict__ base, c
 template <typename S, int D, int DC, bool WIN>
 __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void fwd_gather_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
-    const float *__restrict__ coords_, void *__restrict__ out_, float *__restrict__ lse_, Dims dm)
+    const float *__restrict__ coords_, void *__restrict__ out_, float *__restrict__ lse_,
+    const unsigned char *__restrict__ todo_, int ntl, Dims dm)
 {
     constexpr int G = D / DC;        // lanes per sample
     constexpr int NS = kWave / G;    // samples in flight per wave
@@ -311,6 +312,12 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const int work = xcd_logical_block(blockIdx.x, gridDim.x) * kGatherWaves + wave;
     if (work >= dm.rows) return;
+    // todo_ (may be null): one flag per tile of 16 consecutive pixels of a (b, h, s1), ntl tiles each; a tile
+    // whose flag is 0 has been worked on by fwd_dense_kernel
+    if (todo_) {
+        const int bhs = work / dm.L, l = work - bhs * dm.L;
+        if (!todo_[(size_t)bhs * ntl + (l >> 4)]) return;
+    }
     const RowCtx rc = decode_row(work, dm, D);
     const int g = lane % G, slot = lane / G, lane_elem = g * DC;
     const unsigned lane_byte = (unsigned)lane_elem * S::kBytes;

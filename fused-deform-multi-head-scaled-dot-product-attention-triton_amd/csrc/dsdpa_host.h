@@ -157,7 +157,23 @@ inline DescLayout desc_layout(size_t B, size_t V, size_t Himg, size_t Wimg, size
     return d;
 }
 
-// Forward workspace: the descriptor table alone.
+// Dense-box forward (fwd_dense_kernel): for 16-bit storage and D = 64 or 128 on shapes whose planes do not fit in LDS, with
+// at least a chunk's worth of samples per view. Its workspace is one flag per tile of 16 queries, telling which
+// tiles are left to the gather kernel. bytes = 0: the shape does not take that path.
+struct DenseLayout { size_t todo, bytes; int ntl; };
+inline DenseLayout dense_layout(size_t B, size_t V, size_t H, size_t Himg, size_t Wimg, size_t D, size_t P, size_t esize)
+{
+    DenseLayout d{0, 0, 0};
+    const size_t L = Himg * Wimg, chunks = V * ((P + 63) / 64);
+    if (esize != 2 || (D != 64 && D != 128) || P < 64 || chunks > 32 || Himg >= 65536 || Wimg >= 65536 || plane_path_fits(L, D, esize))
+        return d;
+    d.ntl = (int)((L + 15) / 16);
+    d.todo = 0;
+    d.bytes = round256(B * H * V * (size_t)d.ntl);
+    return d;
+}
+
+// Forward workspace: the descriptor table, or the dense-box forward's flags (never both).
 // Backward workspace, every segment rounded up to 256 bytes:
 //   delta    rows floats                     dout.out per query row
 //   counters B*V*NC u32                      per (batch, key view) cell counts, then fill cursors
@@ -289,10 +305,11 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
 // instantiated in its own translation unit (dsdpa_f32.hip, dsdpa_bf16.hip, dsdpa_f16.hip) so that the
 // three compile in parallel.
 // `strides`: null (everything contiguous) or the 8 element strides of q and of k/v over (batch, view, head, pixel).
+// dense_ok: the workspace has room for dense_layout() (false: the gather kernels alone do those shapes).
 template <typename S>
 int fwd_impl(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
              void *workspace, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale,
-             const long long *strides, void *stream);
+             const long long *strides, void *stream, bool dense_ok = true);
 template <typename S>
 int bwd_impl(const void *q, const void *k, const void *v, const float *coords, const void *out,
              const float *lse, const void *dout, void *dq, void *dk, void *dv, float *dcoords, void *workspace,

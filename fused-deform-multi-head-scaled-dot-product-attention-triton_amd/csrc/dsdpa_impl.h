@@ -7,6 +7,7 @@
 #include "dsdpa_tile.h"
 #include "dsdpa_cell.h"
 #include "dsdpa_plane.h"
+#include "dsdpa_dense.h"
 
 namespace dsdpa {
 
@@ -143,9 +144,10 @@ template <typename S, int D> struct Chunk {
 // 64 consecutive samples (several views each) keep the lanes busy and always gather.
 static inline bool gather_window_mode(int P) { return P >= kWave; }
 
+// todo (may be null): flags of the tiles of 16 queries that fwd_dense_kernel left undone; rows of the other tiles are skipped
 template <typename S, int D>
 int launch_fwd_gather(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
-                      const Dims &dm, hipStream_t st)
+                      const unsigned char *todo, int ntl, const Dims &dm, hipStream_t st)
 {
     constexpr int DC = Chunk<S, D>::value;
     const int blocks = (dm.rows + kGatherWaves - 1) / kGatherWaves;
@@ -153,12 +155,33 @@ int launch_fwd_gather(const void *q, const void *k, const void *v, const float *
     if (gather_window_mode(dm.P))
         DSDPA_LAUNCH((fwd_gather_kernel<S, D, DC, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
-                           q, k, v, coords, out, lse, dm);
+                           q, k, v, coords, out, lse, todo, ntl, dm);
     else
         DSDPA_LAUNCH((fwd_gather_kernel<S, D, DC, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
-                           q, k, v, coords, out, lse, dm);
+                           q, k, v, coords, out, lse, todo, ntl, dm);
     return check_launch();
+}
+
+// The dense-box forward (16-bit storage): one workgroup per tile of 16 queries; the tiles it declines are flagged in
+// the workspace for the gather kernel that the caller launches behind it.
+template <typename S, int D>
+int launch_fwd_dense(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+                     char *ws, const DenseLayout &dn, const Dims &dm, hipStream_t st)
+{
+    if constexpr (S::kBytes != 2 || (D != 64 && D != 128)) {
+        return DSDPA_ERR_UNSUPPORTED;
+    } else {
+        const long long tiles = (long long)dm.B * dm.H * dm.V * dn.ntl;
+        if (tiles > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+        auto kern = fwd_dense_kernel<S, D>;
+        static std::atomic<unsigned long long> lds_set{0};
+        if (int rc = allow_full_lds(kern, lds_set)) return rc;
+        ScopedKernelTimer timer(0, st);
+        DSDPA_LAUNCH(kern, dim3((unsigned)tiles), dim3(kDenseThreads), (size_t)dense_lds_bytes<D>(), st, timer.start(), timer.stop(),
+                     q, k, v, coords, out, lse, (unsigned char *)(ws + dn.todo), dm, dn.ntl);
+        return check_launch();
+    }
 }
 
 template <typename S, int D>
@@ -336,7 +359,7 @@ int launch_bwd_dq_plane(const void *q, const void *k, const void *v, const float
 template <typename S>
 int fwd_impl(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
              void *workspace, int B, int V, int H, int Himg, int Wimg, int D, int P, float sm_scale,
-             const long long *strides, void *stream)
+             const long long *strides, void *stream, bool dense_ok)
 {
     if (!q || !k || !v || !coords || !out || !lse) return DSDPA_ERR_NULL_POINTER;
     Dims dm;
@@ -346,18 +369,23 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
     if ((rc = apply_strides(strides, D, S::kBytes, &dm, &contiguous)) != DSDPA_OK) return rc;
     hipStream_t st = (hipStream_t)stream;
     const DescLayout dl = desc_layout(B, V, Himg, Wimg, D, P, S::kBytes);
-    if (dl.bytes && !workspace) return DSDPA_ERR_NULL_POINTER;
+    const DenseLayout dn = dense_ok ? dense_layout(B, V, H, Himg, Wimg, D, P, S::kBytes) : DenseLayout{0, 0, 0};
+    if ((dl.bytes || dn.bytes) && !workspace) return DSDPA_ERR_NULL_POINTER;
     const int path = g_path.load();
     const bool staged = path != DSDPA_PATH_GATHER && dl.bytes != 0 &&
                         (path == DSDPA_PATH_LDS || !few_samples_prefer_gather(V, P));
+    // (DSDPA_PATH_GATHER keeps its meaning: every tap, or every pixel of a query's window, read by the gather kernel)
+    const bool dense = path == DSDPA_PATH_AUTO && dn.bytes != 0;
     char *ws = (char *)workspace;
     if (staged && (rc = launch_plane_descriptors(coords, dm, ws, dl, false, ZeroJob{}, 4, st)) != DSDPA_OK) return rc;
     const float4 *desc_w = (const float4 *)(ws + dl.w);
     const uint32_t *desc_e = (const uint32_t *)(ws + dl.e);
+    const unsigned char *todo = dense ? (const unsigned char *)(ws + dn.todo) : nullptr;
 #define DSDPA_FWD_CASE(DD)                                                                        \
     case DD:                                                                                      \
-        return staged ? launch_fwd_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dm, st)        \
-                      : launch_fwd_gather<S, DD>(q, k, v, coords, out, lse, dm, st);
+        if (staged) return launch_fwd_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dm, st);    \
+        if (dense && (rc = launch_fwd_dense<S, DD>(q, k, v, coords, out, lse, ws, dn, dm, st)) != DSDPA_OK) return rc; \
+        return launch_fwd_gather<S, DD>(q, k, v, coords, out, lse, todo, dn.ntl, dm, st);
     switch (D) {
         DSDPA_FWD_CASE(16)
         DSDPA_FWD_CASE(32)
