@@ -38,7 +38,8 @@
 // A tile takes this path only if every one of its chunks has a box of at most kDensePix pixels: the first chunk
 // with a larger one ends the work on the tile (nothing of it has been written by then), which is marked in `todo`
 // and left to fwd_gather_kernel; that kernel skips the tiles done here. Pixels of a box that no tap
-// touches take part in the second product with coefficient 0: V must be finite there.
+// touches take part in the second product with coefficient 0; a tile whose sums come out non-finite (an infinity
+// or NaN of V at such a pixel would do that) is left to the gather kernel too.
 #pragma once
 #include "dsdpa_common.h"
 
@@ -434,9 +435,19 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
     }
 
     // ---- out = O / l, lse = m + log2 l
-    if (tid == 0) todo_[tile] = 0;                 // done here
+    // Pixels of a box that no tap touches took part in the second product with coefficient 0: should V hold an
+    // infinity or a NaN there, the sums are NaN where the operator's result is finite. Such a tile is left to the
+    // gather kernel, which reads touched pixels only.
+    bool bad = false;
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt) {
+        const float sum = (oacc[nt][0] + oacc[nt][1]) + (oacc[nt][2] + oacc[nt][3]);
+        bad = bad || !(fabsf(sum) <= 3.0e38f);
+    }
+    if (tid == 0) boxw[0] = 0u;
     xm[sub * 16 + qi] = l_run;
     __syncthreads();
+    if (bad) boxw[0] = 1u;
     float l_tot = 0.f;
 #pragma unroll
     for (int s = 0; s < 16; ++s) l_tot += xm[s * 16 + qi];
@@ -458,6 +469,9 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
             O_s[(4 * g + 3) * OP + col] = oacc[nt][3] * inv.w;
         }
         __syncthreads();
+        const bool redo = boxw[0] != 0u;
+        if (tid == 0) todo_[tile] = redo ? 1 : 0;
+        if (redo) return;
         // 16 rows of D elements, 8 elements (16 bytes of output) a thread and pass
         for (int idx = tid; idx < kDenseQ * (D / 8); idx += kDenseThreads) {
             const int r = idx / (D / 8), c8 = idx - r * (D / 8);

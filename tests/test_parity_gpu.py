@@ -158,6 +158,46 @@ def test_clustered_windows_vs_oracle(case, dtype, path):
     assert rel(dv, rdv) < TOL_BWD[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_dense_box_forward_mixed_tiles_and_untouched_pixels(dtype):
+    """16-bit storage, at least 64 samples per view, planes too large for LDS: tiles of 16 queries whose taps fall
+    into a small box of the key view are worked on as dense products over the box (matrix instructions), the other
+    tiles by the gather kernel. Here (1) every other tile of 16 queries has its samples spread over the whole image
+    (no box), so that both kernels write parts of one output; (2) the clustered queries look at two spots with a
+    gap between them: the box spans the gap, whose pixels no tap touches -- and V holds NaN and infinity there,
+    which must not reach the output (the reference reads touched pixels only, ops/torch.py:14-15)."""
+    say(f"[case] dense box forward, mixed tiles, NaN in untouched pixels {dtype}")
+    g = torch.Generator().manual_seed(81)
+    B, V, H, Himg, Wimg, D, P = 1, 2, 2, 24, 24, 64, 64
+    L = Himg * Wimg
+    q, k, v = (torch.randn(B, V, H, L, D, generator=g).to(dtype) for _ in range(3))
+    spot = torch.where(torch.rand(B, V, L, V, P, 1, generator=g) < 0.5, 0.3, 0.7)          # one of the two spots per sample
+    c = spot + 0.012 * torch.randn(B, V, L, V, P, 2, generator=g)
+    wide = ((torch.arange(L) // 16) % 2 == 1).view(1, 1, L, 1, 1, 1)                       # every other tile of 16 queries
+    c = torch.where(wide, torch.rand(B, V, L, V, P, 2, generator=g), c)
+    # the image centre lies between the spots: 0.5 * 23 = 11.5 -> pixels (11..12, 11..12); the spots' taps stay
+    # within +-0.06 * 23 = 1.4 pixels of 6.9 and 16.1
+    tight = c[:, :, ~wide.view(-1)]
+    assert ((tight - 0.3).abs().amax(-1).clamp(max=1) < 0.07).logical_or((tight - 0.7).abs().amax(-1) < 0.07).all()
+    v_bad = v.clone()
+    for (yy, xx, val) in ((11, 11, float("nan")), (12, 12, float("inf")), (11, 12, float("-inf"))):
+        v_bad[:, :, :, yy * Wimg + xx, :] = val
+    do = torch.randn(B, V, H, L, D, generator=g).to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    # queries of the spread tiles may well touch the centre pixels: compare the clustered rows only for v_bad, and
+    # everything for the clean v
+    out, dq, dk, dv = run_op(q, k, v, c, do, Wimg, Himg, scale)
+    ro, _, rdq, rdk, rdv = oracle_all(q, k, v, c, do, Wimg, Himg, scale)
+    assert rel(out, ro) < TOL_FWD[dtype]
+    assert rel(dq, rdq) < TOL_BWD[dtype] and rel(dk, rdk) < TOL_BWD[dtype] and rel(dv, rdv) < TOL_BWD[dtype]
+    with torch.no_grad():
+        out_bad = deform_sdpa_triton(q.cuda(), k.cuda(), v_bad.cuda(), c.cuda(), Wimg, Himg, scale)
+    torch.cuda.synchronize()
+    rows = ~wide.view(-1)
+    assert torch.isfinite(out_bad[:, :, :, rows.cuda()].float()).all()
+    assert rel(out_bad[:, :, :, rows.cuda()], ro[:, :, :, rows.numpy()]) < TOL_FWD[dtype]
+
+
 GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
 
 
