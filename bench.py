@@ -19,7 +19,8 @@ The headline workload is C5, the largest of the five named shapes. The other fou
 are measured in the same run (a shorter leg each; --only skips them) and reported
 as flat, short keys inside "config": c1_ms (fwd+bwd step), c1_gqs (G query.samples/s),
 c1_frac (fwd+bwd compulsory bytes / step time / 8 TB/s), c1_kfrac (the same for the
-workload's longest kernel on that kernel's own bytes and duration).
+workload's longest kernel on that kernel's own bytes and duration); cg_ms is the headline
+workload's step with the optional gradient of the coordinates switched on.
 Per-workload details go to stderr and, with --details FILE, as JSON into that file.
 """
 import argparse
@@ -138,6 +139,26 @@ def measure_gpu(wl, steps, warmup, extras=True):
     finally:
         op_module.SINGLE_STREAM = False
     res["kernels_single_stream_ms"] = {name: v["ms"] for name, v in collect(5).items()}
+
+    # the same step with the gradient of the coordinates as well (the operator's optional eighth argument; the
+    # reference's fused operator has none, its eager one gets it through grid_sample)
+    cg = coords.clone().requires_grad_(True)
+
+    def step_cg():
+        q.grad = k.grad = v.grad = cg.grad = None
+        deform_sdpa_triton(q, k, v, cg, W, Hh, scale, True).backward(dout)
+
+    for _ in range(3):
+        step_cg()
+    torch.cuda.synchronize()
+    n_cg = max(5, steps // 2)
+    t0 = time.perf_counter()
+    for _ in range(n_cg):
+        step_cg()
+    torch.cuda.synchronize()
+    res["coords_grad_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / n_cg
+    cg.grad = None
+    del cg
 
     torch.cuda.reset_peak_memory_stats()
     base = torch.cuda.memory_allocated()
@@ -309,7 +330,8 @@ def main():
               "query_samples_per_step": qs,
               "fwd_only_ms": round(g["fwd_only_ms"], 5),
               "step_frac": round(details["fwd_bwd_frac_of_roofline_on_step_time"], 5),
-              "peak_extra_bytes": g["peak_extra_bytes"]}
+              "peak_extra_bytes": g["peak_extra_bytes"],
+              "cg_ms": round(g["coords_grad_ms_per_step"], 4)}      # fwd+bwd step that also returns d loss / d coords
     for name, v in g["kernels"].items():
         config["k_" + name + "_ms"] = round(v["ms"], 5)
     for name, v in g["kernels_single_stream_ms"].items():

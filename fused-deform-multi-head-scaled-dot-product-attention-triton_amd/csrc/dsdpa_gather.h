@@ -706,11 +706,13 @@ __global__ __launch_bounds__(kGatherWaves *kWave) void bwd_gather_kernel(
 // elements, combines them with the (slot-uniform) ds, p and tap derivatives and only the two results
 // are reduced over the slot. The H heads share the coordinates: float atomics into dcoords (zeroed by
 // the caller of the kernel).
-// WIN (never together with CG): chunks per key view and the window mode, as in the forward: q.K and dout.V
-// per pixel of the window, each sample's logit and dp blended from those scalars, ds times the bilinear weights
-// scattered into one coefficient per pixel, dq += coefficient * K[pixel] per pixel.
+// WIN: chunks per key view and the window mode, as in the forward: q.K and dout.V per pixel of the window, each
+// sample's logit and dp blended from those scalars, ds times the bilinear weights scattered into one coefficient
+// per pixel, dq += coefficient * K[pixel] per pixel. With CG the per-pixel scalars are all the coordinate gradient
+// needs as well: a sample's g_t is sm_scale*ds*(q.K) + p*(dout.V) of its tap's pixel, four table reads it has
+// made already.
 template <typename S, int D, int DC, bool CG, bool WIN>
-__global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void bwd_dq_gather_kernel(
+__global__ __launch_bounds__(kGatherWaves *kWave, (WIN && !CG && DC <= 8) ? 4 : 1) void bwd_dq_gather_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const void *__restrict__ out_, const float *__restrict__ lse_,
     const void *__restrict__ dout_, void *__restrict__ dq_, float2 *__restrict__ stats_,
@@ -724,8 +726,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     __shared__ uint4 s_e[kGatherWaves][kWave];
     __shared__ float4 s_gx[CG ? kGatherWaves : 1][CG ? kWave : 1];
     __shared__ float4 s_gy[CG ? kGatherWaves : 1][CG ? kWave : 1];
-    __shared__ float2 s_hand[CG ? 1 : kGatherWaves][kWave];                      // (p, sm_scale * ds) of the chunk's samples
-    static_assert(!(CG && WIN), "the window mode has no coordinate gradient");
+    __shared__ float2 s_hand[kGatherWaves][kWave];                               // (p, sm_scale * ds) of the chunk's samples
     constexpr int kTab = WIN ? kGatherWaves : 1, kTabUnits = WIN ? kWinUnits : 1;
     __shared__ __attribute__((aligned(16))) float s_dotk[kTab][4 * kTabUnits + 4];    // window mode: q.K per pixel (+ the dummy entry)
     __shared__ __attribute__((aligned(16))) float s_dotv[kTab][4 * kTabUnits + 4];    // window mode: dout.V per pixel
@@ -746,16 +747,19 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     const char *vb = (const char *)v_ + rc.kv_base * S::kBytes;
     const float2 *coords = (const float2 *)coords_;
 
+    // 16-bit storage: packed pairs for the dot-product instructions -- in the window mode always, tap by tap only
+    // without the coordinate gradient (whose per-tap products take the widened rows)
+    constexpr bool kPackedWin = S::kBytes == 2 && WIN;
     constexpr bool kPacked = S::kBytes == 2 && !CG;
     float qf[DC], dof[DC], of[DC];
-    uint32_t dop[kPacked ? DC / 2 : 1], qp[kPacked && WIN ? DC / 2 : 1];
+    uint32_t dop[(kPacked || kPackedWin) ? DC / 2 : 1], qp[kPackedWin ? DC / 2 : 1];
     const size_t roff = (rc.row * D + lane_elem) * S::kBytes;
     const size_t q_roff = (rc.q_off + lane_elem) * S::kBytes;
     load_chunk<S, DC>((const char *)q_ + q_roff, qf);
     load_chunk<S, DC>((const char *)dout_ + roff, dof);
     load_chunk<S, DC>((const char *)out_ + roff, of);
-    if constexpr (kPacked) load_packed<S, DC>((const char *)dout_ + roff, dop);
-    if constexpr (kPacked && WIN) load_packed<S, DC>((const char *)q_ + q_roff, qp);
+    if constexpr (kPacked || kPackedWin) load_packed<S, DC>((const char *)dout_ + roff, dop);
+    if constexpr (kPackedWin) load_packed<S, DC>((const char *)q_ + q_roff, qp);
     float delta = 0.f;
 #pragma unroll
     for (int d = 0; d < DC; ++d) delta = fmaf(dof[d], of[d], delta);
@@ -763,7 +767,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
     const float qscale = dm.sm_scale * kLog2e;
     const float lse = lse_[rc.row];
     if (stats_ && lane == 0) stats_[rc.row] = make_float2(lse, delta);     // null: a launch of its own does it
-    // handed_ (may be null; never with CG): per sample, (p, sm_scale * ds) for the dk/dv kernel, which then need
+    // handed_ (may be null): per sample, (p, sm_scale * ds) for the dk/dv kernel, which then need
     // not recompute them from the taps: [pair (b, h) of this launch][s1][l][sample], i.e. in the order of the work
     // items of this launch and, inside a row, of its coordinates
     float2 *handed_row = handed_ ? handed_ + (size_t)(work - work0) * dm.N : nullptr;
@@ -801,7 +805,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
             const Window win = window_ok ? chunk_window(tp, counted, dm.Wimg, dm.Himg) : Window{0, 0, 0, 0};
             if (win.nunits > 0 && win.nunits <= kWinUnits && 8 * win.nunits <= 7 * cnt) {
                 const unsigned kRow = (unsigned)dm.kv_sl * S::kBytes;       // bytes between neighbouring pixels of K and V
-                constexpr bool kBlock = kPacked && G >= 4;
+                constexpr bool kBlock = kPackedWin && G >= 4;
                 float *tS = s_dotk[wave], *tT = s_dotv[wave];
                 double *tA = s_coef[wave];
                 uint4 *tC = s_blend[wave];
@@ -831,11 +835,26 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
                 // the samples, one per lane
                 const float w0 = live ? tp.w[0] : 0.f, w1 = live ? tp.w[1] : 0.f;
                 const float w2 = live ? tp.w[2] : 0.f, w3 = live ? tp.w[3] : 0.f;
-                const float dot = fmaf(w0, tS[te.x], fmaf(w1, tS[te.y], fmaf(w2, tS[te.z], w3 * tS[te.w])));
-                const float dp = fmaf(w0, tT[te.x], fmaf(w1, tT[te.y], fmaf(w2, tT[te.z], w3 * tT[te.w])));
+                const float sk0 = tS[te.x], sk1 = tS[te.y], sk2 = tS[te.z], sk3 = tS[te.w];
+                const float sv0 = tT[te.x], sv1 = tT[te.y], sv2 = tT[te.z], sv3 = tT[te.w];
+                const float dot = fmaf(w0, sk0, fmaf(w1, sk1, fmaf(w2, sk2, w3 * sk3)));
+                const float dp = fmaf(w0, sv0, fmaf(w1, sv1, fmaf(w2, sv2, w3 * sv3)));
                 const float p = live ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
                 const float ds = p * (dp - delta);
                 if (handed_row && live) handed_row[nc] = make_float2(p, ds * dm.sm_scale);
+                if constexpr (CG) {
+                    // one sample per lane: the tap derivatives (zero for a tap outside the image, and for a dead
+                    // lane through p = ds = 0) times g_t of the four pixels
+                    const TapGrads tg = make_tap_grads(xy0.x, xy0.y, dm.Wimg, dm.Himg);
+                    const float a = ds * dm.sm_scale;
+                    const float g0 = fmaf(a, sk0, p * sv0), g1 = fmaf(a, sk1, p * sv1);
+                    const float g2 = fmaf(a, sk2, p * sv2), g3 = fmaf(a, sk3, p * sv3);
+                    if (live) {
+                        float *dst = dcoords_ + 2 * (rc.crow + (size_t)nc);
+                        atomicAdd(dst, fmaf(tg.gx[0], g0, fmaf(tg.gx[1], g1, fmaf(tg.gx[2], g2, tg.gx[3] * g3))));
+                        atomicAdd(dst + 1, fmaf(tg.gy[0], g0, fmaf(tg.gy[1], g1, fmaf(tg.gy[2], g2, tg.gy[3] * g3))));
+                    }
+                }
                 atomicAdd(&tA[te.x], (double)(ds * w0));
                 atomicAdd(&tA[te.y], (double)(ds * w1));
                 atomicAdd(&tA[te.z], (double)(ds * w2));
@@ -942,6 +961,7 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
                     dp = group_sum<G>(dp);
                     const float p = (j < cnt) ? __builtin_amdgcn_exp2f(dot * qscale - lse) : 0.f;
                     const float ds = p * (dp - delta);
+                    s_hand[wave][j] = make_float2(p, ds * dm.sm_scale);          // (all lanes of the slot: same value, same place)
 #pragma unroll
                     for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
                     const float4 ax = s_gx[wave][j], ay = s_gy[wave][j];
@@ -980,14 +1000,12 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && DC <= 8) ? 4 : 1) void
                 for (int d = 0; d < DC; ++d) dqa[d] = fmaf(ds, kk[d], dqa[d]);
             }
         }
-        if constexpr (!CG) {
-            // the chunk's pairs, one sample per lane, in one coalesced store (plain stores and loads: streaming
-            // ones keep the pairs out of L2, where the dk/dv kernel finds them: 2.44 -> 2.64 ms at 64x64, D = 128)
-            if (handed_row) {
-                wave_lds_sync();
-                if (live) handed_row[c0 + lane] = s_hand[wave][lane];
-                wave_lds_sync();
-            }
+        // the chunk's pairs, one sample per lane, in one coalesced store (plain stores and loads: streaming
+        // ones keep the pairs out of L2, where the dk/dv kernel finds them: 2.44 -> 2.64 ms at 64x64, D = 128)
+        if (handed_row) {
+            wave_lds_sync();
+            if (live) handed_row[c0 + lane] = s_hand[wave][lane];
+            wave_lds_sync();
         }
     }
 #pragma unroll

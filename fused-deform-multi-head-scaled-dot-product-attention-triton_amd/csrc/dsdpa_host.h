@@ -245,13 +245,12 @@ inline int views_per_group(size_t V, size_t L, size_t D, size_t esize, size_t P,
 // group, the cell lists being shared by all heads -- and the buffer holds one group's pairs: at most
 // kHandedCapBytes, which also stay in the memory-side cache between the two kernels. Returns the (batch, head)
 // pairs per group, 0 when nothing is handed over: shapes on the staged kernels (dq and dk/dv run side by side
-// there), the deterministic backward (its four colour launches recompute), the coordinate gradient (its dq
-// kernel does not write pairs), one pair's samples beyond the cap or beyond 32-bit byte offsets.
+// there), the deterministic backward (its four colour launches recompute), one pair's samples beyond the cap or
+// beyond 32-bit byte offsets.
 constexpr size_t kHandedCapBytes = (size_t)128 << 20;
-inline int handed_group(size_t B, size_t V, size_t H, size_t L, size_t D, size_t P, size_t esize, bool deterministic,
-                        bool coords_grad)
+inline int handed_group(size_t B, size_t V, size_t H, size_t L, size_t D, size_t P, size_t esize, bool deterministic)
 {
-    if (deterministic || coords_grad || plane_path_fits(L, D, esize)) return 0;
+    if (deterministic || plane_path_fits(L, D, esize)) return 0;
     const size_t per_bh = V * L * (V * P) * 8;
     if (per_bh >= ((size_t)1 << 32) || per_bh > kHandedCapBytes) return 0;
     size_t g = kHandedCapBytes / per_bh;
@@ -268,7 +267,7 @@ inline WorkspaceLayout workspace_layout(size_t B, size_t V, size_t H, size_t Him
     w.NC = (int)((Himg + 1) * (Wimg + 1));
     size_t off = 0;
     w.delta = off; off += round256(rows * 8);           // (lse, delta) per row
-    w.bh_group = handed_group(B, V, H, Himg * Wimg, D, P, storage16 ? 2 : 4, deterministic, coords_grad);
+    w.bh_group = handed_group(B, V, H, Himg * Wimg, D, P, storage16 ? 2 : 4, deterministic);
     const bool handed = w.bh_group > 0;
     w.vpg = views_per_group(V, Himg * Wimg, D, storage16 ? 2 : 4, P, (size_t)w.NC, handed);
     w.NK = w.NC * (int)((V + w.vpg - 1) / w.vpg);

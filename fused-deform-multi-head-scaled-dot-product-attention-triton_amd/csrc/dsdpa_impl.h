@@ -208,7 +208,11 @@ int launch_bwd_dq_gather(const void *q, const void *k, const void *v, const floa
     const int work0 = bh0 * dm.V * dm.L, work_end = (bh0 + nbh) * dm.V * dm.L;      // (at most dm.rows)
     const int blocks = (work_end - work0 + kGatherWaves - 1) / kGatherWaves;
     ScopedKernelTimer timer(2, st);
-    if (dcoords)
+    if (dcoords && gather_window_mode(dm.P))
+        DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, true, true>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
+                              timer.start(), timer.stop(),
+                           q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm, work0, work_end);
+    else if (dcoords)
         DSDPA_LAUNCH((bwd_dq_gather_kernel<S, D, DC, true, false>), dim3(blocks), dim3(kGatherWaves * kWave), 0, st,
                               timer.start(), timer.stop(),
                            q, k, v, coords, out, lse, dout, dq, stats, dcoords, handed, dm, work0, work_end);
@@ -589,9 +593,8 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     // (the reordered lists of the deterministic backward have no positions beside them: coordinates are read again)
     const float2 *frac = deterministic ? nullptr : (const float2 *)(ws + wl.frac);
     // (p, sm_scale * ds) per query*sample from the dq kernel to the dk/dv kernel, where the layout has room for it
-    // (shapes on the gather dq kernel, which then runs before dk/dv on the same stream); the dq kernel with the
-    // coordinate gradient does not write it
-    float2 *handed = (wl.handed_bytes && cell_binned && !dcoords) ? (float2 *)(ws + wl.handed) : nullptr;
+    // (shapes on the gather dq kernel, which then runs before dk/dv on the same stream)
+    float2 *handed = (wl.handed_bytes && cell_binned && !staged) ? (float2 *)(ws + wl.handed) : nullptr;
     // fp32 storage: dk and dv are their own accumulators; 16-bit: fp32 accumulators in the workspace
     float *dk_acc = S::kBytes == 4 ? (float *)dk : (float *)(ws + wl.acc);
     float *dv_acc = S::kBytes == 4 ? (float *)dv : dk_acc + n;
