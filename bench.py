@@ -272,6 +272,11 @@ def main():
     roofline = {
         "bound": "hbm", "kernel": dominant, "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": dom["frac"], "traffic": load_traffic(wl.name, dominant),
+        # A kernel may cover the workload in several launches (the backward of the larger shapes goes group by
+        # group of (batch, head) pairs; the forward may be a dense-box launch plus a gather launch for the tiles it
+        # declines): bytes, traffic and kernel_ms are then the sums over the launches of one step, so that
+        # achieved = bytes per launch / average launch duration all the same.
+        "launches_per_step": g["kernels"][dominant]["launches_per_step"],
         "algorithmic_bytes": dom["algorithmic_bytes"], "kernel_ms": dom["kernel_ms"],
         # the same kernel with the backward on one stream (in the timed region the backward's two sides run
         # on two streams and share the CUs where both leave room)

@@ -91,6 +91,17 @@ __device__ __forceinline__ uint2 lds_read_tr16(const unsigned char *p)
     return __builtin_bit_cast(uint2, r);
 }
 
+// Orders this wave's earlier LDS accesses before its later ones for the COMPILER only. The LDS serves the
+// instructions of one wave in the order they were issued, so a read that follows a write of the same wave in
+// program order sees it without waiting for the write to be acknowledged; what must not happen is the compiler
+// moving one across the other. (wave_lds_sync also waits for everything outstanding: a round trip per use.)
+__device__ __forceinline__ void wave_lds_order()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // Bounding box of the clamped tap pixels of a chunk, packed: lo = xmin | ymin << 16, hi = (0xffff - xmax) |
 // (0xffff - ymax) << 16 (so that both are minima), 0xffffffff: no sample of the chunk has a tap inside the image.
 struct DenseBox { int x0, y0, w, npix; };          // npix: w * h rounded up to 32; 0: the chunk does not fit
@@ -280,11 +291,11 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
                 for (int u = 0; u < kRingK; ++u) {
                     const int nb = nb0 + 4 * u;
                     if (nb < nblk) {
-                        wave_lds_sync();                   // (the reads of the previous block are done)
+                        wave_lds_order();                  // (behind the reads of the previous block)
 #pragma unroll
                         for (int r = 0; r < KS; ++r)
                             *reinterpret_cast<dsdpa_u32x4 *>(wstage + (r * (kWave / CH) + krow) * kPitchK + kpiece) = kr[u][r];
-                        wave_lds_sync();
+                        wave_lds_order();
                         DSDPA_DENSE_FETCH_K(u, nb + 4 * kRingK)               // (behind the last one: unused)
                         floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
                         const unsigned char *kfrag = wstage + n16 * kPitchK + g * 16;
@@ -400,7 +411,7 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
                 *reinterpret_cast<dsdpa_u32x4 *>(wstage + ((buf_) * 32 + r * (kWave / VCH) + vrow_l) * kPitchV + vpark) = vr[slot_][r];
 #pragma unroll
             for (int u = 0; u < kRingV; ++u) { DSDPA_DENSE_FETCH_V(u, u) }
-            wave_lds_sync();                       // (the last reads of K's staging are done)
+            wave_lds_order();                      // (behind the last reads of K's staging)
             DSDPA_DENSE_PARK_V(0, 0)
             DSDPA_DENSE_FETCH_V(0, kRingV)
             const int s16 = lane & 15;
@@ -412,7 +423,7 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
                     const int kb = kb0 + u;
                     if (kb < nkb) {
                         const int buf = kb & 1;
-                        wave_lds_sync();                   // (buffer `buf` is parked; the other one's reads are done)
+                        wave_lds_order();                  // (buffer `buf` is parked, the other one's reads are issued)
                         const unsigned char *prow = dense_lds + n16 * kP16 + (kb * 32 + 4 * g) * 2;
                         const uint2 a0 = *reinterpret_cast<const uint2 *>(prow), a1 = *reinterpret_cast<const uint2 *>(prow + 32);
                         const uint4 af = make_uint4(a0.x, a0.y, a1.x, a1.y);
