@@ -35,7 +35,7 @@
 // at most 64 of them per chunk; integer LDS atomics run at 11 lane-adds a clock and CU here, float ones at a
 // third of one), then rounded to the storage type, once per chunk and in place, for the matrix instruction.
 //
-// A tile takes this path only if every one of its chunks has a box of at most kDensePix pixels: the first chunk
+// A tile takes this path only if every one of its chunks has a box of at most DenseCfg::kPix pixels: the first chunk
 // with a larger one ends the work on the tile (nothing of it has been written by then), which is marked in `todo`
 // and left to fwd_gather_kernel; that kernel skips the tiles done here. Pixels of a box that no tap
 // touches take part in the second product with coefficient 0; a tile whose sums come out non-finite (an infinity
@@ -45,28 +45,38 @@
 
 namespace dsdpa {
 
-constexpr int kDenseQ = 16;                      // queries per tile (the M of the matrix instruction)
-constexpr int kDenseThreads = 256;               // four waves per tile
-constexpr int kDensePix = 704;                   // pixels of a box, at most (a multiple of 32)
-constexpr int kDensePitch = 708;                 // P: 32-bit words per query row; 4 mod 64, so that the 16 rows' 16-byte reads spread over all banks
-constexpr int kDenseSpBytes = kDenseQ * kDensePitch * 4;        // S [kDensePix][16] floats fits as well
-constexpr int kDenseMaxChunks = 32;              // chunks of a tile whose boxes are kept in LDS
-static_assert(kDensePix * kDenseQ * 4 <= kDenseSpBytes && kDensePitch >= kDensePix && kDensePitch % 64 == 4, "S and P share the block");
-
-// Staging, per wave: 16 pixel rows of K (row pitch D*2 + 16 bytes: 4 words mod 64, the 16 rows of a 16-byte read land
-// in different banks), or two buffers of 32 pixel rows of the wave's quarter of V's columns (D/4 elements; row pitch 8
-// words mod 64 in 8-bank units: the 8 rows that 32 lanes of a transposing read touch land in different windows).
-template <int D> struct DenseStage {
+// Geometry of the kernel for head dimension D and tiles of TQ queries (16 or 32: one or two row blocks of the
+// matrix instruction; four waves per row block). With two row blocks every staged row of K and V feeds two
+// matrix instructions instead of one -- LDS bandwidth, 128 bytes a clock and CU against the 256 that four SIMDs'
+// matrix units could take with one row block, is what bounds the products -- at twice the S / P block, which
+// leaves room for one workgroup of eight waves per CU: measured slower than two of four, so the launcher
+// instantiates 16.
+template <int D, int TQ> struct DenseCfg {
+    static_assert((D == 64 || D == 128) && (TQ == 16 || TQ == 32), "head dimension 64 or 128, one or two row blocks");
+    static constexpr int kWaves = TQ / 4;                        // 4 or 8
+    static constexpr int kThreads = kWaves * kWave;
+    static constexpr int kSubs = kThreads / TQ;                  // 16 groups of four samples per query and chunk
+    static constexpr int MT = TQ / 16;                           // row blocks
+    static constexpr int NTW = D / 16 / kWaves;                  // column blocks of the second product per wave
+    static_assert(NTW >= 1, "every wave has a column block");
+    // pixels of a box, at most (a multiple of 32), and P's row pitch in 32-bit words: 4 mod 64, so that the 16 rows'
+    // 16-byte reads spread over all banks; S [pixels][TQ] floats and P [TQ][pitch] words share the block
+    static constexpr int kPix = TQ == 16 ? 704 : 768;
+    static constexpr int kPitch = kPix + 4;
+    static constexpr int kSpBytes = TQ * kPitch * 4;
+    static_assert(kPitch % 64 == 4 && kPix * TQ * 4 <= kSpBytes, "S and P share the block");
+    // staging, per wave: 16 pixel rows of K (row pitch D*2 + 16 bytes: 4 words mod 64, the 16 rows of a 16-byte read
+    // land in different banks), or two buffers of 32 pixel rows of the wave's share of V's columns (NTW * 16
+    // elements; row pitch 8 words mod 64 in 8-bank units -- or the 32 bytes themselves: the 8 rows that 32 lanes of a
+    // transposing read touch land in different windows)
     static constexpr int kPitchK = D * 2 + 16;
-    static constexpr int kPitchV = D / 2 + (D > 64 ? 32 : 0);
-    static constexpr int kWaveBytes = (16 * kPitchK > 2 * 32 * kPitchV) ? 16 * kPitchK : 2 * 32 * kPitchV;
-    static constexpr int kBytes = 4 * kWaveBytes;
+    static constexpr int kPitchV = NTW * 32 + (NTW > 1 ? 32 : 0);
+    static constexpr int kWaveStage = (16 * kPitchK > 2 * 32 * kPitchV) ? 16 * kPitchK : 2 * 32 * kPitchV;
+    static constexpr int kStageBytes = kWaves * kWaveStage;
+    static constexpr int kXmBytes = kSubs * TQ * 4;              // per-query exchange: [sample groups][queries]
+    static constexpr int kXqBytes = TQ * 4 + 64;                 // per-query values for the lanes that hold rows of O; the waves' box parts
+    static constexpr int kLdsBytes = kSpBytes + kStageBytes + kXmBytes + kXqBytes + 64 + kPix * 4;
 };
-constexpr int kDenseXchBytes = 16 * 16 * 4 + 256;      // per-query exchange: [16 sample groups][16 queries], then 16 values for the rows of O
-template <int D> constexpr int dense_lds_bytes()
-{
-    return kDenseSpBytes + DenseStage<D>::kBytes + kDenseXchBytes + kDenseMaxChunks * 4 * 16 + kDensePix * 4;
-}
 
 typedef __bf16 dsdpa_bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 dsdpa_f16x8 __attribute__((ext_vector_type(8)));
@@ -106,7 +116,7 @@ __device__ __forceinline__ void wave_lds_order()
 // (0xffff - ymax) << 16 (so that both are minima), 0xffffffff: no sample of the chunk has a tap inside the image.
 struct DenseBox { int x0, y0, w, npix; };          // npix: w * h rounded up to 32; 0: the chunk does not fit
 
-__device__ __forceinline__ DenseBox dense_box_from(uint32_t lo, uint32_t hi)
+__device__ __forceinline__ DenseBox dense_box_from(uint32_t lo, uint32_t hi, int max_pix)
 {
     int xlo = 0, ylo = 0, xhi = 0, yhi = 0;
     if (lo != 0xffffffffu) {                   // else: any one pixel will do
@@ -120,7 +130,7 @@ __device__ __forceinline__ DenseBox dense_box_from(uint32_t lo, uint32_t hi)
     b.y0 = ylo;
     b.w = xhi - xlo + 1;
     const int n = b.w * (yhi - ylo + 1);
-    b.npix = n <= kDensePix ? (n + 31) & ~31 : 0;
+    b.npix = n <= max_pix ? (n + 31) & ~31 : 0;
     return b;
 }
 
@@ -146,43 +156,47 @@ __device__ __forceinline__ uint2 dense_pack_p(const uint4 &a)
     return make_uint2(w[0], w[1]);
 }
 
-template <typename S, int D>
-__global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
+template <typename S, int D, int TQ>
+__global__ __launch_bounds__((DenseCfg<D, TQ>::kThreads), 2) void fwd_dense_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, void *__restrict__ out_, float *__restrict__ lse_,
     unsigned char *__restrict__ todo_, Dims dm, int ntl)
 {
-    static_assert(S::kBytes == 2 && (D == 64 || D == 128), "16-bit storage; every wave takes a quarter of the columns in blocks of 16");
+    static_assert(S::kBytes == 2, "16-bit storage");
+    using C = DenseCfg<D, TQ>;
     constexpr int KS = D / 32;                 // steps of the first product (and 16-byte loads per lane for 16 rows of K)
-    constexpr int NTW = D / 64;                // column blocks of the second product per wave (and loads per lane for 32 rows of its quarter of V)
+    constexpr int MT = C::MT, NTW = C::NTW, kWaves = C::kWaves, kThreads = C::kThreads, kSubs = C::kSubs;
     constexpr int CH = D / 8;                  // 16-byte pieces of a row of K
-    constexpr int VCH = 2 * NTW;               // ... of a wave's quarter of a row of V
-    constexpr int kPitchK = DenseStage<D>::kPitchK, kPitchV = DenseStage<D>::kPitchV;
+    constexpr int VCH = 2 * NTW;               // ... of a wave's share of a row of V
+    constexpr int VLD = (32 * VCH + kWave - 1) / kWave;      // loads per lane for 32 rows of that share
+    constexpr int kPitchK = C::kPitchK, kPitchV = C::kPitchV, kPitch = C::kPitch;
     constexpr int kRingK = 3, kRingV = 6;      // blocks of K, steps of V whose rows are in flight
-    constexpr int kP16 = kDensePitch * 4;      // bytes between the rows of P, as 32-bit sums and as 16-bit values alike
+    constexpr int kP16 = kPitch * 4;           // bytes between the rows of P, as 32-bit sums and as 16-bit values alike
     constexpr float kFix = 16777216.0f;        // 2^24
     constexpr float kUnfix = S::kBf16 ? 0x1p-24f : 0x1p-9f;      // what dense_pack_p leaves of it
     extern __shared__ __attribute__((aligned(16))) unsigned char dense_lds[];
-    float *S_T = reinterpret_cast<float *>(dense_lds);                       // [pixel][16 queries]
-    unsigned *Pm = reinterpret_cast<unsigned *>(dense_lds);                  // [16 queries][kDensePitch]
-    float *xm = reinterpret_cast<float *>(dense_lds + kDenseSpBytes + DenseStage<D>::kBytes);   // [16 sample groups][16 queries]
-    float *xq = xm + 256;                                                    // 16 per-query values for the lanes that hold rows of O
-    uint32_t *boxw = reinterpret_cast<uint32_t *>(xq + 64);                  // [4 waves][lo, hi]: the waves' parts of the chunk's box
-    unsigned *offs = reinterpret_cast<unsigned *>(boxw) + kDenseMaxChunks * 16;     // byte offset of every pixel of the chunk's box
+    float *S_T = reinterpret_cast<float *>(dense_lds);                       // [pixel][TQ queries]
+    unsigned *Pm = reinterpret_cast<unsigned *>(dense_lds);                  // [TQ queries][kPitch]
+    float *xm = reinterpret_cast<float *>(dense_lds + C::kSpBytes + C::kStageBytes);   // [sample groups][TQ queries]
+    float *xq = xm + kSubs * TQ;                                             // TQ per-query values for the lanes that hold rows of O
+    uint32_t *boxw = reinterpret_cast<uint32_t *>(xq + TQ);                  // [waves][lo, hi]: the waves' parts of the chunk's box
+    unsigned *offs = boxw + 32;                                              // byte offset of every pixel of the chunk's box
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    unsigned char *wstage = dense_lds + kDenseSpBytes + wave * DenseStage<D>::kWaveBytes;      // this wave's staging
+    unsigned char *wstage = dense_lds + C::kSpBytes + wave * C::kWaveStage;  // this wave's staging
     const int tile = xcd_logical_block(blockIdx.x, gridDim.x);
-    // tiles in the order (b, h, s1, tile of 16 pixels)
+    // tiles in the order (b, h, s1, tile of TQ pixels)
     int t = tile / ntl;
-    const int l0 = (tile - t * ntl) * kDenseQ;
+    const int l0 = (tile - t * ntl) * TQ;
     const int s1 = t % dm.V;
     t /= dm.V;
     const int h = t % dm.H, b = t / dm.H;
-    const int nq = min(kDenseQ, dm.L - l0);
+    const int nq = min(TQ, dm.L - l0);
+    // (the flags for the gather kernel are kept per 16 queries, whatever TQ: (L + 15) / 16 of them per (b, h, s1))
+    const size_t flag0 = (size_t)(tile / ntl) * (size_t)((dm.L + 15) >> 4) + (size_t)(l0 >> 4);
     // samples: thread (qi, sub) takes the samples [4 sub, 4 sub + 4) of a chunk for query qi
-    const int qi = tid & 15, sub = tid >> 4;
+    const int qi = tid % TQ, sub = tid / TQ;
     const bool qlive = qi < nq;
     const int lq = l0 + min(qi, nq - 1);
     const float2 *crd_row = reinterpret_cast<const float2 *>(coords_) + (((size_t)b * dm.V + s1) * dm.L + lq) * (size_t)dm.N;
@@ -192,21 +206,24 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
     const int view_chunks = (dm.P + kWave - 1) / kWave;
     const int nchunks = dm.V * view_chunks;
 
-    // Q as the A operand: row = query n16, eight consecutive elements per step at 8 g
-    uint4 qf[KS];
-    {
-        const char *qrow = (const char *)q_ + dm.q_row(b, s1, h, l0 + min(n16, nq - 1)) * 2;
+    // Q as the A operand, per row block: row = query 16 mt + n16, eight consecutive elements per step at 8 g
+    uint4 qf[MT][KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const uint4 *>(qrow + ks * 64 + g * 16);
+    for (int mt = 0; mt < MT; ++mt) {
+        const char *qrow = (const char *)q_ + dm.q_row(b, s1, h, l0 + min(mt * 16 + n16, nq - 1)) * 2;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[mt][ks] = *reinterpret_cast<const uint4 *>(qrow + ks * 64 + g * 16);
     }
     const float qscale = dm.sm_scale * kLog2e;
     const char *kplane0 = (const char *)k_ + dm.kv_plane(b, 0, h) * 2;
     const char *vplane0 = (const char *)v_ + dm.kv_plane(b, 0, h) * 2;
     const unsigned row_bytes = (unsigned)dm.kv_sl * 2u;
 
-    floatx4 oacc[NTW];                             // rows: queries 4 g .. 4 g + 3; column: element (wave * NTW + nt) * 16 + n16
+    floatx4 oacc[MT][NTW];                         // rows: queries 16 mt + 4 g .. + 3; column: element (wave * NTW + nt) * 16 + n16
 #pragma unroll
-    for (int nt = 0; nt < NTW; ++nt) oacc[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NTW; ++nt) oacc[mt][nt] = floatx4{0.f, 0.f, 0.f, 0.f};
     float m_run = kNegBig, l_run = 0.f;            // of query qi; l_run: this thread's samples only
 
     for (int ci = 0; ci < nchunks; ++ci) {
@@ -246,16 +263,16 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
             }
             __syncthreads();
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
+            for (int w = 0; w < kWaves; ++w) {
                 const uint32_t l = boxw[w * 2], u = boxw[w * 2 + 1];
                 blo = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, blo), __builtin_bit_cast(u16x2, l)));
                 bhi = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, bhi), __builtin_bit_cast(u16x2, u)));
             }
         }
-        const DenseBox bxv = dense_box_from(__builtin_amdgcn_readfirstlane(blo), __builtin_amdgcn_readfirstlane(bhi));
+        const DenseBox bxv = dense_box_from(__builtin_amdgcn_readfirstlane(blo), __builtin_amdgcn_readfirstlane(bhi), C::kPix);
         if (bxv.npix == 0) {
             // this chunk's box is too large: nothing of the tile has been written yet; the gather kernel takes it
-            if (tid == 0) todo_[tile] = 1;
+            if (tid < TQ / 16 && l0 + 16 * tid < dm.L) todo_[flag0 + tid] = 1;
             return;
         }
         const int bx0 = bxv.x0, by0 = bxv.y0, bw = bxv.w, npix = bxv.npix;
@@ -263,7 +280,7 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
         const unsigned view_off = (unsigned)s2 * (unsigned)dm.kv_sv * 2u;
         // byte offset, in a (batch, head)'s K or V, of every box pixel (row-major over the box; the padding behind
         // the last pixel repeats pixels of the box)
-        for (int pidx = tid; pidx < npix; pidx += kDenseThreads) {
+        for (int pidx = tid; pidx < npix; pidx += kThreads) {
             const int ry = (int)(((float)pidx + 0.5f) * rbw);                 // pidx / bw, exact for these small numbers
             const int rx = pidx - ry * bw;
             const int y = min(by0 + ry, dm.Himg - 1), x = min(bx0 + rx, dm.Wimg - 1);
@@ -273,7 +290,7 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
 
         // ---- S = scale * Q . K^T: the waves take the blocks of 16 pixels in turn. A block's rows come in with
         // neighbouring lanes on neighbouring bytes (lane -> piece lane % CH of row lane / CH, + 64 / CH rows per
-        // further load), are parked in the wave's staging and read back as the B operand.
+        // further load), are parked in the wave's staging and read back as the B operand, once for all row blocks.
         {
             const int nblk = npix >> 4;
             const int krow = lane / CH;
@@ -285,26 +302,33 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
             _Pragma("unroll") for (int r = 0; r < KS; ++r)                                                     \
                 kr[slot_][r] = *reinterpret_cast<const dsdpa_u32x4 *>(kplane0 + offs[min((nb_), nblk - 1) * 16 + r * (kWave / CH) + krow] + kpiece);
 #pragma unroll
-            for (int u = 0; u < kRingK; ++u) { DSDPA_DENSE_FETCH_K(u, wave + 4 * u) }
-            for (int nb0 = wave; nb0 < nblk; nb0 += 4 * kRingK) {
+            for (int u = 0; u < kRingK; ++u) { DSDPA_DENSE_FETCH_K(u, wave + kWaves * u) }
+            for (int nb0 = wave; nb0 < nblk; nb0 += kWaves * kRingK) {
 #pragma unroll
                 for (int u = 0; u < kRingK; ++u) {
-                    const int nb = nb0 + 4 * u;
+                    const int nb = nb0 + kWaves * u;
                     if (nb < nblk) {
                         wave_lds_order();                  // (behind the reads of the previous block)
 #pragma unroll
                         for (int r = 0; r < KS; ++r)
                             *reinterpret_cast<dsdpa_u32x4 *>(wstage + (r * (kWave / CH) + krow) * kPitchK + kpiece) = kr[u][r];
                         wave_lds_order();
-                        DSDPA_DENSE_FETCH_K(u, nb + 4 * kRingK)               // (behind the last one: unused)
-                        floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+                        DSDPA_DENSE_FETCH_K(u, nb + kWaves * kRingK)          // (behind the last one: unused)
+                        floatx4 acc[MT];
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
                         const unsigned char *kfrag = wstage + n16 * kPitchK + g * 16;
 #pragma unroll
-                        for (int ks = 0; ks < KS; ++ks)
-                            acc = mfma_16x16x32<S>(qf[ks], *reinterpret_cast<const uint4 *>(kfrag + ks * 64), acc);
-                        // rows 4 g .. 4 g + 3 (queries) of column n16 (pixel nb * 16 + n16)
-                        *reinterpret_cast<float4 *>(S_T + (nb * 16 + n16) * 16 + 4 * g) =
-                            make_float4(acc[0] * qscale, acc[1] * qscale, acc[2] * qscale, acc[3] * qscale);
+                        for (int ks = 0; ks < KS; ++ks) {
+                            const uint4 bf = *reinterpret_cast<const uint4 *>(kfrag + ks * 64);
+#pragma unroll
+                            for (int mt = 0; mt < MT; ++mt) acc[mt] = mfma_16x16x32<S>(qf[mt][ks], bf, acc[mt]);
+                        }
+                        // rows 16 mt + 4 g .. + 3 (queries) of column n16 (pixel nb * 16 + n16)
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt)
+                            *reinterpret_cast<float4 *>(S_T + (nb * 16 + n16) * TQ + mt * 16 + 4 * g) =
+                                make_float4(acc[mt][0] * qscale, acc[mt][1] * qscale, acc[mt][2] * qscale, acc[mt][3] * qscale);
                     }
                 }
             }
@@ -327,24 +351,24 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
             const int dy = ((cstep[i] & 2u) && e0 + bw + dx < npix) ? 1 : 0;
             ent[i] = (unsigned)e0 | ((unsigned)dx << 16) | ((unsigned)dy << 17);
             const int e1 = min(e0 + dx, npix - 1), e2 = e0 + dy * bw, e3 = min(e2 + dx, npix - 1);
-            const float lg = fmaf(wgt[i][0], S_T[e0 * 16 + qi], fmaf(wgt[i][1], S_T[e1 * 16 + qi],
-                             fmaf(wgt[i][2], S_T[e2 * 16 + qi], wgt[i][3] * S_T[e3 * 16 + qi])));
+            const float lg = fmaf(wgt[i][0], S_T[e0 * TQ + qi], fmaf(wgt[i][1], S_T[e1 * TQ + qi],
+                             fmaf(wgt[i][2], S_T[e2 * TQ + qi], wgt[i][3] * S_T[e3 * TQ + qi])));
             logit[i] = live ? lg : kNegBig;
             m_chunk = fmaxf(m_chunk, logit[i]);
         }
-        xm[sub * 16 + qi] = m_chunk;
+        xm[sub * TQ + qi] = m_chunk;
         __syncthreads();                           // (every S value has been read as well)
 #pragma unroll
-        for (int s = 0; s < 16; ++s) m_chunk = fmaxf(m_chunk, xm[s * 16 + qi]);
+        for (int s = 0; s < kSubs; ++s) m_chunk = fmaxf(m_chunk, xm[s * TQ + qi]);
         const float m_new = fmaxf(m_run, m_chunk);
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         m_run = m_new;
         l_run *= alpha;
         if (sub == 0) xq[qi] = alpha;
         // clear P where the box reaches
-        for (int idx = tid; idx < kDenseQ * (kDensePitch / 4); idx += kDenseThreads) {
-            const int r = idx / (kDensePitch / 4), c = idx - r * (kDensePitch / 4);
-            if (4 * c < npix) *reinterpret_cast<uint4 *>(Pm + r * kDensePitch + 4 * c) = make_uint4(0u, 0u, 0u, 0u);
+        for (int idx = tid; idx < TQ * (kPitch / 4); idx += kThreads) {
+            const int r = idx / (kPitch / 4), c = idx - r * (kPitch / 4);
+            if (4 * c < npix) *reinterpret_cast<uint4 *>(Pm + r * kPitch + 4 * c) = make_uint4(0u, 0u, 0u, 0u);
         }
         __syncthreads();
 #pragma unroll
@@ -352,62 +376,63 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
             const float p = __builtin_amdgcn_exp2f(logit[i] - m_new);          // (a dead sample: 2^(-huge) = 0)
             l_run += p;
             const unsigned e0 = ent[i] & 0xffffu, dx = (ent[i] >> 16) & 1u, dyw = ((ent[i] >> 17) & 1u) * (unsigned)bw;
-            unsigned *prow = Pm + qi * kDensePitch;
+            unsigned *prow = Pm + qi * kPitch;
             const float pf = p * kFix;
             atomicAdd(prow + e0, (unsigned)(pf * wgt[i][0] + 0.5f));
             atomicAdd(prow + min(e0 + dx, (unsigned)npix - 1u), (unsigned)(pf * wgt[i][1] + 0.5f));
             atomicAdd(prow + e0 + dyw, (unsigned)(pf * wgt[i][2] + 0.5f));
             atomicAdd(prow + min(e0 + dyw + dx, (unsigned)npix - 1u), (unsigned)(pf * wgt[i][3] + 0.5f));
         }
-        // rows of O are queries 4 g .. 4 g + 3 in this lane
-        {
-            const float4 al = *reinterpret_cast<const float4 *>(xq + 4 * g);
+        // rows of O are queries 16 mt + 4 g .. + 3 in this lane
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const float4 al = *reinterpret_cast<const float4 *>(xq + mt * 16 + 4 * g);
 #pragma unroll
             for (int nt = 0; nt < NTW; ++nt) {
-                oacc[nt][0] *= al.x; oacc[nt][1] *= al.y; oacc[nt][2] *= al.z; oacc[nt][3] *= al.w;
+                oacc[mt][nt][0] *= al.x; oacc[mt][nt][1] *= al.y; oacc[mt][nt][2] *= al.z; oacc[mt][nt][3] *= al.w;
             }
         }
         __syncthreads();                           // P is complete
         // P as 16-bit values for the matrix instruction, in place: every thread takes its pieces of four sums into
         // registers, and after a barrier leaves four values where the row's first half was
         {
-            constexpr int kQuads = kDensePitch / 4;                              // 16-byte pieces of a row
-            constexpr int kMine = (kDenseQ * kQuads + kDenseThreads - 1) / kDenseThreads;
+            constexpr int kQuads = kPitch / 4;                                   // 16-byte pieces of a row
+            constexpr int kMine = (TQ * kQuads + kThreads - 1) / kThreads;
             uint2 mine[kMine];
 #pragma unroll
             for (int i = 0; i < kMine; ++i) {
-                const int idx = tid + i * kDenseThreads, r = idx / kQuads, c = idx - r * kQuads;
+                const int idx = tid + i * kThreads, r = idx / kQuads, c = idx - r * kQuads;
                 mine[i] = make_uint2(0u, 0u);
-                if (r < kDenseQ && 4 * c < npix) mine[i] = dense_pack_p<S>(*reinterpret_cast<const uint4 *>(Pm + r * kDensePitch + 4 * c));
+                if (r < TQ && 4 * c < npix) mine[i] = dense_pack_p<S>(*reinterpret_cast<const uint4 *>(Pm + r * kPitch + 4 * c));
             }
             __syncthreads();
 #pragma unroll
             for (int i = 0; i < kMine; ++i) {
-                const int idx = tid + i * kDenseThreads, r = idx / kQuads, c = idx - r * kQuads;
-                if (r < kDenseQ && 4 * c < npix) *reinterpret_cast<uint2 *>(dense_lds + r * kP16 + c * 8) = mine[i];
+                const int idx = tid + i * kThreads, r = idx / kQuads, c = idx - r * kQuads;
+                if (r < TQ && 4 * c < npix) *reinterpret_cast<uint2 *>(dense_lds + r * kP16 + c * 8) = mine[i];
             }
             __syncthreads();
         }
 
-        // ---- O += P . V, 32 pixels a step; this wave's quarter of the columns, two staging buffers used in turn.
+        // ---- O += P . V, 32 pixels a step; this wave's share of the columns, two staging buffers used in turn.
         // Contraction slot j of k-group g is pixel 4 g + j of the step for j < 4, 16 + 4 g + (j - 4) after: the A
         // operand is then two 8-byte reads of P, and the 8 rows that 32 lanes of a transposing read touch are 8
         // consecutive ones.
         {
             const int nkb = npix >> 5;
-            // row of a load's 64 / VCH that this lane fetches and parks. Four lanes per row (D = 128): the 16 lanes
-            // that one cycle of a 16-byte LDS write serves take every other row (rows of 96 bytes: 0, 2, 4, 6 start
-            // in four different quarters of the banks, 0, 1, 2, 3 do not)
+            // row of a load's 64 / VCH that this lane fetches and parks. Four lanes per row: the 16 lanes that one
+            // cycle of a 16-byte LDS write serves take every other row (rows of 96 bytes: 0, 2, 4, 6 start in four
+            // different quarters of the banks, 0, 1, 2, 3 do not)
             const int vrow_l = VCH == 4 ? 8 * (lane >> 5) + ((lane >> 4) & 1) + 2 * ((lane & 15) >> 2) : lane / VCH;
             const unsigned vpiece = (unsigned)(wave * NTW * 32 + (lane % VCH) * 16);   // byte in the row of V
             const unsigned vpark = (unsigned)(lane % VCH) * 16u;
             // the next kRingV steps' rows are in flight, the next step's are parked while this one is worked on
-            dsdpa_u32x4 vr[kRingV][NTW];
+            dsdpa_u32x4 vr[kRingV][VLD];
 #define DSDPA_DENSE_FETCH_V(slot_, kb_)                                                                        \
-            _Pragma("unroll") for (int r = 0; r < NTW; ++r)                                                    \
+            _Pragma("unroll") for (int r = 0; r < VLD; ++r)                                                    \
                 vr[slot_][r] = *reinterpret_cast<const dsdpa_u32x4 *>(vplane0 + offs[min((kb_), nkb - 1) * 32 + r * (kWave / VCH) + vrow_l] + vpiece);
 #define DSDPA_DENSE_PARK_V(slot_, buf_)                                                                        \
-            _Pragma("unroll") for (int r = 0; r < NTW; ++r)                                                    \
+            _Pragma("unroll") for (int r = 0; r < VLD; ++r)                                                    \
                 *reinterpret_cast<dsdpa_u32x4 *>(wstage + ((buf_) * 32 + r * (kWave / VCH) + vrow_l) * kPitchV + vpark) = vr[slot_][r];
 #pragma unroll
             for (int u = 0; u < kRingV; ++u) { DSDPA_DENSE_FETCH_V(u, u) }
@@ -424,14 +449,20 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
                     if (kb < nkb) {
                         const int buf = kb & 1;
                         wave_lds_order();                  // (buffer `buf` is parked, the other one's reads are issued)
-                        const unsigned char *prow = dense_lds + n16 * kP16 + (kb * 32 + 4 * g) * 2;
-                        const uint2 a0 = *reinterpret_cast<const uint2 *>(prow), a1 = *reinterpret_cast<const uint2 *>(prow + 32);
-                        const uint4 af = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                        uint4 af[MT];
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) {
+                            const unsigned char *prow = dense_lds + (mt * 16 + n16) * kP16 + (kb * 32 + 4 * g) * 2;
+                            const uint2 a0 = *reinterpret_cast<const uint2 *>(prow), a1 = *reinterpret_cast<const uint2 *>(prow + 32);
+                            af[mt] = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                        }
                         const unsigned char *vfrag = wstage + (buf * 32 + 4 * g + (s16 >> 2)) * kPitchV + 4 * (s16 & 3) * 2;
 #pragma unroll
                         for (int nt = 0; nt < NTW; ++nt) {
                             const uint2 b0 = lds_read_tr16(vfrag + nt * 32), b1 = lds_read_tr16(vfrag + 16 * kPitchV + nt * 32);
-                            oacc[nt] = mfma_16x16x32<S>(af, make_uint4(b0.x, b0.y, b1.x, b1.y), oacc[nt]);
+                            const uint4 bf = make_uint4(b0.x, b0.y, b1.x, b1.y);
+#pragma unroll
+                            for (int mt = 0; mt < MT; ++mt) oacc[mt][nt] = mfma_16x16x32<S>(af[mt], bf, oacc[mt][nt]);
                         }
                         const int un = (u + 1) % kRingV;                      // (a constant once the loop is unrolled)
                         DSDPA_DENSE_PARK_V(un, buf ^ 1)                       // (step kb + 1; behind the last one: unused)
@@ -451,17 +482,19 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
     // gather kernel, which reads touched pixels only.
     bool bad = false;
 #pragma unroll
-    for (int nt = 0; nt < NTW; ++nt) {
-        const float sum = (oacc[nt][0] + oacc[nt][1]) + (oacc[nt][2] + oacc[nt][3]);
-        bad = bad || !(fabsf(sum) <= 3.0e38f);
-    }
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NTW; ++nt) {
+            const float sum = (oacc[mt][nt][0] + oacc[mt][nt][1]) + (oacc[mt][nt][2] + oacc[mt][nt][3]);
+            bad = bad || !(fabsf(sum) <= 3.0e38f);
+        }
     if (tid == 0) boxw[0] = 0u;
-    xm[sub * 16 + qi] = l_run;
+    xm[sub * TQ + qi] = l_run;
     __syncthreads();
     if (bad) boxw[0] = 1u;
     float l_tot = 0.f;
 #pragma unroll
-    for (int s = 0; s < 16; ++s) l_tot += xm[s * 16 + qi];
+    for (int s = 0; s < kSubs; ++s) l_tot += xm[s * TQ + qi];
     if (sub == 0) {
         xq[qi] = kUnfix / l_tot;
         if (qlive) lse_[(((size_t)b * dm.V + s1) * dm.H + h) * dm.L + lq] = m_run + __log2f(l_tot);
@@ -470,21 +503,24 @@ __global__ __launch_bounds__(kDenseThreads, 2) void fwd_dense_kernel(
     {
         constexpr int OP = D + 4;                 // pitch of the staging rows: the four row groups land in different banks
         float *O_s = reinterpret_cast<float *>(dense_lds);
-        const float4 inv = *reinterpret_cast<const float4 *>(xq + 4 * g);
 #pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) {
-            const int col = (wave * NTW + nt) * 16 + n16;
-            O_s[(4 * g + 0) * OP + col] = oacc[nt][0] * inv.x;
-            O_s[(4 * g + 1) * OP + col] = oacc[nt][1] * inv.y;
-            O_s[(4 * g + 2) * OP + col] = oacc[nt][2] * inv.z;
-            O_s[(4 * g + 3) * OP + col] = oacc[nt][3] * inv.w;
+        for (int mt = 0; mt < MT; ++mt) {
+            const float4 inv = *reinterpret_cast<const float4 *>(xq + mt * 16 + 4 * g);
+#pragma unroll
+            for (int nt = 0; nt < NTW; ++nt) {
+                const int col = (wave * NTW + nt) * 16 + n16;
+                O_s[(mt * 16 + 4 * g + 0) * OP + col] = oacc[mt][nt][0] * inv.x;
+                O_s[(mt * 16 + 4 * g + 1) * OP + col] = oacc[mt][nt][1] * inv.y;
+                O_s[(mt * 16 + 4 * g + 2) * OP + col] = oacc[mt][nt][2] * inv.z;
+                O_s[(mt * 16 + 4 * g + 3) * OP + col] = oacc[mt][nt][3] * inv.w;
+            }
         }
         __syncthreads();
         const bool redo = boxw[0] != 0u;
-        if (tid == 0) todo_[tile] = redo ? 1 : 0;
+        if (tid < TQ / 16 && l0 + 16 * tid < dm.L) todo_[flag0 + tid] = redo ? 1 : 0;
         if (redo) return;
-        // 16 rows of D elements, 8 elements (16 bytes of output) a thread and pass
-        for (int idx = tid; idx < kDenseQ * (D / 8); idx += kDenseThreads) {
+        // TQ rows of D elements, 8 elements (16 bytes of output) a thread and pass
+        for (int idx = tid; idx < TQ * (D / 8); idx += kThreads) {
             const int r = idx / (D / 8), c8 = idx - r * (D / 8);
             if (r < nq) {
                 float v8[8];

@@ -165,7 +165,7 @@ inline DenseLayout dense_layout(size_t B, size_t V, size_t H, size_t Himg, size_
 {
     DenseLayout d{0, 0, 0};
     const size_t L = Himg * Wimg, chunks = V * ((P + 63) / 64);
-    if (esize != 2 || (D != 64 && D != 128) || P < 64 || chunks > 32 || Himg >= 65536 || Wimg >= 65536 || plane_path_fits(L, D, esize))
+    if (esize != 2 || (D != 64 && D != 128) || P < 64 || chunks > 4096 || Himg >= 65536 || Wimg >= 65536 || plane_path_fits(L, D, esize))
         return d;
     d.ntl = (int)((L + 15) / 16);
     d.todo = 0;
