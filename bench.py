@@ -251,8 +251,8 @@ def main():
         sys.exit("bench.py: this build targets one GPU; run with --gpus 1 "
                  "(the operator shards over (batch, head) with no exchange between the shards)")
 
-    from workloads import WORKLOADS, oob_fractions
-    wl = WORKLOADS[args.workload]
+    from workloads import WORKLOADS, find_workload, oob_fractions
+    wl = find_workload(args.workload)            # (one of the five named shapes, or an extra one such as C5c)
     if args.copy_calibration:
         import torch
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0").normal_()

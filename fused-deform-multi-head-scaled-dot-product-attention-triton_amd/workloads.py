@@ -24,7 +24,7 @@ class Workload:
     P: int          # N_SAMPLES per (query, view)
     sm_scale: float
     dtype: str      # "fp32" | "bf16" | "fp16"
-    coords: str     # "unit" | "border" | "clustered"
+    coords: str     # "unit" | "border" | "clustered" | "coherent"
     seed: int
 
     @property
@@ -73,7 +73,20 @@ WORKLOADS = {
 }
 
 
-def gen_coords(kind, B, V, L, P, gen):
+# Not one of the five named shapes: C5's shape with coordinates as deformable attention produces them, every query
+# looking around its own pixel in the other views (reference point = the query's position, scaled to the middle
+# 60 % of the image and shifted a little per (batch, query view, key view), samples N(0, 0.03^2) around it), so
+# that neighbouring queries look at neighbouring places. C5 itself draws every query's centre at random.
+EXTRA_WORKLOADS = {
+    "C5c": Workload("C5c", 2, 4, 8, 128, 64, 64, 64, 1.0 / math.sqrt(128), "bf16", "coherent", 5),
+}
+
+
+def find_workload(name):
+    return WORKLOADS.get(name) or EXTRA_WORKLOADS[name]
+
+
+def gen_coords(kind, B, V, L, P, gen, W_IMG=None, H_IMG=None):
     """coords (B, V, L, V, P, 2) fp32; last axis is (x, y) normalised to [0, 1]."""
     shape = (B, V, L, V, P, 2)
     if kind == "unit":
@@ -82,6 +95,12 @@ def gen_coords(kind, B, V, L, P, gen):
         return torch.rand(shape, generator=gen, dtype=torch.float32) * 1.2 - 0.1
     if kind == "clustered":
         mu = torch.rand((B, V, L, V, 1, 2), generator=gen, dtype=torch.float32) * 0.2 + 0.4
+        eps = torch.randn(shape, generator=gen, dtype=torch.float32) * 0.03
+        return (mu + eps).clamp_(0.0, 1.0)
+    if kind == "coherent":
+        ys, xs = torch.meshgrid(torch.arange(H_IMG), torch.arange(W_IMG), indexing="ij")
+        base = torch.stack([xs.reshape(-1) / max(W_IMG - 1, 1), ys.reshape(-1) / max(H_IMG - 1, 1)], -1).float()
+        mu = base.view(1, 1, L, 1, 1, 2) * 0.6 + 0.2 + 0.02 * torch.randn((B, V, 1, V, 1, 2), generator=gen, dtype=torch.float32)
         eps = torch.randn(shape, generator=gen, dtype=torch.float32) * 0.03
         return (mu + eps).clamp_(0.0, 1.0)
     raise ValueError(kind)
@@ -94,7 +113,7 @@ def gen_inputs(wl, device="cpu", with_dout=True):
     q = torch.randn(shape, generator=gen, dtype=torch.float32)
     k = torch.randn(shape, generator=gen, dtype=torch.float32)
     v = torch.randn(shape, generator=gen, dtype=torch.float32)
-    coords = gen_coords(wl.coords, wl.B, wl.V, wl.L, wl.P, gen)
+    coords = gen_coords(wl.coords, wl.B, wl.V, wl.L, wl.P, gen, wl.W_IMG, wl.H_IMG)
     outs = [q, k, v]
     if with_dout:
         outs.append(torch.randn(shape, generator=gen, dtype=torch.float32))
@@ -111,7 +130,7 @@ def oob_fractions(wl):
     shape = (wl.B, wl.V, wl.H, wl.L, wl.D)
     for _ in range(3):                      # q, k, v come first in the draw order
         torch.randn(shape, generator=gen, dtype=torch.float32)
-    c = gen_coords(wl.coords, wl.B, wl.V, wl.L, wl.P, gen)
+    c = gen_coords(wl.coords, wl.B, wl.V, wl.L, wl.P, gen, wl.W_IMG, wl.H_IMG)
     x0 = torch.floor(c[..., 0] * (wl.W_IMG - 1)).to(torch.int64)
     y0 = torch.floor(c[..., 1] * (wl.H_IMG - 1)).to(torch.int64)
     inside = []

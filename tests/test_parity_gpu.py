@@ -17,7 +17,7 @@ import torch
 from oracle import oracle_bwd, oracle_fwd
 from ops import _native
 from ops.triton import deform_sdpa_triton
-from workloads import WORKLOADS, gen_inputs
+from workloads import WORKLOADS, find_workload, gen_inputs
 from parity_util import oracle_on_slices, rel, slice_bh, spread_slices
 
 pytestmark = pytest.mark.gpu
@@ -362,7 +362,7 @@ def test_unreadable_layouts_are_copied():
 
 
 # ------------------------------------------------------------------ the five named workloads
-@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5", "C5c"])
 def test_named_workloads_full_size(name):
     """Full-size run of each workload (the reference checks out, dq, dk, dv on the whole tensors,
     benchmark.py:116-149).
@@ -374,7 +374,7 @@ def test_named_workloads_full_size(name):
     * every (batch, head), sliced or not: the identities <q,dq> = <K,dK> (the logits are bilinear in q and K)
       and <V,dV> = <dout,out>, taken PER (batch, head) -- with `out` pinned everywhere by the full forward,
       a gradient plane that landed in another head's or batch item's place breaks them."""
-    wl = WORKLOADS[name]
+    wl = find_workload(name)               # (C5c: C5's shape with every query looking around its own pixel)
     say(f"[case] workload {name} {wl}")
     q, k, v, c, do = gen_inputs(wl)
     dt = wl.torch_dtype()
