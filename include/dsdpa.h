@@ -79,9 +79,12 @@ enum { DSDPA_F32 = 0, DSDPA_BF16 = 1, DSDPA_F16 = 2 };
  * Writes out (storage dtype) and lse (fp32).
  *
  * `workspace` must hold dsdpa_fwd_workspace_bytes(...) bytes (256-byte aligned; may be NULL when that is
- * 0). It is scratch for the duration of the call on `stream`: a table of the bilinear weights and tap
- * addresses of every coordinate pair, computed once from coords and shared by all H heads (the
- * reference recomputes them per head inside `_fwd_kernel`, ops/triton.py:118-140).
+ * 0). It is scratch for the duration of the call on `stream`. Shapes whose K and V planes fit in LDS: a
+ * table of the bilinear weights and tap addresses of every coordinate pair, computed once from coords and
+ * shared by all H heads (the reference recomputes them per head inside `_fwd_kernel`,
+ * ops/triton.py:118-140). 16-bit storage with D = 64 or 128, P >= 64 and larger planes: one byte per
+ * (batch, head, query view, 16 consecutive queries), by which the kernel that works on tiles of 16 queries
+ * tells the per-query kernel launched behind it which tiles are left to do.
  */
 int dsdpa_fwd_f32(const float *q, const float *k, const float *v, const float *coords,
                   float *out, float *lse, void *workspace,
@@ -103,7 +106,8 @@ int dsdpa_fwd_f16(const void *q, const void *k, const void *v, const float *coor
  * workspace is not an argument: it is a buffer of DSDPA_NOALLOC_SCRATCH_BYTES built into the library, one
  * copy per GPU, held until the process ends. The call allocates and frees nothing. A shape whose
  * dsdpa_fwd_workspace_bytes() exceeds the buffer is refused with DSDPA_ERR_SCRATCH before anything is
- * launched (shapes that need no workspace always pass). All calls on one GPU share that GPU's buffer: calls
+ * launched (shapes that need no workspace always pass; where only the tile flags of the 16-query kernel do
+ * not fit, the per-query kernel does all the work instead). All calls on one GPU share that GPU's buffer: calls
  * that overlap on one GPU (two streams, two threads) race on it; calls on one stream, or otherwise ordered,
  * are fine, since every call rewrites all of the scratch it reads.
  */
@@ -175,8 +179,9 @@ int dsdpa_bwd_f16(const void *q, const void *k, const void *v, const float *coor
                   float sm_scale, const long long *strides, unsigned flags, void *stream);
 
 /* Bytes of device workspace dsdpa_fwd_* needs for a storage dtype: 20 bytes per coordinate pair when the
- * K and V planes of one view fit in LDS (the staged kernels), else 0; 0 also if an argument is invalid.
- * No counterpart in the reference. */
+ * K and V planes of one view fit in LDS (the staged kernels); else one byte per 16 queries of every
+ * (batch, head, view) for 16-bit storage with D = 64 or 128 and P >= 64, else 0; 0 also if an argument is
+ * invalid. No counterpart in the reference. */
 size_t dsdpa_fwd_workspace_bytes(int dtype, int B, int V, int H, int Himg, int Wimg, int D, int P);
 
 /* Bytes of device workspace dsdpa_bwd_* needs for a storage dtype (0 if an argument is invalid).
@@ -202,7 +207,9 @@ int dsdpa_version(void);
 /* Forward and backward-dq: AUTO and LDS stage each key view's K/V planes in LDS
  * when a plane pair fits (AUTO: unless there are at most 3 samples per view and 8
  * or more views, where staging costs more than it saves), GATHER always reads the
- * taps from global memory.
+ * taps from global memory, one query at a time. AUTO alone lets the forward work on
+ * tiles of 16 queries with the matrix instructions where the shape allows it
+ * (16-bit storage, D = 64 or 128, P >= 64, planes too large for LDS).
  * Backward dk/dv: AUTO = cell-binned register accumulation, LDS = tiles of the
  * plane accumulated in LDS with fp64 atomics, GATHER = global float atomics per
  * tap as in the reference (ops/triton.py:345-360). */
