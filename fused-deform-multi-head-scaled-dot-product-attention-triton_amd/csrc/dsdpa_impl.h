@@ -8,6 +8,7 @@
 #include "dsdpa_cell.h"
 #include "dsdpa_plane.h"
 #include "dsdpa_dense.h"
+#include "dsdpa_slab.h"
 
 namespace dsdpa {
 
@@ -161,6 +162,32 @@ int launch_fwd_gather(const void *q, const void *k, const void *v, const float *
                               timer.start(), timer.stop(),
                            q, k, v, coords, out, lse, todo, ntl, dm);
     return check_launch();
+}
+
+// The slab forward (fp32 storage, 16 samples per view): a workgroup of 16 waves per block of 64 * IT query rows of a
+// (batch, head); the whole image of a view in LDS, 16 columns at a time, in two buffers.
+template <typename S, int D>
+int launch_fwd_slab(const void *q, const void *k, const void *v, const float *coords, void *out, float *lse,
+                    const Dims &dm, hipStream_t st)
+{
+    if constexpr (S::kBytes != 4 || (D != 32 && D != 64 && D != 128)) {
+        return DSDPA_ERR_UNSUPPORTED;
+    } else {
+        constexpr int IT = 3;
+        constexpr int RB = kSlabWaves * 4 * IT;
+        const int nblk = (dm.V * dm.L + RB - 1) / RB;
+        const long long blocks = (long long)dm.B * dm.H * nblk;
+        if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
+        auto kern = fwd_slab_kernel<D, IT>;
+        static std::atomic<unsigned long long> lds_set{0};
+        if (int rc = allow_full_lds(kern, lds_set)) return rc;
+        ScopedKernelTimer timer(0, st);
+        const unsigned buf_bytes = (unsigned)slab_buffer_bytes(dm.Himg, dm.Wimg);
+        DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(kSlabWaves * kWave), (size_t)2 * buf_bytes + kSlabWaves * 4 * IT * kSlabBytes, st, timer.start(),
+                     timer.stop(), (const float *)q, (const float *)k, (const float *)v, coords, (float *)out, lse, dm, nblk,
+                     slab_pitch(dm.Wimg), buf_bytes);
+        return check_launch();
+    }
 }
 
 // The dense-box forward (16-bit storage, D = 64 or 128): one workgroup per tile of 16 queries; the tiles it
@@ -387,6 +414,7 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
                         (path == DSDPA_PATH_LDS || !few_samples_prefer_gather(V, P));
     // (DSDPA_PATH_GATHER keeps its meaning: every tap, or every pixel of a query's window, read by the gather kernel)
     const bool dense = path == DSDPA_PATH_AUTO && dn.bytes != 0;
+    const bool slab = path == DSDPA_PATH_AUTO && !staged && slab_path_fits(V, Himg, Wimg, D, P, S::kBytes);
     char *ws = (char *)workspace;
     if (staged && (rc = launch_plane_descriptors(coords, dm, ws, dl, false, ZeroJob{}, 4, st)) != DSDPA_OK) return rc;
     const float4 *desc_w = (const float4 *)(ws + dl.w);
@@ -395,6 +423,7 @@ int fwd_impl(const void *q, const void *k, const void *v, const float *coords, v
 #define DSDPA_FWD_CASE(DD)                                                                        \
     case DD:                                                                                      \
         if (staged) return launch_fwd_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dm, st);    \
+        if (slab) return launch_fwd_slab<S, DD>(q, k, v, coords, out, lse, dm, st);               \
         if (dense && (rc = launch_fwd_dense<S, DD>(q, k, v, coords, out, lse, ws, dn, dm, st)) != DSDPA_OK) return rc; \
         return launch_fwd_gather<S, DD>(q, k, v, coords, out, lse, todo, dn.ntl, dm, st);
     switch (D) {

@@ -1,0 +1,311 @@
+// Forward for fp32 storage and 16 samples per view on images whose K/V planes do not fit in LDS but whose planes
+// cut to 16 columns do, twice: "slabs" of 64 bytes per pixel (`ops/triton.py:118-170` is the sampling and softmax
+// loop this replaces; the reference gathers every tap from global memory).
+//
+// A workgroup owns a block of query rows of one (batch, head). For every key view it walks the column slabs of K
+// and then those of V, each the whole image at 64 bytes per pixel, in two LDS buffers: the slab of the next step
+// is fetched into registers before the work on the present one and written to the other buffer after it, one
+// barrier per step. One lane owns one (query row, sample) pair for a whole view: it reads its four tap rows from
+// the slab in 16-byte pieces and keeps the partial dot product (K slabs) in a register, so the tap weights and
+// addresses are computed once per sample and view and nothing is summed across lanes for the logits. For the V
+// slabs the 16 samples of a query row sit in 16 neighbouring lanes, whose weighted sums are combined by a
+// reduce-scatter over those lanes: every lane ends up with one column of the slab.
+//
+// LDS banks (64 banks of 4 bytes; a 16-byte read is served 16 lanes a clock): the piece a lane reads at step c is
+// (c + lane) mod 4, so four neighbouring lanes cover the 16 banks of one slab row; which quarter of the banks a
+// row lies in is its index mod 4. Image rows are stored with a pitch of 2 mod 4 pixels, which gives the four
+// taps of a sample (x, x+1, x+pitch, x+pitch+1) four different quarters, and lanes 4g .. 4g+3 of every 16 read
+// their taps in the order that starts in quarter g: the 16 lanes of a clock then touch all 64 banks once,
+// whatever the coordinates (taps clamped at the image border share a row and take a second clock).
+#pragma once
+#include "dsdpa_common.h"
+
+namespace dsdpa {
+
+constexpr int kSlabBytes = 64;             // bytes of one pixel in a slab: 16 fp32 columns
+constexpr int kSlabCols = 16;
+constexpr int kSlabWaves = 16;
+constexpr int kSlabSamples = 16;           // samples per (query row, view) this kernel is written for
+constexpr int kSlabStage = 4;              // runs of 16 pixels of an image row a wave moves per slab
+
+// slab rows between two image rows: the width rounded up to 2 mod 4
+__host__ __device__ inline int slab_pitch(int Wimg) { return Wimg + ((6 - (Wimg & 3)) & 3); }
+
+// maximum over aligned groups of 16 lanes; every lane gets it
+__device__ __forceinline__ float group16_max(float x)
+{
+    x = fmaxf(x, dpp_f32<0xB1>(x));
+    x = fmaxf(x, dpp_f32<0x4E>(x));
+    x = fmaxf(x, dpp_f32<0x141>(x));
+    x = fmaxf(x, dpp_f32<0x140>(x));
+    return x;
+}
+
+// The four tap rows of a sample, made opaque to the compiler at the place they are used: the addresses formed
+// from them (16 per sample and slab) are then computed there, next to their reads, and not once for all slabs.
+__device__ __forceinline__ void keep_here(unsigned (&o)[4])
+{
+    asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
+}
+
+__device__ __forceinline__ void pin_here(float (&o)[4])
+{
+    asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
+}
+
+// rows of 16 lanes rotated: lane i of a row receives the value of lane (i - N) mod 16
+#define DSDPA_ROW_ROR(N) (0x120 + (N))
+
+// the value of lane i ^ 4: a rotation by 12 for the lanes with bit 2 clear (banks 0 and 2 of a row), by 4 for the others
+__device__ __forceinline__ float dpp_xor4(float x)
+{
+    int r = __builtin_amdgcn_update_dpp(0, __float_as_int(x), DSDPA_ROW_ROR(12), 0xf, 0x5, false);
+    r = __builtin_amdgcn_update_dpp(r, __float_as_int(x), DSDPA_ROW_ROR(4), 0xf, 0xa, false);
+    return __int_as_float(r);
+}
+
+template <int D, int IT>
+__global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
+    const float *__restrict__ q_, const float *__restrict__ k_, const float *__restrict__ v_,
+    const float *__restrict__ coords_, float *__restrict__ out_, float *__restrict__ lse_, Dims dm, int nblk,
+    int pitch, unsigned buf_bytes)
+{
+    constexpr int NSLAB = D / kSlabCols;
+    constexpr int RB = kSlabWaves * 4 * IT;          // query rows per workgroup
+    extern __shared__ __attribute__((aligned(16))) char slab[];
+    const float4 *slab4 = reinterpret_cast<const float4 *>(slab);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int i3 = lane & 3, g4 = (lane >> 2) & 3, smp = lane & 15, rg = lane >> 4;
+    const int blk = xcd_logical_block(blockIdx.x, gridDim.x);
+    const int bh = blk / nblk, rb = blk - bh * nblk;
+    const int b = bh / dm.H, h = bh - b * dm.H;
+    const int VL = dm.V * dm.L;
+    const float *qb = q_ + (size_t)((long long)b * dm.q_sb + (long long)h * dm.q_sh);
+    const size_t kvb = dm.kv_plane(b, 0, h);
+    const float2 *cb = reinterpret_cast<const float2 *>(coords_) + (size_t)b * VL * dm.N;
+    const float qscale = dm.sm_scale * kLog2e;
+
+    // the pieces of a 64-byte slab row in this lane's order (in 16-byte units)
+    unsigned chv[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) chv[c] = (unsigned)((c + i3) & 3);
+
+    bool live[IT];
+    unsigned coff[IT];
+    float m[IT], lsum[IT], acc[IT][NSLAB];
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int rr = rb * RB + (wave * IT + it) * 4 + rg;
+        live[it] = rr < VL;
+        const int rc = min(rr, VL - 1);
+        coff[it] = (unsigned)rc * (unsigned)dm.N + (unsigned)smp;
+        m[it] = kNegBig;
+        lsum[it] = 0.f;
+#pragma unroll
+        for (int s = 0; s < NSLAB; ++s) acc[it][s] = 0.f;
+    }
+
+    // q goes through LDS too, 16 columns of the wave's 4 * IT rows at a time (a region per wave: no barrier): a load
+    // issued behind the slab's loads would only return after them (loads return in order), at the start of
+    // every K step. The piece for the next K step is requested before that step's slab and parked after the work
+    // on the present step; lane i moves piece i & 3 of row i >> 2.
+    float4 *qlds = reinterpret_cast<float4 *>(slab + 2 * buf_bytes) + wave * (4 * IT * 4);
+    unsigned qst_off;
+    {
+        const int rc = min(rb * RB + wave * (4 * IT) + min(lane >> 2, 4 * IT - 1), VL - 1);
+        const int s1 = rc / dm.L, l = rc - s1 * dm.L;
+        qst_off = (unsigned)s1 * (unsigned)dm.q_sv + (unsigned)l * (unsigned)dm.q_sl + (unsigned)(lane & 3) * 4;
+    }
+    float4 qnext = *reinterpret_cast<const float4 *>(qb + qst_off);          // K slab 0 of the first view
+    if (lane < 16 * IT) qlds[lane] = qnext;
+
+    // Staging: a wave moves runs of 16 pixels of one image row (four lanes per pixel, 16 bytes each), run
+    // wave + 16 j of the image's Himg * nxb runs at its step j: where a run starts is the same for all lanes (scalar
+    // registers), a lane adds its own place in the run. Offsets inside one (batch, head) fit 32 bits.
+    const int nxb = (dm.Wimg + 15) >> 4, nruns = dm.Himg * nxb;
+    int st_pix[kSlabStage], st_dst[kSlabStage], st_x0[kSlabStage];       // per wave: scalar registers
+#pragma unroll
+    for (int j = 0; j < kSlabStage; ++j) {
+        const int run = min(wave + kSlabWaves * j, nruns - 1);           // (a run past the image: the last one once more)
+        const int y = run / nxb, x0 = (run - y * nxb) * 16;
+        st_pix[j] = __builtin_amdgcn_readfirstlane(y * dm.Wimg + x0);
+        st_dst[j] = __builtin_amdgcn_readfirstlane((y * pitch + x0) * kSlabBytes);
+        st_x0[j] = __builtin_amdgcn_readfirstlane(x0);
+    }
+    // step ph of the walk: view ph / (2 NSLAB), K slabs first, then V slabs
+    const int nsteps = dm.V * 2 * NSLAB;
+    // The slab goes from memory to LDS without passing through registers (global_load_lds_dwordx4: lane i of a wave
+    // writes 16 bytes at the wave's LDS base + 16 i, which is the layout of a run). stage_fetch only issues the
+    // loads; stage_wait, before the barrier that ends a step, waits for this wave's.
+    auto stage_fetch = [&](int ph) {
+        const int s2 = ph / (2 * NSLAB), r = ph - s2 * (2 * NSLAB);
+        const float *plane = (r < NSLAB ? k_ : v_) + kvb + (size_t)s2 * dm.kv_sv + (r % NSLAB) * kSlabCols + (lane & 3) * 4;
+        const unsigned dst0 = (unsigned)(uintptr_t)slab + (unsigned)(ph & 1) * buf_bytes;
+#pragma unroll
+        for (int j = 0; j < kSlabStage; ++j) {
+            // (lanes past the end of the image row stay out)
+            if (st_x0[j] + (lane >> 2) < dm.Wimg) {
+                const unsigned pix = (unsigned)(st_pix[j] + (lane >> 2));
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void *)(plane + pix * (unsigned)dm.kv_sl),
+                    (__attribute__((address_space(3))) void *)(uintptr_t)(dst0 + (unsigned)st_dst[j]), 16, 0, 0);
+            }
+        }
+    };
+    auto stage_wait = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+    stage_fetch(0);
+    stage_wait();
+    __syncthreads();
+
+    int ph = 0;
+    for (int s2 = 0; s2 < dm.V; ++s2) {
+        // this lane's samples of the view: tap rows (in 16-byte units of the slab) and weights, the four taps in
+        // the order that starts in this lane's quarter of the banks
+        unsigned off[IT][4];
+        float w[IT][4], part[IT];
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const float2 xy = cb[coff[it] + (unsigned)s2 * (unsigned)dm.P];
+            const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
+            // slab rows of the taps: image row y at y * pitch. The taps 00, 01, 10, 11 of a sample inside the image lie
+            // in the quarters r, r+1, r+2, r+3 (mod 4) with r that of tap 00. A tap outside the image has weight 0 and
+            // may read any row: it reads one of the first four, the one in the quarter it would have had (clamped
+            // into the image it would share a row with its neighbour, and the 16 lanes of a clock would collide).
+            const int n0 = tp.y0 * pitch + tp.x0;
+            const bool vx0 = (unsigned)tp.x0 < (unsigned)dm.Wimg, vx1 = (unsigned)(tp.x0 + 1) < (unsigned)dm.Wimg;
+            const bool vy0 = (unsigned)tp.y0 < (unsigned)dm.Himg, vy1 = (unsigned)(tp.y0 + 1) < (unsigned)dm.Himg;
+            unsigned o[4] = { (unsigned)((vx0 && vy0) ? n0 : (n0 & 3)), (unsigned)((vx1 && vy0) ? n0 + 1 : ((n0 + 1) & 3)),
+                              (unsigned)((vx0 && vy1) ? n0 + pitch : ((n0 + pitch) & 3)),
+                              (unsigned)((vx1 && vy1) ? n0 + pitch + 1 : ((n0 + pitch + 1) & 3)) };
+            float ww[4] = { tp.w[0], tp.w[1], tp.w[2], tp.w[3] };
+            const int rot = (g4 - n0) & 3;                 // read order: tap (k + rot) mod 4 at step k
+            if (rot & 1) {
+                const unsigned t0 = o[0]; o[0] = o[1]; o[1] = o[2]; o[2] = o[3]; o[3] = t0;
+                const float f0 = ww[0]; ww[0] = ww[1]; ww[1] = ww[2]; ww[2] = ww[3]; ww[3] = f0;
+            }
+            if (rot & 2) {
+                const unsigned t0 = o[0], t1 = o[1]; o[0] = o[2]; o[1] = o[3]; o[2] = t0; o[3] = t1;
+                const float f0 = ww[0], f1 = ww[1]; ww[0] = ww[2]; ww[1] = ww[3]; ww[2] = f0; ww[3] = f1;
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                off[it][k] = o[k] * (kSlabBytes / 16);
+                w[it][k] = ww[k];
+            }
+            part[it] = 0.f;
+        }
+        // ---- logits: K slab by slab
+#pragma unroll 1
+        for (int s = 0; s < NSLAB; ++s, ++ph) {
+            if (s + 1 < NSLAB) qnext = *reinterpret_cast<const float4 *>(qb + qst_off + (s + 1) * kSlabCols);
+            stage_fetch(ph + 1);                      // (a K step is never the last one)
+            const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
+#pragma unroll
+            for (int it = 0; it < IT; ++it) {
+                const float4 *qrow = qlds + (it * 4 + rg) * 4;
+                unsigned ob[4] = { off[it][0] + cur, off[it][1] + cur, off[it][2] + cur, off[it][3] + cur };
+                keep_here(ob);
+                float d[4] = { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float4 x = qrow[chv[c]];
+                    float4 t[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) t[k] = slab4[ob[k] + chv[c]];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        d[k] = fmaf(x.x, t[k].x, fmaf(x.y, t[k].y, fmaf(x.z, t[k].z, fmaf(x.w, t[k].w, d[k]))));
+                    pin_here(d);                      // (the arithmetic on a piece stays next to its reads)
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                part[it] += fmaf(w[it][0], d[0], fmaf(w[it][1], d[1], fmaf(w[it][2], d[2], w[it][3] * d[3])));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (s + 1 < NSLAB && lane < 16 * IT) qlds[lane] = qnext;      // (this wave has read the present piece)
+            stage_wait();
+            __syncthreads();
+        }
+        // ---- softmax bookkeeping of the view; the weights become p * w
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const float sc = part[it] * qscale;
+            const float m_new = fmaxf(m[it], group16_max(sc));
+            const float alpha = __builtin_amdgcn_exp2f(m[it] - m_new);
+            const float p = __builtin_amdgcn_exp2f(sc - m_new);
+            m[it] = m_new;
+            lsum[it] = fmaf(lsum[it], alpha, p);
+#pragma unroll
+            for (int s = 0; s < NSLAB; ++s) acc[it][s] *= alpha;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) w[it][t] *= p;
+        }
+        // ---- out: V slab by slab
+#pragma unroll
+        for (int s = 0; s < NSLAB; ++s, ++ph) {
+            if (s == NSLAB - 1) qnext = *reinterpret_cast<const float4 *>(qb + qst_off);      // the next view starts with K slab 0
+            if (ph + 1 < nsteps) stage_fetch(ph + 1);
+            const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
+#pragma unroll
+            for (int it = 0; it < IT; ++it) {
+                // register c of lane j holds piece (c + j) mod 4: the same piece is in register c + 2 of lane
+                // j + 2 and in register c + 1 of lane j - 1 (lanes mod 16)
+                unsigned ob[4] = { off[it][0] + cur, off[it][1] + cur, off[it][2] + cur, off[it][3] + cur };
+                keep_here(ob);
+                float o[2][4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float4 t[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) t[k] = slab4[ob[k] + chv[c]];
+                    const float x0 = fmaf(w[it][0], t[0].x, fmaf(w[it][1], t[1].x, fmaf(w[it][2], t[2].x, w[it][3] * t[3].x)));
+                    const float x1 = fmaf(w[it][0], t[0].y, fmaf(w[it][1], t[1].y, fmaf(w[it][2], t[2].y, w[it][3] * t[3].y)));
+                    const float x2 = fmaf(w[it][0], t[0].z, fmaf(w[it][1], t[1].z, fmaf(w[it][2], t[2].z, w[it][3] * t[3].z)));
+                    const float x3 = fmaf(w[it][0], t[0].w, fmaf(w[it][1], t[1].w, fmaf(w[it][2], t[2].w, w[it][3] * t[3].w)));
+                    if (c < 2) {
+                        o[c][0] = x0; o[c][1] = x1; o[c][2] = x2; o[c][3] = x3;
+                    } else {
+                        o[c - 2][0] += dpp_f32<DSDPA_ROW_ROR(14)>(x0);
+                        o[c - 2][1] += dpp_f32<DSDPA_ROW_ROR(14)>(x1);
+                        o[c - 2][2] += dpp_f32<DSDPA_ROW_ROR(14)>(x2);
+                        o[c - 2][3] += dpp_f32<DSDPA_ROW_ROR(14)>(x3);
+                    }
+                    pin_here(o[c & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[0][e] += dpp_f32<DSDPA_ROW_ROR(1)>(o[1][e]);
+                // piece j mod 4 summed over four lanes; lanes j ^ 8, j ^ 4, j ^ 12 hold the other twelve: two
+                // halving steps leave lane j with column 2 * bit 3 + bit 2 of the piece
+                const bool b8 = (lane & 8) != 0, b4 = (lane & 4) != 0;
+                const float k0 = b8 ? o[0][2] : o[0][0], k1 = b8 ? o[0][3] : o[0][1];
+                const float g0 = b8 ? o[0][0] : o[0][2], g1 = b8 ? o[0][1] : o[0][3];
+                const float h0 = k0 + dpp_f32<DSDPA_ROW_ROR(8)>(g0), h1 = k1 + dpp_f32<DSDPA_ROW_ROR(8)>(g1);
+                const float kk = b4 ? h1 : h0, gg = b4 ? h0 : h1;
+                acc[it][s] += kk + dpp_xor4(gg);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (s == NSLAB - 1 && lane < 16 * IT) qlds[lane] = qnext;
+            stage_wait();
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue: lane j of a row's 16 lanes holds column 16 s + 4 (j & 3) + 2 * bit 3 + bit 2 of the row
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const float l16 = group_sum<16>(lsum[it]);
+        if (!live[it]) continue;
+        const int rr = rb * RB + (wave * IT + it) * 4 + rg;
+        const int s1 = rr / dm.L, l = rr - s1 * dm.L;
+        const size_t row = (((size_t)b * dm.V + s1) * dm.H + h) * dm.L + l;
+        const float inv = 1.0f / l16;
+        const int col = 4 * i3 + 2 * ((lane >> 3) & 1) + ((lane >> 2) & 1);
+#pragma unroll
+        for (int s = 0; s < NSLAB; ++s) out_[row * D + s * kSlabCols + col] = acc[it][s] * inv;
+        if (smp == 0) lse_[row] = m[it] + __log2f(l16);
+    }
+}
+
+}  // namespace dsdpa

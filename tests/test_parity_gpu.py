@@ -113,6 +113,44 @@ def test_staged_forward_two_row_blocks(dtype):
     assert rel(dv, rdv) < TOL_BWD[dtype]
 
 
+# fp32 storage, 16 samples per view, planes too large for LDS but small enough for two 16-column slabs of the whole
+# image: the forward walks the planes slab by slab through LDS (fwd_slab_kernel), every tap read from there.
+SLABS = [
+    # seed B  V  H  Himg Wimg D    lo     hi
+    (81, 1, 2, 2, 20, 20, 64, -0.1, 1.1),       # width a multiple of 4: two padding columns per image row; 800 query rows: 4 full workgroups and a part
+    (82, 2, 3, 1, 23, 19, 64, -0.3, 1.3),       # odd width, runs of 16 pixels cut by the row end, heavy out-of-image
+    (83, 1, 2, 2, 17, 17, 128, 0.0, 1.0),       # eight slabs per plane
+    (84, 1, 1, 3, 20, 32, 32, -0.05, 1.05),     # two slabs per plane, one view
+    (85, 1, 2, 1, 32, 32, 64, -0.1, 1.1),       # the largest image the kernel takes (64 runs)
+]
+
+
+@pytest.mark.parametrize("case", SLABS, ids=[f"b{c[0]}" for c in SLABS])
+def test_slab_forward_vs_oracle(case):
+    seed, B, V, H, Himg, Wimg, D, lo, hi = case
+    P, dtype = 16, torch.float32
+    say(f"[case] slabs seed={seed} B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} {dtype}")
+    q, k, v, c, do = make_case(seed, B, V, H, Himg, Wimg, D, P, lo, hi, dtype)
+    c[0, 0, 1, 0, 3, 0] = float("nan")                     # a sample without taps
+    c[0, V - 1, 5, 0, 7] = torch.tensor([1.0, 1.0])        # exactly on the last pixel: x1, y1 outside with weight 0
+    c[0, 0, 6, V - 1, 2] = torch.tensor([-0.5, 0.5])       # far outside
+    scale = 1.0 / math.sqrt(D)
+    out, dq, dk, dv = run_op(q, k, v, c, do, Wimg, Himg, scale)
+    prev = _native.set_path(_native.PATH_GATHER)           # the same forward by the gather kernel
+    try:
+        with torch.no_grad():
+            og = deform_sdpa_triton(q.cuda(), k.cuda(), v.cuda(), c.cuda(), Wimg, Himg, scale)
+    finally:
+        _native.set_path(prev)
+    ro, _, rdq, rdk, rdv = oracle_all(q, k, v, c, do, Wimg, Himg, scale)
+    assert torch.isfinite(out).all()
+    assert rel(out, ro) < TOL_FWD[dtype]
+    assert rel(out, og.cpu().numpy()) < TOL_FWD[dtype]
+    assert rel(dq, rdq) < TOL_BWD[dtype]                   # (lse of the slab forward feeds the backward)
+    assert rel(dk, rdk) < TOL_BWD[dtype]
+    assert rel(dv, rdv) < TOL_BWD[dtype]
+
+
 # Clustered coordinates with at least 64 samples per view: the gather kernels then cut chunks per key view and
 # work on the pixels of the window a chunk's samples fall into (fp32: multiply-adds; 16-bit storage: the 4x4x4
 # block matrix instruction), or gather tap by tap where the window is too large or the image too narrow.
