@@ -64,6 +64,141 @@ __device__ __forceinline__ float dpp_xor4(float x)
     return __int_as_float(r);
 }
 
+// ------------------------------------------------------------------ pieces shared by the forward and dq kernels
+// What a lane keeps of one of its samples for a view: the slab rows of the four taps (in 16-byte units, in this
+// lane's read order) and their weights in the same order.
+// Slab rows: image row y at y * pitch. The taps 00, 01, 10, 11 of a sample inside the image lie in the quarters
+// r, r+1, r+2, r+3 (mod 4) with r that of tap 00. A tap outside the image has weight 0 and may read any row: it
+// reads one of the first four, the one in the quarter it would have had (clamped into the image it would share a
+// row with its neighbour, and the 16 lanes of a clock would collide).
+__device__ __forceinline__ void slab_sample(float2 xy, const Dims &dm, int pitch, int g4, unsigned (&off)[4], float (&w)[4])
+{
+    const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
+    const int n0 = tp.y0 * pitch + tp.x0;
+    const bool vx0 = (unsigned)tp.x0 < (unsigned)dm.Wimg, vx1 = (unsigned)(tp.x0 + 1) < (unsigned)dm.Wimg;
+    const bool vy0 = (unsigned)tp.y0 < (unsigned)dm.Himg, vy1 = (unsigned)(tp.y0 + 1) < (unsigned)dm.Himg;
+    unsigned o[4] = { (unsigned)((vx0 && vy0) ? n0 : (n0 & 3)), (unsigned)((vx1 && vy0) ? n0 + 1 : ((n0 + 1) & 3)),
+                      (unsigned)((vx0 && vy1) ? n0 + pitch : ((n0 + pitch) & 3)),
+                      (unsigned)((vx1 && vy1) ? n0 + pitch + 1 : ((n0 + pitch + 1) & 3)) };
+    float ww[4] = { tp.w[0], tp.w[1], tp.w[2], tp.w[3] };
+    const int rot = (g4 - n0) & 3;                 // read order: tap (k + rot) mod 4 at step k
+    if (rot & 1) {
+        const unsigned t0 = o[0]; o[0] = o[1]; o[1] = o[2]; o[2] = o[3]; o[3] = t0;
+        const float f0 = ww[0]; ww[0] = ww[1]; ww[1] = ww[2]; ww[2] = ww[3]; ww[3] = f0;
+    }
+    if (rot & 2) {
+        const unsigned t0 = o[0], t1 = o[1]; o[0] = o[2]; o[1] = o[3]; o[2] = t0; o[3] = t1;
+        const float f0 = ww[0], f1 = ww[1]; ww[0] = ww[2]; ww[1] = ww[3]; ww[2] = f0; ww[3] = f1;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        off[k] = o[k] * (kSlabBytes / 16);
+        w[k] = ww[k];
+    }
+}
+
+// x . (sum_t w_t * row_t) over the 16 columns of the slab in buffer `cur`: x is the wave's parked vector of the
+// sample's query row (q or dout), read from LDS in the same rotated pieces as the taps.
+__device__ __forceinline__ float slab_dot(const float4 *slab4, const float4 *xrow, const unsigned (&off)[4], unsigned cur,
+                                          const unsigned (&chv)[4], const float (&w)[4])
+{
+    unsigned ob[4] = { off[0] + cur, off[1] + cur, off[2] + cur, off[3] + cur };
+    keep_here(ob);
+    float d[4] = { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const float4 x = xrow[chv[c]];
+        float4 t[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) t[k] = slab4[ob[k] + chv[c]];
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            d[k] = fmaf(x.x, t[k].x, fmaf(x.y, t[k].y, fmaf(x.z, t[k].z, fmaf(x.w, t[k].w, d[k]))));
+        pin_here(d);                      // (the arithmetic on a piece stays next to its reads)
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    return fmaf(w[0], d[0], fmaf(w[1], d[1], fmaf(w[2], d[2], w[3] * d[3])));
+}
+
+// sum over the 16 lanes of a query row of (sum_t w_t * row_t) on the slab in buffer `cur`; lane j of the 16 gets
+// column 4 (j & 3) + 2 * bit 3 + bit 2 of the slab.
+// Register c of lane j holds piece (c + j) mod 4: the same piece is in register c + 2 of lane j + 2 and in
+// register c + 1 of lane j - 1 (lanes mod 16); the lanes j ^ 8, j ^ 4, j ^ 12 then hold the other twelve lanes'
+// sums of piece j mod 4, and two halving steps leave one column each.
+__device__ __forceinline__ float slab_axpy(const float4 *slab4, const unsigned (&off)[4], unsigned cur,
+                                           const unsigned (&chv)[4], const float (&w)[4], int lane)
+{
+    unsigned ob[4] = { off[0] + cur, off[1] + cur, off[2] + cur, off[3] + cur };
+    keep_here(ob);
+    float o[2][4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        float4 t[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) t[k] = slab4[ob[k] + chv[c]];
+        const float x0 = fmaf(w[0], t[0].x, fmaf(w[1], t[1].x, fmaf(w[2], t[2].x, w[3] * t[3].x)));
+        const float x1 = fmaf(w[0], t[0].y, fmaf(w[1], t[1].y, fmaf(w[2], t[2].y, w[3] * t[3].y)));
+        const float x2 = fmaf(w[0], t[0].z, fmaf(w[1], t[1].z, fmaf(w[2], t[2].z, w[3] * t[3].z)));
+        const float x3 = fmaf(w[0], t[0].w, fmaf(w[1], t[1].w, fmaf(w[2], t[2].w, w[3] * t[3].w)));
+        if (c < 2) {
+            o[c][0] = x0; o[c][1] = x1; o[c][2] = x2; o[c][3] = x3;
+        } else {
+            o[c - 2][0] += dpp_f32<DSDPA_ROW_ROR(14)>(x0);
+            o[c - 2][1] += dpp_f32<DSDPA_ROW_ROR(14)>(x1);
+            o[c - 2][2] += dpp_f32<DSDPA_ROW_ROR(14)>(x2);
+            o[c - 2][3] += dpp_f32<DSDPA_ROW_ROR(14)>(x3);
+        }
+        pin_here(o[c & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[0][e] += dpp_f32<DSDPA_ROW_ROR(1)>(o[1][e]);
+    const bool b8 = (lane & 8) != 0, b4 = (lane & 4) != 0;
+    const float k0 = b8 ? o[0][2] : o[0][0], k1 = b8 ? o[0][3] : o[0][1];
+    const float g0 = b8 ? o[0][0] : o[0][2], g1 = b8 ? o[0][1] : o[0][3];
+    const float h0 = k0 + dpp_f32<DSDPA_ROW_ROR(8)>(g0), h1 = k1 + dpp_f32<DSDPA_ROW_ROR(8)>(g1);
+    const float kk = b4 ? h1 : h0, gg = b4 ? h0 : h1;
+    return kk + dpp_xor4(gg);
+}
+
+// Staging of the slabs: a wave moves runs of 16 pixels of one image row (four lanes per pixel, 16 bytes each), run
+// wave + 16 j of the image's Himg * nxb runs at its step j: where a run starts is the same for all lanes (scalar
+// registers), a lane adds its own place in the run. Offsets inside one (batch, head) fit 32 bits. The slab goes
+// from memory to LDS without passing through registers (global_load_lds_dwordx4: lane i of a wave writes 16 bytes
+// at the wave's LDS base + 16 i, which is the layout of a run); fetch() only issues the loads, wait() -- before the
+// barrier that ends a step -- waits for this wave's.
+struct SlabStager {
+    int pix[kSlabStage], dst[kSlabStage], x0[kSlabStage];       // per wave: scalar registers
+    __device__ __forceinline__ void init(int wave, const Dims &dm, int pitch)
+    {
+        const int nxb = (dm.Wimg + 15) >> 4, nruns = dm.Himg * nxb;
+#pragma unroll
+        for (int j = 0; j < kSlabStage; ++j) {
+            const int run = min(wave + kSlabWaves * j, nruns - 1);           // (a run past the image: the last one once more)
+            const int y = run / nxb, xs = (run - y * nxb) * 16;
+            pix[j] = __builtin_amdgcn_readfirstlane(y * dm.Wimg + xs);
+            dst[j] = __builtin_amdgcn_readfirstlane((y * pitch + xs) * kSlabBytes);
+            x0[j] = __builtin_amdgcn_readfirstlane(xs);
+        }
+    }
+    // columns [col, col + 16) of `plane` into the LDS buffer at byte offset lds_base
+    __device__ __forceinline__ void fetch(const float *plane, int col, unsigned lds_base, int lane, const Dims &dm) const
+    {
+        const float *src = plane + col + (lane & 3) * 4;
+#pragma unroll
+        for (int j = 0; j < kSlabStage; ++j) {
+            if (x0[j] + (lane >> 2) < dm.Wimg) {       // (lanes past the end of the image row stay out)
+                const unsigned px = (unsigned)(pix[j] + (lane >> 2));
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + px * (unsigned)dm.kv_sl),
+                                                 (__attribute__((address_space(3))) void *)(uintptr_t)(lds_base + (unsigned)dst[j]),
+                                                 16, 0, 0);
+            }
+        }
+    }
+    __device__ __forceinline__ static void wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+};
+
+// ------------------------------------------------------------------ forward
 template <int D, int IT>
 __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
     const float *__restrict__ q_, const float *__restrict__ k_, const float *__restrict__ v_,
@@ -74,6 +209,7 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
     constexpr int RB = kSlabWaves * 4 * IT;          // query rows per workgroup
     extern __shared__ __attribute__((aligned(16))) char slab[];
     const float4 *slab4 = reinterpret_cast<const float4 *>(slab);
+    const unsigned slab_base = (unsigned)(uintptr_t)slab;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -121,79 +257,27 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
     float4 qnext = *reinterpret_cast<const float4 *>(qb + qst_off);          // K slab 0 of the first view
     if (lane < 16 * IT) qlds[lane] = qnext;
 
-    // Staging: a wave moves runs of 16 pixels of one image row (four lanes per pixel, 16 bytes each), run
-    // wave + 16 j of the image's Himg * nxb runs at its step j: where a run starts is the same for all lanes (scalar
-    // registers), a lane adds its own place in the run. Offsets inside one (batch, head) fit 32 bits.
-    const int nxb = (dm.Wimg + 15) >> 4, nruns = dm.Himg * nxb;
-    int st_pix[kSlabStage], st_dst[kSlabStage], st_x0[kSlabStage];       // per wave: scalar registers
-#pragma unroll
-    for (int j = 0; j < kSlabStage; ++j) {
-        const int run = min(wave + kSlabWaves * j, nruns - 1);           // (a run past the image: the last one once more)
-        const int y = run / nxb, x0 = (run - y * nxb) * 16;
-        st_pix[j] = __builtin_amdgcn_readfirstlane(y * dm.Wimg + x0);
-        st_dst[j] = __builtin_amdgcn_readfirstlane((y * pitch + x0) * kSlabBytes);
-        st_x0[j] = __builtin_amdgcn_readfirstlane(x0);
-    }
+    SlabStager stg;
+    stg.init(wave, dm, pitch);
     // step ph of the walk: view ph / (2 NSLAB), K slabs first, then V slabs
     const int nsteps = dm.V * 2 * NSLAB;
-    // The slab goes from memory to LDS without passing through registers (global_load_lds_dwordx4: lane i of a wave
-    // writes 16 bytes at the wave's LDS base + 16 i, which is the layout of a run). stage_fetch only issues the
-    // loads; stage_wait, before the barrier that ends a step, waits for this wave's.
     auto stage_fetch = [&](int ph) {
         const int s2 = ph / (2 * NSLAB), r = ph - s2 * (2 * NSLAB);
-        const float *plane = (r < NSLAB ? k_ : v_) + kvb + (size_t)s2 * dm.kv_sv + (r % NSLAB) * kSlabCols + (lane & 3) * 4;
-        const unsigned dst0 = (unsigned)(uintptr_t)slab + (unsigned)(ph & 1) * buf_bytes;
-#pragma unroll
-        for (int j = 0; j < kSlabStage; ++j) {
-            // (lanes past the end of the image row stay out)
-            if (st_x0[j] + (lane >> 2) < dm.Wimg) {
-                const unsigned pix = (unsigned)(st_pix[j] + (lane >> 2));
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void *)(plane + pix * (unsigned)dm.kv_sl),
-                    (__attribute__((address_space(3))) void *)(uintptr_t)(dst0 + (unsigned)st_dst[j]), 16, 0, 0);
-            }
-        }
+        stg.fetch((r < NSLAB ? k_ : v_) + kvb + (size_t)s2 * dm.kv_sv, (r % NSLAB) * kSlabCols,
+                  slab_base + (unsigned)(ph & 1) * buf_bytes, lane, dm);
     };
-    auto stage_wait = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
     stage_fetch(0);
-    stage_wait();
+    SlabStager::wait();
     __syncthreads();
 
     int ph = 0;
     for (int s2 = 0; s2 < dm.V; ++s2) {
-        // this lane's samples of the view: tap rows (in 16-byte units of the slab) and weights, the four taps in
-        // the order that starts in this lane's quarter of the banks
+        // this lane's samples of the view
         unsigned off[IT][4];
         float w[IT][4], part[IT];
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
-            const float2 xy = cb[coff[it] + (unsigned)s2 * (unsigned)dm.P];
-            const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
-            // slab rows of the taps: image row y at y * pitch. The taps 00, 01, 10, 11 of a sample inside the image lie
-            // in the quarters r, r+1, r+2, r+3 (mod 4) with r that of tap 00. A tap outside the image has weight 0 and
-            // may read any row: it reads one of the first four, the one in the quarter it would have had (clamped
-            // into the image it would share a row with its neighbour, and the 16 lanes of a clock would collide).
-            const int n0 = tp.y0 * pitch + tp.x0;
-            const bool vx0 = (unsigned)tp.x0 < (unsigned)dm.Wimg, vx1 = (unsigned)(tp.x0 + 1) < (unsigned)dm.Wimg;
-            const bool vy0 = (unsigned)tp.y0 < (unsigned)dm.Himg, vy1 = (unsigned)(tp.y0 + 1) < (unsigned)dm.Himg;
-            unsigned o[4] = { (unsigned)((vx0 && vy0) ? n0 : (n0 & 3)), (unsigned)((vx1 && vy0) ? n0 + 1 : ((n0 + 1) & 3)),
-                              (unsigned)((vx0 && vy1) ? n0 + pitch : ((n0 + pitch) & 3)),
-                              (unsigned)((vx1 && vy1) ? n0 + pitch + 1 : ((n0 + pitch + 1) & 3)) };
-            float ww[4] = { tp.w[0], tp.w[1], tp.w[2], tp.w[3] };
-            const int rot = (g4 - n0) & 3;                 // read order: tap (k + rot) mod 4 at step k
-            if (rot & 1) {
-                const unsigned t0 = o[0]; o[0] = o[1]; o[1] = o[2]; o[2] = o[3]; o[3] = t0;
-                const float f0 = ww[0]; ww[0] = ww[1]; ww[1] = ww[2]; ww[2] = ww[3]; ww[3] = f0;
-            }
-            if (rot & 2) {
-                const unsigned t0 = o[0], t1 = o[1]; o[0] = o[2]; o[1] = o[3]; o[2] = t0; o[3] = t1;
-                const float f0 = ww[0], f1 = ww[1]; ww[0] = ww[2]; ww[1] = ww[3]; ww[2] = f0; ww[3] = f1;
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                off[it][k] = o[k] * (kSlabBytes / 16);
-                w[it][k] = ww[k];
-            }
+            slab_sample(cb[coff[it] + (unsigned)s2 * (unsigned)dm.P], dm, pitch, g4, off[it], w[it]);
             part[it] = 0.f;
         }
         // ---- logits: K slab by slab
@@ -204,27 +288,11 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
             const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                const float4 *qrow = qlds + (it * 4 + rg) * 4;
-                unsigned ob[4] = { off[it][0] + cur, off[it][1] + cur, off[it][2] + cur, off[it][3] + cur };
-                keep_here(ob);
-                float d[4] = { 0.f, 0.f, 0.f, 0.f };
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const float4 x = qrow[chv[c]];
-                    float4 t[4];
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) t[k] = slab4[ob[k] + chv[c]];
-#pragma unroll
-                    for (int k = 0; k < 4; ++k)
-                        d[k] = fmaf(x.x, t[k].x, fmaf(x.y, t[k].y, fmaf(x.z, t[k].z, fmaf(x.w, t[k].w, d[k]))));
-                    pin_here(d);                      // (the arithmetic on a piece stays next to its reads)
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                part[it] += fmaf(w[it][0], d[0], fmaf(w[it][1], d[1], fmaf(w[it][2], d[2], w[it][3] * d[3])));
+                part[it] += slab_dot(slab4, qlds + (it * 4 + rg) * 4, off[it], cur, chv, w[it]);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (s + 1 < NSLAB && lane < 16 * IT) qlds[lane] = qnext;      // (this wave has read the present piece)
-            stage_wait();
+            SlabStager::wait();
             __syncthreads();
         }
         // ---- softmax bookkeeping of the view; the weights become p * w
@@ -249,45 +317,11 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
             const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                // register c of lane j holds piece (c + j) mod 4: the same piece is in register c + 2 of lane
-                // j + 2 and in register c + 1 of lane j - 1 (lanes mod 16)
-                unsigned ob[4] = { off[it][0] + cur, off[it][1] + cur, off[it][2] + cur, off[it][3] + cur };
-                keep_here(ob);
-                float o[2][4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    float4 t[4];
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) t[k] = slab4[ob[k] + chv[c]];
-                    const float x0 = fmaf(w[it][0], t[0].x, fmaf(w[it][1], t[1].x, fmaf(w[it][2], t[2].x, w[it][3] * t[3].x)));
-                    const float x1 = fmaf(w[it][0], t[0].y, fmaf(w[it][1], t[1].y, fmaf(w[it][2], t[2].y, w[it][3] * t[3].y)));
-                    const float x2 = fmaf(w[it][0], t[0].z, fmaf(w[it][1], t[1].z, fmaf(w[it][2], t[2].z, w[it][3] * t[3].z)));
-                    const float x3 = fmaf(w[it][0], t[0].w, fmaf(w[it][1], t[1].w, fmaf(w[it][2], t[2].w, w[it][3] * t[3].w)));
-                    if (c < 2) {
-                        o[c][0] = x0; o[c][1] = x1; o[c][2] = x2; o[c][3] = x3;
-                    } else {
-                        o[c - 2][0] += dpp_f32<DSDPA_ROW_ROR(14)>(x0);
-                        o[c - 2][1] += dpp_f32<DSDPA_ROW_ROR(14)>(x1);
-                        o[c - 2][2] += dpp_f32<DSDPA_ROW_ROR(14)>(x2);
-                        o[c - 2][3] += dpp_f32<DSDPA_ROW_ROR(14)>(x3);
-                    }
-                    pin_here(o[c & 1]);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[0][e] += dpp_f32<DSDPA_ROW_ROR(1)>(o[1][e]);
-                // piece j mod 4 summed over four lanes; lanes j ^ 8, j ^ 4, j ^ 12 hold the other twelve: two
-                // halving steps leave lane j with column 2 * bit 3 + bit 2 of the piece
-                const bool b8 = (lane & 8) != 0, b4 = (lane & 4) != 0;
-                const float k0 = b8 ? o[0][2] : o[0][0], k1 = b8 ? o[0][3] : o[0][1];
-                const float g0 = b8 ? o[0][0] : o[0][2], g1 = b8 ? o[0][1] : o[0][3];
-                const float h0 = k0 + dpp_f32<DSDPA_ROW_ROR(8)>(g0), h1 = k1 + dpp_f32<DSDPA_ROW_ROR(8)>(g1);
-                const float kk = b4 ? h1 : h0, gg = b4 ? h0 : h1;
-                acc[it][s] += kk + dpp_xor4(gg);
+                acc[it][s] += slab_axpy(slab4, off[it], cur, chv, w[it], lane);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (s == NSLAB - 1 && lane < 16 * IT) qlds[lane] = qnext;
-            stage_wait();
+            SlabStager::wait();
             __syncthreads();
         }
     }
@@ -305,6 +339,183 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
 #pragma unroll
         for (int s = 0; s < NSLAB; ++s) out_[row * D + s * kSlabCols + col] = acc[it][s] * inv;
         if (smp == 0) lse_[row] = m[it] + __log2f(l16);
+    }
+}
+
+// ------------------------------------------------------------------ backward, dq (`ops/triton.py:219-365` computes
+// dq, dk and dv in one kernel; here dk/dv come from the cell-binned kernel, which takes (p, sm_scale * ds) of
+// every sample from this one).
+// Three walks per key view: the K slabs for the logits (q parked in LDS), the V slabs for dp = dout . v~ (dout
+// parked the same way), then p = 2^(s - lse), ds = p (dp - delta), and the K slabs again for dq += ds * k~, the
+// 16 samples of a row combined as in the forward's V walk. Covers the query rows of the (batch, head) pairs
+// [bh0, bh0 + gridDim.x / nblk).
+template <int D, int IT>
+__global__ __launch_bounds__(kSlabWaves *kWave) void bwd_dq_slab_kernel(
+    const float *__restrict__ q_, const float *__restrict__ k_, const float *__restrict__ v_,
+    const float *__restrict__ coords_, const float *__restrict__ out_, const float *__restrict__ lse_,
+    const float *__restrict__ dout_, float *__restrict__ dq_, float2 *__restrict__ stats_,
+    float2 *__restrict__ handed_, Dims dm, int bh0, int nblk, int pitch, unsigned buf_bytes)
+{
+    constexpr int NSLAB = D / kSlabCols;
+    constexpr int RB = kSlabWaves * 4 * IT;
+    extern __shared__ __attribute__((aligned(16))) char slab[];
+    const float4 *slab4 = reinterpret_cast<const float4 *>(slab);
+    const unsigned slab_base = (unsigned)(uintptr_t)slab;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int i3 = lane & 3, g4 = (lane >> 2) & 3, smp = lane & 15, rg = lane >> 4;
+    const int blk = xcd_logical_block(blockIdx.x, gridDim.x);
+    const int bhl = blk / nblk, rb = blk - bhl * nblk, bh = bh0 + bhl;
+    const int b = bh / dm.H, h = bh - b * dm.H;
+    const int VL = dm.V * dm.L;
+    const float *qb = q_ + (size_t)((long long)b * dm.q_sb + (long long)h * dm.q_sh);
+    const size_t kvb = dm.kv_plane(b, 0, h);
+    const float2 *cb = reinterpret_cast<const float2 *>(coords_) + (size_t)b * VL * dm.N;
+    const float qscale = dm.sm_scale * kLog2e;
+    const int col = 4 * i3 + 2 * ((lane >> 3) & 1) + ((lane >> 2) & 1);      // this lane's column of a slab after slab_axpy
+
+    unsigned chv[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) chv[c] = (unsigned)((c + i3) & 3);
+
+    // contiguous row (out, dout, dq, lse) of query row rr of this (batch, head)
+    auto row_of = [&](int rr) {
+        const int s1 = rr / dm.L, l = rr - s1 * dm.L;
+        return (((size_t)b * dm.V + s1) * dm.H + h) * dm.L + l;
+    };
+    bool live[IT];
+    unsigned coff[IT];
+    float lse[IT], delta[IT], acc[IT][NSLAB];
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int rr = rb * RB + (wave * IT + it) * 4 + rg;
+        live[it] = rr < VL;
+        const int rc = min(rr, VL - 1);
+        coff[it] = (unsigned)rc * (unsigned)dm.N + (unsigned)smp;
+        const size_t row = row_of(rc);
+        lse[it] = lse_[row];
+        // delta = dout . out (the reference's _bwd_preprocess, ops/triton.py:197-215): 4 columns a lane
+        float dl = 0.f;
+#pragma unroll
+        for (int j = 0; j < D / 64; ++j) {
+            const float4 a = *reinterpret_cast<const float4 *>(dout_ + row * D + j * 64 + smp * 4);
+            const float4 o = *reinterpret_cast<const float4 *>(out_ + row * D + j * 64 + smp * 4);
+            dl = fmaf(a.x, o.x, fmaf(a.y, o.y, fmaf(a.z, o.z, fmaf(a.w, o.w, dl))));
+        }
+        if constexpr (D < 64) {
+            if (smp < D / 4) {
+                const float4 a = *reinterpret_cast<const float4 *>(dout_ + row * D + smp * 4);
+                const float4 o = *reinterpret_cast<const float4 *>(out_ + row * D + smp * 4);
+                dl = fmaf(a.x, o.x, fmaf(a.y, o.y, fmaf(a.z, o.z, a.w * o.w)));
+            }
+        }
+        delta[it] = group_sum<16>(dl);
+        if (stats_ && live[it] && smp == 0) stats_[row] = make_float2(lse[it], delta[it]);
+#pragma unroll
+        for (int s = 0; s < NSLAB; ++s) acc[it][s] = 0.f;
+    }
+
+    // q and dout through LDS, a slab ahead (see the forward): lane i moves piece i & 3 of the wave's row i >> 2
+    float4 *xlds = reinterpret_cast<float4 *>(slab + 2 * buf_bytes) + wave * (4 * IT * 4);
+    unsigned qst_off;
+    size_t dst_off;
+    {
+        const int rc = min(rb * RB + wave * (4 * IT) + min(lane >> 2, 4 * IT - 1), VL - 1);
+        const int s1 = rc / dm.L, l = rc - s1 * dm.L;
+        qst_off = (unsigned)s1 * (unsigned)dm.q_sv + (unsigned)l * (unsigned)dm.q_sl + (unsigned)(lane & 3) * 4;
+        dst_off = row_of(rc) * D + (size_t)(lane & 3) * 4;
+    }
+    float4 xnext = *reinterpret_cast<const float4 *>(qb + qst_off);
+    if (lane < 16 * IT) xlds[lane] = xnext;
+
+    SlabStager stg;
+    stg.init(wave, dm, pitch);
+    // step ph of the walk: view ph / (3 NSLAB): K slabs, V slabs, K slabs
+    const int nsteps = dm.V * 3 * NSLAB;
+    auto stage_fetch = [&](int ph) {
+        const int s2 = ph / (3 * NSLAB), r = ph - s2 * (3 * NSLAB);
+        stg.fetch(((r >= NSLAB && r < 2 * NSLAB) ? v_ : k_) + kvb + (size_t)s2 * dm.kv_sv, (r % NSLAB) * kSlabCols,
+                  slab_base + (unsigned)(ph & 1) * buf_bytes, lane, dm);
+    };
+    stage_fetch(0);
+    SlabStager::wait();
+    __syncthreads();
+
+    int ph = 0;
+    for (int s2 = 0; s2 < dm.V; ++s2) {
+        unsigned off[IT][4];
+        float w[IT][4], ps[IT], pd[IT];
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            slab_sample(cb[coff[it] + (unsigned)s2 * (unsigned)dm.P], dm, pitch, g4, off[it], w[it]);
+            ps[it] = 0.f;
+            pd[it] = 0.f;
+        }
+        // ---- logits: K slabs, q parked
+#pragma unroll 1
+        for (int s = 0; s < NSLAB; ++s, ++ph) {
+            xnext = (s + 1 < NSLAB) ? *reinterpret_cast<const float4 *>(qb + qst_off + (s + 1) * kSlabCols)
+                                    : *reinterpret_cast<const float4 *>(dout_ + dst_off);
+            stage_fetch(ph + 1);
+            const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
+#pragma unroll
+            for (int it = 0; it < IT; ++it) {
+                ps[it] += slab_dot(slab4, xlds + (it * 4 + rg) * 4, off[it], cur, chv, w[it]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (lane < 16 * IT) xlds[lane] = xnext;
+            SlabStager::wait();
+            __syncthreads();
+        }
+        // ---- dp = dout . v~: V slabs, dout parked
+#pragma unroll 1
+        for (int s = 0; s < NSLAB; ++s, ++ph) {
+            if (s + 1 < NSLAB) xnext = *reinterpret_cast<const float4 *>(dout_ + dst_off + (s + 1) * kSlabCols);
+            stage_fetch(ph + 1);
+            const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
+#pragma unroll
+            for (int it = 0; it < IT; ++it) {
+                pd[it] += slab_dot(slab4, xlds + (it * 4 + rg) * 4, off[it], cur, chv, w[it]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (s + 1 < NSLAB && lane < 16 * IT) xlds[lane] = xnext;
+            SlabStager::wait();
+            __syncthreads();
+        }
+        // ---- p, ds; the pair goes to the dk/dv kernel ([pair of this launch][s1][l][sample]); the weights become ds * w
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const float p = __builtin_amdgcn_exp2f(ps[it] * qscale - lse[it]);
+            const float ds = p * (pd[it] - delta[it]);
+            if (handed_ && live[it])
+                handed_[(size_t)bhl * VL * dm.N + coff[it] + (unsigned)s2 * (unsigned)dm.P] = make_float2(p, ds * dm.sm_scale);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) w[it][t] *= ds;
+        }
+        // ---- dq += ds * k~: K slabs again
+#pragma unroll
+        for (int s = 0; s < NSLAB; ++s, ++ph) {
+            if (s == NSLAB - 1) xnext = *reinterpret_cast<const float4 *>(qb + qst_off);      // the next view starts with q, slab 0
+            if (ph + 1 < nsteps) stage_fetch(ph + 1);
+            const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
+#pragma unroll
+            for (int it = 0; it < IT; ++it) {
+                acc[it][s] += slab_axpy(slab4, off[it], cur, chv, w[it], lane);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (s == NSLAB - 1 && lane < 16 * IT) xlds[lane] = xnext;
+            SlabStager::wait();
+            __syncthreads();
+        }
+    }
+
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        if (!live[it]) continue;
+        const size_t row = row_of(rb * RB + (wave * IT + it) * 4 + rg);
+#pragma unroll
+        for (int s = 0; s < NSLAB; ++s) dq_[row * D + s * kSlabCols + col] = acc[it][s] * dm.sm_scale;
     }
 }
 
