@@ -114,7 +114,8 @@ def test_staged_forward_two_row_blocks(dtype):
 
 
 # fp32 storage, 16 samples per view, planes too large for LDS but small enough for two 16-column slabs of the whole
-# image: the forward walks the planes slab by slab through LDS (fwd_slab_kernel), every tap read from there.
+# image: the forward and the dq kernel walk the planes slab by slab through LDS (fwd_slab_kernel,
+# bwd_dq_slab_kernel), every tap read from there.
 SLABS = [
     # seed B  V  H  Himg Wimg D    lo     hi
     (81, 1, 2, 2, 20, 20, 64, -0.1, 1.1),       # width a multiple of 4: two padding columns per image row; 800 query rows: 4 full workgroups and a part
@@ -122,6 +123,9 @@ SLABS = [
     (83, 1, 2, 2, 17, 17, 128, 0.0, 1.0),       # eight slabs per plane
     (84, 1, 1, 3, 20, 32, 32, -0.05, 1.05),     # two slabs per plane, one view
     (85, 1, 2, 1, 32, 32, 64, -0.1, 1.1),       # the largest image the kernel takes (64 runs)
+    (86, 1, 1, 2, 21, 48, 64, -0.1, 1.1),       # three runs per image row, 63 runs
+    (87, 1, 2, 1, 40, 16, 64, 0.0, 1.0),        # one run per image row, tall image
+    (88, 1, 2, 1, 16, 17, 128, -0.2, 1.2),      # second run of a row holds one pixel
 ]
 
 
@@ -146,7 +150,7 @@ def test_slab_forward_vs_oracle(case):
     assert torch.isfinite(out).all()
     assert rel(out, ro) < TOL_FWD[dtype]
     assert rel(out, og.cpu().numpy()) < TOL_FWD[dtype]
-    assert rel(dq, rdq) < TOL_BWD[dtype]                   # (lse of the slab forward feeds the backward)
+    assert rel(dq, rdq) < TOL_BWD[dtype]                   # (dq by the slab kernel, dk/dv from the pairs it hands over)
     assert rel(dk, rdk) < TOL_BWD[dtype]
     assert rel(dv, rdv) < TOL_BWD[dtype]
 
