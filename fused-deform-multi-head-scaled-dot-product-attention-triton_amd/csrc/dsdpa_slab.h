@@ -24,9 +24,7 @@ namespace dsdpa {
 
 constexpr int kSlabBytes = 64;             // bytes of one pixel in a slab: 16 fp32 columns
 constexpr int kSlabCols = 16;
-constexpr int kSlabWaves = 16;
 constexpr int kSlabSamples = 16;           // samples per (query row, view) this kernel is written for
-constexpr int kSlabStage = 4;              // runs of 16 pixels of an image row a wave moves per slab
 
 // slab rows between two image rows: the width rounded up to 2 mod 4
 __host__ __device__ inline int slab_pitch(int Wimg) { return Wimg + ((6 - (Wimg & 3)) & 3); }
@@ -167,14 +165,16 @@ __device__ __forceinline__ float slab_axpy(const float4 *slab4, const unsigned (
 // from memory to LDS without passing through registers (global_load_lds_dwordx4: lane i of a wave writes 16 bytes
 // at the wave's LDS base + 16 i, which is the layout of a run); fetch() only issues the loads, wait() -- before the
 // barrier that ends a step -- waits for this wave's.
+template <int NW>
 struct SlabStager {
-    int pix[kSlabStage], dst[kSlabStage], x0[kSlabStage];       // per wave: scalar registers
+    static constexpr int kStage = (64 + NW - 1) / NW;       // runs of 16 pixels a wave moves per slab (an image has at most 64)
+    int pix[kStage], dst[kStage], x0[kStage];       // per wave: scalar registers
     __device__ __forceinline__ void init(int wave, const Dims &dm, int pitch)
     {
         const int nxb = (dm.Wimg + 15) >> 4, nruns = dm.Himg * nxb;
 #pragma unroll
-        for (int j = 0; j < kSlabStage; ++j) {
-            const int run = min(wave + kSlabWaves * j, nruns - 1);           // (a run past the image: the last one once more)
+        for (int j = 0; j < kStage; ++j) {
+            const int run = min(wave + NW * j, nruns - 1);           // (a run past the image: the last one once more)
             const int y = run / nxb, xs = (run - y * nxb) * 16;
             pix[j] = __builtin_amdgcn_readfirstlane(y * dm.Wimg + xs);
             dst[j] = __builtin_amdgcn_readfirstlane((y * pitch + xs) * kSlabBytes);
@@ -186,7 +186,7 @@ struct SlabStager {
     {
         const float *src = plane + col + (lane & 3) * 4;
 #pragma unroll
-        for (int j = 0; j < kSlabStage; ++j) {
+        for (int j = 0; j < kStage; ++j) {
             if (x0[j] + (lane >> 2) < dm.Wimg) {       // (lanes past the end of the image row stay out)
                 const unsigned px = (unsigned)(pix[j] + (lane >> 2));
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + px * (unsigned)dm.kv_sl),
@@ -199,14 +199,14 @@ struct SlabStager {
 };
 
 // ------------------------------------------------------------------ forward
-template <int D, int IT>
-__global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
+template <int D, int IT, int NW>
+__global__ __launch_bounds__(NW *kWave) void fwd_slab_kernel(
     const float *__restrict__ q_, const float *__restrict__ k_, const float *__restrict__ v_,
     const float *__restrict__ coords_, float *__restrict__ out_, float *__restrict__ lse_, Dims dm, int nblk,
     int pitch, unsigned buf_bytes)
 {
     constexpr int NSLAB = D / kSlabCols;
-    constexpr int RB = kSlabWaves * 4 * IT;          // query rows per workgroup
+    constexpr int RB = NW * 4 * IT;                  // query rows per workgroup
     extern __shared__ __attribute__((aligned(16))) char slab[];
     const float4 *slab4 = reinterpret_cast<const float4 *>(slab);
     const unsigned slab_base = (unsigned)(uintptr_t)slab;
@@ -257,7 +257,7 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
     float4 qnext = *reinterpret_cast<const float4 *>(qb + qst_off);          // K slab 0 of the first view
     if (lane < 16 * IT) qlds[lane] = qnext;
 
-    SlabStager stg;
+    SlabStager<NW> stg;
     stg.init(wave, dm, pitch);
     // step ph of the walk: view ph / (2 NSLAB), K slabs first, then V slabs
     const int nsteps = dm.V * 2 * NSLAB;
@@ -267,7 +267,7 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
                   slab_base + (unsigned)(ph & 1) * buf_bytes, lane, dm);
     };
     stage_fetch(0);
-    SlabStager::wait();
+    SlabStager<NW>::wait();
     __syncthreads();
 
     int ph = 0;
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (s + 1 < NSLAB && lane < 16 * IT) qlds[lane] = qnext;      // (this wave has read the present piece)
-            SlabStager::wait();
+            SlabStager<NW>::wait();
             __syncthreads();
         }
         // ---- softmax bookkeeping of the view; the weights become p * w
@@ -321,7 +321,7 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (s == NSLAB - 1 && lane < 16 * IT) qlds[lane] = qnext;
-            SlabStager::wait();
+            SlabStager<NW>::wait();
             __syncthreads();
         }
     }
@@ -349,15 +349,15 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void fwd_slab_kernel(
 // parked the same way), then p = 2^(s - lse), ds = p (dp - delta), and the K slabs again for dq += ds * k~, the
 // 16 samples of a row combined as in the forward's V walk. Covers the query rows of the (batch, head) pairs
 // [bh0, bh0 + gridDim.x / nblk).
-template <int D, int IT>
-__global__ __launch_bounds__(kSlabWaves *kWave) void bwd_dq_slab_kernel(
+template <int D, int IT, int NW>
+__global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
     const float *__restrict__ q_, const float *__restrict__ k_, const float *__restrict__ v_,
     const float *__restrict__ coords_, const float *__restrict__ out_, const float *__restrict__ lse_,
     const float *__restrict__ dout_, float *__restrict__ dq_, float2 *__restrict__ stats_,
     float2 *__restrict__ handed_, Dims dm, int bh0, int nblk, int pitch, unsigned buf_bytes)
 {
     constexpr int NSLAB = D / kSlabCols;
-    constexpr int RB = kSlabWaves * 4 * IT;
+    constexpr int RB = NW * 4 * IT;
     extern __shared__ __attribute__((aligned(16))) char slab[];
     const float4 *slab4 = reinterpret_cast<const float4 *>(slab);
     const unsigned slab_base = (unsigned)(uintptr_t)slab;
@@ -429,7 +429,7 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void bwd_dq_slab_kernel(
     float4 xnext = *reinterpret_cast<const float4 *>(qb + qst_off);
     if (lane < 16 * IT) xlds[lane] = xnext;
 
-    SlabStager stg;
+    SlabStager<NW> stg;
     stg.init(wave, dm, pitch);
     // step ph of the walk: view ph / (3 NSLAB): K slabs, V slabs, K slabs
     const int nsteps = dm.V * 3 * NSLAB;
@@ -439,7 +439,7 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void bwd_dq_slab_kernel(
                   slab_base + (unsigned)(ph & 1) * buf_bytes, lane, dm);
     };
     stage_fetch(0);
-    SlabStager::wait();
+    SlabStager<NW>::wait();
     __syncthreads();
 
     int ph = 0;
@@ -465,7 +465,7 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void bwd_dq_slab_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (lane < 16 * IT) xlds[lane] = xnext;
-            SlabStager::wait();
+            SlabStager<NW>::wait();
             __syncthreads();
         }
         // ---- dp = dout . v~: V slabs, dout parked
@@ -480,7 +480,7 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void bwd_dq_slab_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (s + 1 < NSLAB && lane < 16 * IT) xlds[lane] = xnext;
-            SlabStager::wait();
+            SlabStager<NW>::wait();
             __syncthreads();
         }
         // ---- p, ds; the pair goes to the dk/dv kernel ([pair of this launch][s1][l][sample]); the weights become ds * w
@@ -505,7 +505,7 @@ __global__ __launch_bounds__(kSlabWaves *kWave) void bwd_dq_slab_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (s == NSLAB - 1 && lane < 16 * IT) xlds[lane] = xnext;
-            SlabStager::wait();
+            SlabStager<NW>::wait();
             __syncthreads();
         }
     }
