@@ -173,7 +173,7 @@ inline DenseLayout dense_layout(size_t B, size_t V, size_t H, size_t Himg, size_
     return d;
 }
 
-// Slab forward (fwd_slab_kernel): fp32 storage, 16 samples per view, planes that do not fit in LDS whole but do,
+// Slab kernels (fwd_slab_kernel, bwd_dq_slab_kernel): fp32 storage, 16 or 32 samples per view, planes that do not fit in LDS whole but do,
 // twice, as slabs of 16 columns (64 bytes per pixel, image rows at a pitch of 2 mod 4 pixels), at most 1024 pixels,
 // query rows of a (batch, head) within 31 bits of coordinate pairs. Needs no workspace.
 inline size_t slab_buffer_bytes(size_t Himg, size_t Wimg)
@@ -185,7 +185,8 @@ inline bool slab_path_fits(size_t V, size_t Himg, size_t Wimg, size_t D, size_t 
 {
     const size_t L = Himg * Wimg;
     // (a wave stages runs of 16 pixels of an image row, four per slab)
-    return esize == 4 && P == 16 && (D == 32 || D == 64 || D == 128) && Himg * ((Wimg + 15) / 16) <= 64 &&
+    // (64 samples per view go to the gather kernels, whose window mode pays where the samples cluster)
+    return esize == 4 && (P == 16 || P == 32) && (D == 32 || D == 64 || D == 128) && Himg * ((Wimg + 15) / 16) <= 64 &&
            2 * slab_buffer_bytes(Himg, Wimg) + 12 * 1024 <= kLdsBytes && !plane_path_fits(L, D, esize) &&
            V * L * V * P < ((size_t)1 << 31);
 }

@@ -177,13 +177,14 @@ int launch_fwd_slab(const void *q, const void *k, const void *v, const float *co
         return DSDPA_ERR_UNSUPPORTED;
     } else {
         constexpr int IT = kSlabItems, NW = kSlabWaves;
-        constexpr int RB = NW * 4 * IT;
+        const int kb = dm.P / kSlabSamples;                  // 1 or 2 (slab_path_fits)
+        const int RB = NW * 4 * IT / kb;
         const int nblk = (dm.V * dm.L + RB - 1) / RB;
         const long long blocks = (long long)dm.B * dm.H * nblk;
         if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
-        auto kern = fwd_slab_kernel<D, IT, NW>;
-        static std::atomic<unsigned long long> lds_set{0};
-        if (int rc = allow_full_lds(kern, lds_set)) return rc;
+        auto kern = kb == 1 ? fwd_slab_kernel<D, IT, NW, 1> : fwd_slab_kernel<D, IT, NW, 2>;
+        static std::atomic<unsigned long long> lds_set[2];
+        if (int rc = allow_full_lds(kern, lds_set[kb >> 1])) return rc;
         ScopedKernelTimer timer(0, st);
         const unsigned buf_bytes = (unsigned)slab_buffer_bytes(dm.Himg, dm.Wimg);
         DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(NW * kWave), (size_t)2 * buf_bytes + NW * 4 * IT * kSlabBytes, st, timer.start(),
@@ -203,13 +204,14 @@ int launch_bwd_dq_slab(const void *q, const void *k, const void *v, const float 
         return DSDPA_ERR_UNSUPPORTED;
     } else {
         constexpr int IT = kSlabItems, NW = kSlabWaves;
-        constexpr int RB = NW * 4 * IT;
+        const int kb = dm.P / kSlabSamples;
+        const int RB = NW * 4 * IT / kb;
         const int nblk = (dm.V * dm.L + RB - 1) / RB;
         const long long blocks = (long long)nbh * nblk;
         if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
-        auto kern = bwd_dq_slab_kernel<D, IT, NW>;
-        static std::atomic<unsigned long long> lds_set{0};
-        if (int rc = allow_full_lds(kern, lds_set)) return rc;
+        auto kern = kb == 1 ? bwd_dq_slab_kernel<D, IT, NW, 1> : bwd_dq_slab_kernel<D, IT, NW, 2>;
+        static std::atomic<unsigned long long> lds_set[2];
+        if (int rc = allow_full_lds(kern, lds_set[kb >> 1])) return rc;
         ScopedKernelTimer timer(2, st);
         const unsigned buf_bytes = (unsigned)slab_buffer_bytes(dm.Himg, dm.Wimg);
         DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(NW * kWave), (size_t)2 * buf_bytes + NW * 4 * IT * kSlabBytes, st,

@@ -1,4 +1,4 @@
-// Forward for fp32 storage and 16 samples per view on images whose K/V planes do not fit in LDS but whose planes
+// Forward and dq for fp32 storage and 16 or 32 samples per view on images whose K/V planes do not fit in LDS but whose planes
 // cut to 16 columns do, twice: "slabs" of 64 bytes per pixel (`ops/triton.py:118-170` is the sampling and softmax
 // loop this replaces; the reference gathers every tap from global memory).
 //
@@ -24,7 +24,7 @@ namespace dsdpa {
 
 constexpr int kSlabBytes = 64;             // bytes of one pixel in a slab: 16 fp32 columns
 constexpr int kSlabCols = 16;
-constexpr int kSlabSamples = 16;           // samples per (query row, view) this kernel is written for
+constexpr int kSlabSamples = 16;           // samples of a (query row, view) per block: the 16 lanes of a DPP row
 
 // slab rows between two image rows: the width rounded up to 2 mod 4
 __host__ __device__ inline int slab_pitch(int Wimg) { return Wimg + ((6 - (Wimg & 3)) & 3); }
@@ -199,14 +199,20 @@ struct SlabStager {
 };
 
 // ------------------------------------------------------------------ forward
-template <int D, int IT, int NW>
+// KB: blocks of 16 samples per (query row, view), P = 16 KB. A lane's IT samples of a view are the KB blocks of IT / KB
+// query rows: the blocks of one row sit in the same 16 lanes, so what a row's blocks share (running maximum, sum,
+// output columns) is combined inside a lane.
+template <int D, int IT, int NW, int KB>
 __global__ __launch_bounds__(NW *kWave) void fwd_slab_kernel(
     const float *__restrict__ q_, const float *__restrict__ k_, const float *__restrict__ v_,
     const float *__restrict__ coords_, float *__restrict__ out_, float *__restrict__ lse_, Dims dm, int nblk,
     int pitch, unsigned buf_bytes)
 {
     constexpr int NSLAB = D / kSlabCols;
-    constexpr int RB = NW * 4 * IT;                  // query rows per workgroup
+    constexpr int NR = IT / KB;                      // query rows a lane works on
+    constexpr int RW = 4 * NR;                       // query rows per wave
+    constexpr int RB = NW * RW;                      // query rows per workgroup
+    static_assert(NR * KB == IT, "whole rows per lane");
     extern __shared__ __attribute__((aligned(16))) char slab[];
     const float4 *slab4 = reinterpret_cast<const float4 *>(slab);
     const unsigned slab_base = (unsigned)(uintptr_t)slab;
@@ -228,34 +234,36 @@ __global__ __launch_bounds__(NW *kWave) void fwd_slab_kernel(
 #pragma unroll
     for (int c = 0; c < 4; ++c) chv[c] = (unsigned)((c + i3) & 3);
 
-    bool live[IT];
-    unsigned coff[IT];
-    float m[IT], lsum[IT], acc[IT][NSLAB];
+    // row r of this lane: query row rb * RB + wave * RW + 4 r + rg of the (batch, head); sample it: block it % KB of
+    // row it / KB
+    bool live[NR];
+    unsigned coff[NR];
+    float m[NR], lsum[NR], acc[NR][NSLAB];
 #pragma unroll
-    for (int it = 0; it < IT; ++it) {
-        const int rr = rb * RB + (wave * IT + it) * 4 + rg;
-        live[it] = rr < VL;
+    for (int r = 0; r < NR; ++r) {
+        const int rr = rb * RB + wave * RW + 4 * r + rg;
+        live[r] = rr < VL;
         const int rc = min(rr, VL - 1);
-        coff[it] = (unsigned)rc * (unsigned)dm.N + (unsigned)smp;
-        m[it] = kNegBig;
-        lsum[it] = 0.f;
+        coff[r] = (unsigned)rc * (unsigned)dm.N + (unsigned)smp;
+        m[r] = kNegBig;
+        lsum[r] = 0.f;
 #pragma unroll
-        for (int s = 0; s < NSLAB; ++s) acc[it][s] = 0.f;
+        for (int s = 0; s < NSLAB; ++s) acc[r][s] = 0.f;
     }
 
-    // q goes through LDS too, 16 columns of the wave's 4 * IT rows at a time (a region per wave: no barrier): a load
+    // q goes through LDS too, 16 columns of the wave's RW rows at a time (a region per wave: no barrier): a load
     // issued behind the slab's loads would only return after them (loads return in order), at the start of
     // every K step. The piece for the next K step is requested before that step's slab and parked after the work
     // on the present step; lane i moves piece i & 3 of row i >> 2.
-    float4 *qlds = reinterpret_cast<float4 *>(slab + 2 * buf_bytes) + wave * (4 * IT * 4);
+    float4 *qlds = reinterpret_cast<float4 *>(slab + 2 * buf_bytes) + wave * (RW * 4);
     unsigned qst_off;
     {
-        const int rc = min(rb * RB + wave * (4 * IT) + min(lane >> 2, 4 * IT - 1), VL - 1);
+        const int rc = min(rb * RB + wave * RW + min(lane >> 2, RW - 1), VL - 1);
         const int s1 = rc / dm.L, l = rc - s1 * dm.L;
         qst_off = (unsigned)s1 * (unsigned)dm.q_sv + (unsigned)l * (unsigned)dm.q_sl + (unsigned)(lane & 3) * 4;
     }
     float4 qnext = *reinterpret_cast<const float4 *>(qb + qst_off);          // K slab 0 of the first view
-    if (lane < 16 * IT) qlds[lane] = qnext;
+    if (lane < 4 * RW) qlds[lane] = qnext;
 
     SlabStager<NW> stg;
     stg.init(wave, dm, pitch);
@@ -277,7 +285,8 @@ __global__ __launch_bounds__(NW *kWave) void fwd_slab_kernel(
         float w[IT][4], part[IT];
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
-            slab_sample(cb[coff[it] + (unsigned)s2 * (unsigned)dm.P], dm, pitch, g4, off[it], w[it]);
+            slab_sample(cb[coff[it / KB] + (unsigned)s2 * (unsigned)dm.P + (unsigned)(it % KB) * kSlabSamples], dm, pitch, g4,
+                        off[it], w[it]);
             part[it] = 0.f;
         }
         // ---- logits: K slab by slab
@@ -288,26 +297,33 @@ __global__ __launch_bounds__(NW *kWave) void fwd_slab_kernel(
             const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                part[it] += slab_dot(slab4, qlds + (it * 4 + rg) * 4, off[it], cur, chv, w[it]);
+                part[it] += slab_dot(slab4, qlds + ((it / KB) * 4 + rg) * 4, off[it], cur, chv, w[it]);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (s + 1 < NSLAB && lane < 16 * IT) qlds[lane] = qnext;      // (this wave has read the present piece)
+            if (s + 1 < NSLAB && lane < 4 * RW) qlds[lane] = qnext;      // (this wave has read the present piece)
             SlabStager<NW>::wait();
             __syncthreads();
         }
-        // ---- softmax bookkeeping of the view; the weights become p * w
+        // ---- softmax bookkeeping of the view, row by row; the weights become p * w
 #pragma unroll
-        for (int it = 0; it < IT; ++it) {
-            const float sc = part[it] * qscale;
-            const float m_new = fmaxf(m[it], group16_max(sc));
-            const float alpha = __builtin_amdgcn_exp2f(m[it] - m_new);
-            const float p = __builtin_amdgcn_exp2f(sc - m_new);
-            m[it] = m_new;
-            lsum[it] = fmaf(lsum[it], alpha, p);
+        for (int r = 0; r < NR; ++r) {
+            float mx = kNegBig;
 #pragma unroll
-            for (int s = 0; s < NSLAB; ++s) acc[it][s] *= alpha;
+            for (int kb = 0; kb < KB; ++kb) mx = fmaxf(mx, part[r * KB + kb] * qscale);
+            const float m_new = fmaxf(m[r], group16_max(mx));
+            const float alpha = __builtin_amdgcn_exp2f(m[r] - m_new);
+            m[r] = m_new;
+            lsum[r] *= alpha;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) w[it][t] *= p;
+            for (int s = 0; s < NSLAB; ++s) acc[r][s] *= alpha;
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const int it = r * KB + kb;
+                const float p = __builtin_amdgcn_exp2f(part[it] * qscale - m_new);
+                lsum[r] += p;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) w[it][t] *= p;
+            }
         }
         // ---- out: V slab by slab
 #pragma unroll
@@ -317,10 +333,10 @@ __global__ __launch_bounds__(NW *kWave) void fwd_slab_kernel(
             const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                acc[it][s] += slab_axpy(slab4, off[it], cur, chv, w[it], lane);
+                acc[it / KB][s] += slab_axpy(slab4, off[it], cur, chv, w[it], lane);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (s == NSLAB - 1 && lane < 16 * IT) qlds[lane] = qnext;
+            if (s == NSLAB - 1 && lane < 4 * RW) qlds[lane] = qnext;
             SlabStager<NW>::wait();
             __syncthreads();
         }
@@ -328,17 +344,17 @@ __global__ __launch_bounds__(NW *kWave) void fwd_slab_kernel(
 
     // ---- epilogue: lane j of a row's 16 lanes holds column 16 s + 4 (j & 3) + 2 * bit 3 + bit 2 of the row
 #pragma unroll
-    for (int it = 0; it < IT; ++it) {
-        const float l16 = group_sum<16>(lsum[it]);
-        if (!live[it]) continue;
-        const int rr = rb * RB + (wave * IT + it) * 4 + rg;
+    for (int r = 0; r < NR; ++r) {
+        const float l16 = group_sum<16>(lsum[r]);
+        if (!live[r]) continue;
+        const int rr = rb * RB + wave * RW + 4 * r + rg;
         const int s1 = rr / dm.L, l = rr - s1 * dm.L;
         const size_t row = (((size_t)b * dm.V + s1) * dm.H + h) * dm.L + l;
         const float inv = 1.0f / l16;
         const int col = 4 * i3 + 2 * ((lane >> 3) & 1) + ((lane >> 2) & 1);
 #pragma unroll
-        for (int s = 0; s < NSLAB; ++s) out_[row * D + s * kSlabCols + col] = acc[it][s] * inv;
-        if (smp == 0) lse_[row] = m[it] + __log2f(l16);
+        for (int s = 0; s < NSLAB; ++s) out_[row * D + s * kSlabCols + col] = acc[r][s] * inv;
+        if (smp == 0) lse_[row] = m[r] + __log2f(l16);
     }
 }
 
@@ -349,7 +365,7 @@ __global__ __launch_bounds__(NW *kWave) void fwd_slab_kernel(
 // parked the same way), then p = 2^(s - lse), ds = p (dp - delta), and the K slabs again for dq += ds * k~, the
 // 16 samples of a row combined as in the forward's V walk. Covers the query rows of the (batch, head) pairs
 // [bh0, bh0 + gridDim.x / nblk).
-template <int D, int IT, int NW>
+template <int D, int IT, int NW, int KB>
 __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
     const float *__restrict__ q_, const float *__restrict__ k_, const float *__restrict__ v_,
     const float *__restrict__ coords_, const float *__restrict__ out_, const float *__restrict__ lse_,
@@ -357,7 +373,8 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
     float2 *__restrict__ handed_, Dims dm, int bh0, int nblk, int pitch, unsigned buf_bytes)
 {
     constexpr int NSLAB = D / kSlabCols;
-    constexpr int RB = NW * 4 * IT;
+    constexpr int NR = IT / KB, RW = 4 * NR, RB = NW * RW;       // query rows per lane, wave, workgroup (see the forward)
+    static_assert(NR * KB == IT, "whole rows per lane");
     extern __shared__ __attribute__((aligned(16))) char slab[];
     const float4 *slab4 = reinterpret_cast<const float4 *>(slab);
     const unsigned slab_base = (unsigned)(uintptr_t)slab;
@@ -384,17 +401,17 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
         const int s1 = rr / dm.L, l = rr - s1 * dm.L;
         return (((size_t)b * dm.V + s1) * dm.H + h) * dm.L + l;
     };
-    bool live[IT];
-    unsigned coff[IT];
-    float lse[IT], delta[IT], acc[IT][NSLAB];
+    bool live[NR];
+    unsigned coff[NR];
+    float lse[NR], delta[NR], acc[NR][NSLAB];
 #pragma unroll
-    for (int it = 0; it < IT; ++it) {
-        const int rr = rb * RB + (wave * IT + it) * 4 + rg;
-        live[it] = rr < VL;
+    for (int r = 0; r < NR; ++r) {
+        const int rr = rb * RB + wave * RW + 4 * r + rg;
+        live[r] = rr < VL;
         const int rc = min(rr, VL - 1);
-        coff[it] = (unsigned)rc * (unsigned)dm.N + (unsigned)smp;
+        coff[r] = (unsigned)rc * (unsigned)dm.N + (unsigned)smp;
         const size_t row = row_of(rc);
-        lse[it] = lse_[row];
+        lse[r] = lse_[row];
         // delta = dout . out (the reference's _bwd_preprocess, ops/triton.py:197-215): 4 columns a lane
         float dl = 0.f;
 #pragma unroll
@@ -410,24 +427,24 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
                 dl = fmaf(a.x, o.x, fmaf(a.y, o.y, fmaf(a.z, o.z, a.w * o.w)));
             }
         }
-        delta[it] = group_sum<16>(dl);
-        if (stats_ && live[it] && smp == 0) stats_[row] = make_float2(lse[it], delta[it]);
+        delta[r] = group_sum<16>(dl);
+        if (stats_ && live[r] && smp == 0) stats_[row] = make_float2(lse[r], delta[r]);
 #pragma unroll
-        for (int s = 0; s < NSLAB; ++s) acc[it][s] = 0.f;
+        for (int s = 0; s < NSLAB; ++s) acc[r][s] = 0.f;
     }
 
     // q and dout through LDS, a slab ahead (see the forward): lane i moves piece i & 3 of the wave's row i >> 2
-    float4 *xlds = reinterpret_cast<float4 *>(slab + 2 * buf_bytes) + wave * (4 * IT * 4);
+    float4 *xlds = reinterpret_cast<float4 *>(slab + 2 * buf_bytes) + wave * (RW * 4);
     unsigned qst_off;
     size_t dst_off;
     {
-        const int rc = min(rb * RB + wave * (4 * IT) + min(lane >> 2, 4 * IT - 1), VL - 1);
+        const int rc = min(rb * RB + wave * RW + min(lane >> 2, RW - 1), VL - 1);
         const int s1 = rc / dm.L, l = rc - s1 * dm.L;
         qst_off = (unsigned)s1 * (unsigned)dm.q_sv + (unsigned)l * (unsigned)dm.q_sl + (unsigned)(lane & 3) * 4;
         dst_off = row_of(rc) * D + (size_t)(lane & 3) * 4;
     }
     float4 xnext = *reinterpret_cast<const float4 *>(qb + qst_off);
-    if (lane < 16 * IT) xlds[lane] = xnext;
+    if (lane < 4 * RW) xlds[lane] = xnext;
 
     SlabStager<NW> stg;
     stg.init(wave, dm, pitch);
@@ -448,7 +465,8 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
         float w[IT][4], ps[IT], pd[IT];
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
-            slab_sample(cb[coff[it] + (unsigned)s2 * (unsigned)dm.P], dm, pitch, g4, off[it], w[it]);
+            slab_sample(cb[coff[it / KB] + (unsigned)s2 * (unsigned)dm.P + (unsigned)(it % KB) * kSlabSamples], dm, pitch, g4,
+                        off[it], w[it]);
             ps[it] = 0.f;
             pd[it] = 0.f;
         }
@@ -461,10 +479,10 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
             const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                ps[it] += slab_dot(slab4, xlds + (it * 4 + rg) * 4, off[it], cur, chv, w[it]);
+                ps[it] += slab_dot(slab4, xlds + ((it / KB) * 4 + rg) * 4, off[it], cur, chv, w[it]);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (lane < 16 * IT) xlds[lane] = xnext;
+            if (lane < 4 * RW) xlds[lane] = xnext;
             SlabStager<NW>::wait();
             __syncthreads();
         }
@@ -476,20 +494,22 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
             const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                pd[it] += slab_dot(slab4, xlds + (it * 4 + rg) * 4, off[it], cur, chv, w[it]);
+                pd[it] += slab_dot(slab4, xlds + ((it / KB) * 4 + rg) * 4, off[it], cur, chv, w[it]);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (s + 1 < NSLAB && lane < 16 * IT) xlds[lane] = xnext;
+            if (s + 1 < NSLAB && lane < 4 * RW) xlds[lane] = xnext;
             SlabStager<NW>::wait();
             __syncthreads();
         }
         // ---- p, ds; the pair goes to the dk/dv kernel ([pair of this launch][s1][l][sample]); the weights become ds * w
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
-            const float p = __builtin_amdgcn_exp2f(ps[it] * qscale - lse[it]);
-            const float ds = p * (pd[it] - delta[it]);
-            if (handed_ && live[it])
-                handed_[(size_t)bhl * VL * dm.N + coff[it] + (unsigned)s2 * (unsigned)dm.P] = make_float2(p, ds * dm.sm_scale);
+            const int r = it / KB;
+            const float p = __builtin_amdgcn_exp2f(ps[it] * qscale - lse[r]);
+            const float ds = p * (pd[it] - delta[r]);
+            if (handed_ && live[r])
+                handed_[(size_t)bhl * VL * dm.N + coff[r] + (unsigned)s2 * (unsigned)dm.P + (unsigned)(it % KB) * kSlabSamples] =
+                    make_float2(p, ds * dm.sm_scale);
 #pragma unroll
             for (int t = 0; t < 4; ++t) w[it][t] *= ds;
         }
@@ -501,21 +521,21 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
             const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                acc[it][s] += slab_axpy(slab4, off[it], cur, chv, w[it], lane);
+                acc[it / KB][s] += slab_axpy(slab4, off[it], cur, chv, w[it], lane);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (s == NSLAB - 1 && lane < 16 * IT) xlds[lane] = xnext;
+            if (s == NSLAB - 1 && lane < 4 * RW) xlds[lane] = xnext;
             SlabStager<NW>::wait();
             __syncthreads();
         }
     }
 
 #pragma unroll
-    for (int it = 0; it < IT; ++it) {
-        if (!live[it]) continue;
-        const size_t row = row_of(rb * RB + (wave * IT + it) * 4 + rg);
+    for (int r = 0; r < NR; ++r) {
+        if (!live[r]) continue;
+        const size_t row = row_of(rb * RB + wave * RW + 4 * r + rg);
 #pragma unroll
-        for (int s = 0; s < NSLAB; ++s) dq_[row * D + s * kSlabCols + col] = acc[it][s] * dm.sm_scale;
+        for (int s = 0; s < NSLAB; ++s) dq_[row * D + s * kSlabCols + col] = acc[r][s] * dm.sm_scale;
     }
 }
 

@@ -113,26 +113,29 @@ def test_staged_forward_two_row_blocks(dtype):
     assert rel(dv, rdv) < TOL_BWD[dtype]
 
 
-# fp32 storage, 16 samples per view, planes too large for LDS but small enough for two 16-column slabs of the whole
-# image: the forward and the dq kernel walk the planes slab by slab through LDS (fwd_slab_kernel,
+# fp32 storage, 16 or 32 samples per view, planes too large for LDS but small enough for two 16-column slabs of the
+# whole image: the forward and the dq kernel walk the planes slab by slab through LDS (fwd_slab_kernel,
 # bwd_dq_slab_kernel), every tap read from there.
 SLABS = [
-    # seed B  V  H  Himg Wimg D    lo     hi
-    (81, 1, 2, 2, 20, 20, 64, -0.1, 1.1),       # width a multiple of 4: two padding columns per image row; 800 query rows: 4 full workgroups and a part
-    (82, 2, 3, 1, 23, 19, 64, -0.3, 1.3),       # odd width, runs of 16 pixels cut by the row end, heavy out-of-image
-    (83, 1, 2, 2, 17, 17, 128, 0.0, 1.0),       # eight slabs per plane
-    (84, 1, 1, 3, 20, 32, 32, -0.05, 1.05),     # two slabs per plane, one view
-    (85, 1, 2, 1, 32, 32, 64, -0.1, 1.1),       # the largest image the kernel takes (64 runs)
-    (86, 1, 1, 2, 21, 48, 64, -0.1, 1.1),       # three runs per image row, 63 runs
-    (87, 1, 2, 1, 40, 16, 64, 0.0, 1.0),        # one run per image row, tall image
-    (88, 1, 2, 1, 16, 17, 128, -0.2, 1.2),      # second run of a row holds one pixel
+    # seed B  V  H  Himg Wimg D    P   lo     hi
+    (81, 1, 2, 2, 20, 20, 64, 16, -0.1, 1.1),   # width a multiple of 4: two padding columns per image row; 800 query rows: 4 full workgroups and a part
+    (82, 2, 3, 1, 23, 19, 64, 16, -0.3, 1.3),   # odd width, runs of 16 pixels cut by the row end, heavy out-of-image
+    (83, 1, 2, 2, 17, 17, 128, 16, 0.0, 1.0),   # eight slabs per plane
+    (84, 1, 1, 3, 20, 32, 32, 16, -0.05, 1.05), # two slabs per plane, one view
+    (85, 1, 2, 1, 32, 32, 64, 16, -0.1, 1.1),   # the largest image the kernel takes (64 runs)
+    (86, 1, 1, 2, 21, 48, 64, 16, -0.1, 1.1),   # three runs per image row, 63 runs
+    (87, 1, 2, 1, 40, 16, 64, 16, 0.0, 1.0),    # one run per image row, tall image
+    (88, 1, 2, 1, 16, 17, 128, 16, -0.2, 1.2),  # second run of a row holds one pixel
+    (89, 1, 2, 2, 20, 20, 64, 32, -0.1, 1.1),   # 32 samples per view: two blocks of 16 per query row in one lane
+    (90, 2, 1, 1, 25, 30, 32, 32, -0.2, 1.2),
+    (91, 1, 3, 1, 18, 18, 128, 32, 0.0, 1.0),
 ]
 
 
 @pytest.mark.parametrize("case", SLABS, ids=[f"b{c[0]}" for c in SLABS])
 def test_slab_forward_vs_oracle(case):
-    seed, B, V, H, Himg, Wimg, D, lo, hi = case
-    P, dtype = 16, torch.float32
+    seed, B, V, H, Himg, Wimg, D, P, lo, hi = case
+    dtype = torch.float32
     say(f"[case] slabs seed={seed} B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} {dtype}")
     q, k, v, c, do = make_case(seed, B, V, H, Himg, Wimg, D, P, lo, hi, dtype)
     c[0, 0, 1, 0, 3, 0] = float("nan")                     # a sample without taps
