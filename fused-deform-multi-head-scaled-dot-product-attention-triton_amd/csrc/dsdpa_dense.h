@@ -226,11 +226,22 @@ __global__ __launch_bounds__((DenseCfg<D, TQ>::kThreads), 2) void fwd_dense_kern
         for (int nt = 0; nt < NTW; ++nt) oacc[mt][nt] = floatx4{0.f, 0.f, 0.f, 0.f};
     float m_run = kNegBig, l_run = 0.f;            // of query qi; l_run: this thread's samples only
 
+    // the coordinates of a chunk are requested a chunk ahead (they come from HBM or the memory-side cache, once per head)
+    float2 xy_next[4];
+    auto fetch_coords = [&](int ci) {
+        const int s2 = ci / view_chunks, p0 = (ci - s2 * view_chunks) * kWave;
+        const int cnt = min(kWave, dm.P - p0);
+        const float2 *crd = crd_row + s2 * dm.P + p0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xy_next[i] = crd[min(4 * sub + i, cnt - 1)];
+    };
+    fetch_coords(0);
     for (int ci = 0; ci < nchunks; ++ci) {
         const int s2 = ci / view_chunks, p0 = (ci - s2 * view_chunks) * kWave;
         const int cnt = min(kWave, dm.P - p0);
         // this thread's four samples of query qi: taps once, kept for the logits and the scatter further down
-        const float2 *crd = crd_row + s2 * dm.P + p0;
+        const float2 xy_cur[4] = { xy_next[0], xy_next[1], xy_next[2], xy_next[3] };
+        if (ci + 1 < nchunks) fetch_coords(ci + 1);
         float wgt[4][4];
         unsigned cpix[4];                       // clamped pixel of tap 00: column | row << 16
         unsigned cstep[4];                      // bit 0: tap 01 lies one column on, bit 1: tap 10 one row on
@@ -241,7 +252,7 @@ __global__ __launch_bounds__((DenseCfg<D, TQ>::kThreads), 2) void fwd_dense_kern
             for (int i = 0; i < 4; ++i) {
                 const int p = 4 * sub + i;
                 const bool live = qlive && p < cnt;
-                const float2 xy = crd[min(p, cnt - 1)];
+                const float2 xy = xy_cur[i];
                 const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
 #pragma unroll
                 for (int tpi = 0; tpi < 4; ++tpi) wgt[i][tpi] = live ? tp.w[tpi] : 0.f;
@@ -336,6 +347,26 @@ __global__ __launch_bounds__((DenseCfg<D, TQ>::kThreads), 2) void fwd_dense_kern
         }
         __syncthreads();
 
+        // the first steps' rows of V are requested here already, under the work on the samples: their addresses are
+        // known (offs), and the registers are there (two waves per SIMD)
+        const int nkb = npix >> 5;
+        // row of a load's 64 / VCH that this lane fetches and parks. Four lanes per row: the 16 lanes that one
+        // cycle of a 16-byte LDS write serves take every other row (rows of 96 bytes: 0, 2, 4, 6 start in four
+        // different quarters of the banks, 0, 1, 2, 3 do not)
+        const int vrow_l = VCH == 4 ? 8 * (lane >> 5) + ((lane >> 4) & 1) + 2 * ((lane & 15) >> 2) : lane / VCH;
+        const unsigned vpiece = (unsigned)(wave * NTW * 32 + (lane % VCH) * 16);   // byte in the row of V
+        const unsigned vpark = (unsigned)(lane % VCH) * 16u;
+        // the next kRingV steps' rows are in flight, the next step's are parked while this one is worked on
+        dsdpa_u32x4 vr[kRingV][VLD];
+#define DSDPA_DENSE_FETCH_V(slot_, kb_)                                                                        \
+        _Pragma("unroll") for (int r = 0; r < VLD; ++r)                                                    \
+            vr[slot_][r] = *reinterpret_cast<const dsdpa_u32x4 *>(vplane0 + offs[min((kb_), nkb - 1) * 32 + r * (kWave / VCH) + vrow_l] + vpiece);
+#define DSDPA_DENSE_PARK_V(slot_, buf_)                                                                        \
+        _Pragma("unroll") for (int r = 0; r < VLD; ++r)                                                    \
+            *reinterpret_cast<dsdpa_u32x4 *>(wstage + ((buf_) * 32 + r * (kWave / VCH) + vrow_l) * kPitchV + vpark) = vr[slot_][r];
+#pragma unroll
+        for (int u = 0; u < kRingV; ++u) { DSDPA_DENSE_FETCH_V(u, u) }
+
         // ---- the samples of query qi, four per thread: logits from S, then the softmax bookkeeping of the chunk
         float logit[4];
         unsigned ent[4];                        // entry of tap 00 | (column step << 16) | (row step << 17)
@@ -419,23 +450,6 @@ __global__ __launch_bounds__((DenseCfg<D, TQ>::kThreads), 2) void fwd_dense_kern
         // operand is then two 8-byte reads of P, and the 8 rows that 32 lanes of a transposing read touch are 8
         // consecutive ones.
         {
-            const int nkb = npix >> 5;
-            // row of a load's 64 / VCH that this lane fetches and parks. Four lanes per row: the 16 lanes that one
-            // cycle of a 16-byte LDS write serves take every other row (rows of 96 bytes: 0, 2, 4, 6 start in four
-            // different quarters of the banks, 0, 1, 2, 3 do not)
-            const int vrow_l = VCH == 4 ? 8 * (lane >> 5) + ((lane >> 4) & 1) + 2 * ((lane & 15) >> 2) : lane / VCH;
-            const unsigned vpiece = (unsigned)(wave * NTW * 32 + (lane % VCH) * 16);   // byte in the row of V
-            const unsigned vpark = (unsigned)(lane % VCH) * 16u;
-            // the next kRingV steps' rows are in flight, the next step's are parked while this one is worked on
-            dsdpa_u32x4 vr[kRingV][VLD];
-#define DSDPA_DENSE_FETCH_V(slot_, kb_)                                                                        \
-            _Pragma("unroll") for (int r = 0; r < VLD; ++r)                                                    \
-                vr[slot_][r] = *reinterpret_cast<const dsdpa_u32x4 *>(vplane0 + offs[min((kb_), nkb - 1) * 32 + r * (kWave / VCH) + vrow_l] + vpiece);
-#define DSDPA_DENSE_PARK_V(slot_, buf_)                                                                        \
-            _Pragma("unroll") for (int r = 0; r < VLD; ++r)                                                    \
-                *reinterpret_cast<dsdpa_u32x4 *>(wstage + ((buf_) * 32 + r * (kWave / VCH) + vrow_l) * kPitchV + vpark) = vr[slot_][r];
-#pragma unroll
-            for (int u = 0; u < kRingV; ++u) { DSDPA_DENSE_FETCH_V(u, u) }
             wave_lds_order();                      // (behind the last reads of K's staging)
             DSDPA_DENSE_PARK_V(0, 0)
             DSDPA_DENSE_FETCH_V(0, kRingV)
