@@ -1,14 +1,14 @@
-// Forward and dq for fp32 storage and 16 or 32 samples per view on images whose K/V planes do not fit in LDS but whose planes
-// cut to 16 columns do, twice: "slabs" of 64 bytes per pixel (`ops/triton.py:118-170` is the sampling and softmax
-// loop this replaces; the reference gathers every tap from global memory).
+// Forward and dq for fp32 storage and 16 or 32 samples per view on images whose K/V planes do not fit in LDS but
+// whose planes cut to 16 columns do, twice: "slabs" of 64 bytes per pixel (`ops/triton.py:118-170` is the sampling
+// and softmax loop this replaces; the reference gathers every tap from global memory).
 //
 // A workgroup owns a block of query rows of one (batch, head). For every key view it walks the column slabs of K
 // and then those of V, each the whole image at 64 bytes per pixel, in two LDS buffers: the slab of the next step
-// is fetched into registers before the work on the present one and written to the other buffer after it, one
+// is loaded straight into the other buffer (global_load_lds_dwordx4) while the present one is worked on, one
 // barrier per step. One lane owns one (query row, sample) pair for a whole view: it reads its four tap rows from
 // the slab in 16-byte pieces and keeps the partial dot product (K slabs) in a register, so the tap weights and
 // addresses are computed once per sample and view and nothing is summed across lanes for the logits. For the V
-// slabs the 16 samples of a query row sit in 16 neighbouring lanes, whose weighted sums are combined by a
+// slabs the 16 samples of a block sit in 16 neighbouring lanes, whose weighted sums are combined by a
 // reduce-scatter over those lanes: every lane ends up with one column of the slab.
 //
 // LDS banks (64 banks of 4 bytes; a 16-byte read is served 16 lanes a clock): the piece a lane reads at step c is
@@ -16,7 +16,7 @@
 // row lies in is its index mod 4. Image rows are stored with a pitch of 2 mod 4 pixels, which gives the four
 // taps of a sample (x, x+1, x+pitch, x+pitch+1) four different quarters, and lanes 4g .. 4g+3 of every 16 read
 // their taps in the order that starts in quarter g: the 16 lanes of a clock then touch all 64 banks once,
-// whatever the coordinates (taps clamped at the image border share a row and take a second clock).
+// whatever the coordinates (a tap outside the image reads a row of the quarter it would have had: slab_sample).
 #pragma once
 #include "dsdpa_common.h"
 
