@@ -54,6 +54,7 @@ CASES = [
     (45, 1, 2, 1, 1, 1, 16, 1, 0.0, 1.0),        # 1x1 image: every colour pass but one is empty of pixels
     (46, 1, 3, 2, 1, 11, 128, 5, -0.2, 1.2),
     (47, 1, 2, 1, 40, 40, 16, 4, 0.45, 0.55),    # clustered: a few very long cell lists
+    (48, 1, 2, 2, 20, 20, 64, 16, -0.1, 1.1),    # fp32: dq by the slab kernel (no pairs handed over on this path)
 ]
 
 

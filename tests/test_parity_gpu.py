@@ -331,6 +331,8 @@ STRIDED = [
     (62, 1, 2, 3, 5, 7, 64, 9, "fused-qkv"),
     (63, 1, 2, 2, 40, 40, 64, 6, "permuted"),     # planes too large for LDS: gather kernels
     (64, 1, 2, 2, 24, 20, 32, 64, "fused-qkv"),   # 64 samples per view: chunks per view, window mode
+    (65, 1, 2, 2, 20, 22, 64, 16, "permuted"),    # fp32: the slab kernels (planes staged into LDS from strided rows)
+    (66, 1, 2, 2, 19, 21, 64, 32, "fused-qkv"),
 ]
 
 
