@@ -194,32 +194,42 @@ int launch_fwd_slab(const void *q, const void *k, const void *v, const float *co
     }
 }
 
-// dq of the same shapes, for the (batch, head) pairs [bh0, bh0 + nbh).
-template <typename S, int D>
-int launch_bwd_dq_slab(const void *q, const void *k, const void *v, const float *coords, const void *out,
-                       const float *lse, const void *dout, void *dq, float2 *stats, float2 *handed,
-                       const Dims &dm, int bh0, int nbh, hipStream_t st)
+// dq of the same shapes, for the (batch, head) pairs [bh0, bh0 + nbh). With the coordinate gradient a lane takes
+// half as many samples per view (the per-tap products it then keeps take the registers): 96 query rows a workgroup.
+template <typename S, int D, bool CG>
+int launch_bwd_dq_slab_cg(const void *q, const void *k, const void *v, const float *coords, const void *out,
+                          const float *lse, const void *dout, void *dq, float2 *stats, float2 *handed, float *dcoords,
+                          const Dims &dm, int bh0, int nbh, hipStream_t st)
 {
     if constexpr (S::kBytes != 4 || (D != 32 && D != 64 && D != 128)) {
         return DSDPA_ERR_UNSUPPORTED;
     } else {
-        constexpr int IT = kSlabItems, NW = kSlabWaves;
+        constexpr int IT = CG ? kSlabItems / 2 : kSlabItems, NW = kSlabWaves;
         const int kb = dm.P / kSlabSamples;
         const int RB = NW * 4 * IT / kb;
         const int nblk = (dm.V * dm.L + RB - 1) / RB;
         const long long blocks = (long long)nbh * nblk;
         if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
-        auto kern = kb == 1 ? bwd_dq_slab_kernel<D, IT, NW, 1> : bwd_dq_slab_kernel<D, IT, NW, 2>;
+        auto kern = kb == 1 ? bwd_dq_slab_kernel<D, IT, NW, 1, CG> : bwd_dq_slab_kernel<D, IT, NW, 2, CG>;
         static std::atomic<unsigned long long> lds_set[2];
         if (int rc = allow_full_lds(kern, lds_set[kb >> 1])) return rc;
         ScopedKernelTimer timer(2, st);
         const unsigned buf_bytes = (unsigned)slab_buffer_bytes(dm.Himg, dm.Wimg);
         DSDPA_LAUNCH(kern, dim3((unsigned)blocks), dim3(NW * kWave), (size_t)2 * buf_bytes + NW * 4 * IT * kSlabBytes, st,
                      timer.start(), timer.stop(), (const float *)q, (const float *)k, (const float *)v, coords,
-                     (const float *)out, lse, (const float *)dout, (float *)dq, stats, handed, dm, bh0, nblk,
+                     (const float *)out, lse, (const float *)dout, (float *)dq, stats, handed, dcoords, dm, bh0, nblk,
                      slab_pitch(dm.Wimg), buf_bytes);
         return check_launch();
     }
+}
+
+template <typename S, int D>
+int launch_bwd_dq_slab(const void *q, const void *k, const void *v, const float *coords, const void *out,
+                       const float *lse, const void *dout, void *dq, float2 *stats, float2 *handed, float *dcoords,
+                       const Dims &dm, int bh0, int nbh, hipStream_t st)
+{
+    return dcoords ? launch_bwd_dq_slab_cg<S, D, true>(q, k, v, coords, out, lse, dout, dq, stats, handed, dcoords, dm, bh0, nbh, st)
+                   : launch_bwd_dq_slab_cg<S, D, false>(q, k, v, coords, out, lse, dout, dq, stats, handed, dcoords, dm, bh0, nbh, st);
 }
 
 // The dense-box forward (16-bit storage, D = 64 or 128): one workgroup per tile of 16 queries; the tiles it
@@ -714,8 +724,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     // group's pairs (workspace_layout), and the dk/dv kernel of a group finds them where the dq kernel of the same
     // group has just left them. Otherwise one launch each covers all pairs.
     const int nbh_all = dm.B * dm.H, bh_step = handed ? wl.bh_group : nbh_all;
-    // (the slab dq kernel has no coordinate gradient)
-    const bool slab = path == DSDPA_PATH_AUTO && !staged && !dcoords && slab_path_fits(V, Himg, Wimg, D, P, S::kBytes);
+    const bool slab = path == DSDPA_PATH_AUTO && !staged && slab_path_fits(V, Himg, Wimg, D, P, S::kBytes);
 #define DSDPA_BWD_CASE(DD)                                                                                      \
     case DD:                                                                                                    \
         if (fused_atomics && !dcoords) {                                                                        \
@@ -726,8 +735,8 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
             const int nbh = bh_step < nbh_all - bh0 ? bh_step : nbh_all - bh0;                                  \
             rc = staged ? launch_bwd_dq_plane<S, DD>(q, k, v, desc_w, desc_e, out, lse, dout, dq, dq_stats,     \
                                                      desc_g, dcoords, dm, st)                                   \
-                 : slab ? launch_bwd_dq_slab<S, DD>(q, k, v, coords, out, lse, dout, dq, dq_stats, handed, dm,  \
-                                                    bh0, nbh, st)                                               \
+                 : slab ? launch_bwd_dq_slab<S, DD>(q, k, v, coords, out, lse, dout, dq, dq_stats, handed, dcoords,\
+                                                    dm, bh0, nbh, st)                                           \
                         : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dq_stats, dcoords,   \
                                                       handed, dm, bh0, nbh, st);                                \
             if (rc == DSDPA_OK && cell_binned)                                                                  \

@@ -69,7 +69,8 @@ __device__ __forceinline__ float dpp_xor4(float x)
 // r, r+1, r+2, r+3 (mod 4) with r that of tap 00. A tap outside the image has weight 0 and may read any row: it
 // reads one of the first four, the one in the quarter it would have had (clamped into the image it would share a
 // row with its neighbour, and the 16 lanes of a clock would collide).
-__device__ __forceinline__ void slab_sample(float2 xy, const Dims &dm, int pitch, int g4, unsigned (&off)[4], float (&w)[4])
+// Returns the rotation: place k of the lane's order holds tap (k + rot) mod 4.
+__device__ __forceinline__ int slab_sample(float2 xy, const Dims &dm, int pitch, int g4, unsigned (&off)[4], float (&w)[4])
 {
     const Taps tp = make_taps(xy.x, xy.y, dm.Wimg, dm.Himg);
     const int n0 = tp.y0 * pitch + tp.x0;
@@ -93,16 +94,29 @@ __device__ __forceinline__ void slab_sample(float2 xy, const Dims &dm, int pitch
         off[k] = o[k] * (kSlabBytes / 16);
         w[k] = ww[k];
     }
+    return rot;
+}
+
+// four values in tap order 00, 01, 10, 11 into a lane's read order (place k: tap (k + rot) mod 4)
+__device__ __forceinline__ void slab_rotate(float (&a)[4], int rot)
+{
+    if (rot & 1) {
+        const float f0 = a[0]; a[0] = a[1]; a[1] = a[2]; a[2] = a[3]; a[3] = f0;
+    }
+    if (rot & 2) {
+        const float f0 = a[0], f1 = a[1]; a[0] = a[2]; a[1] = a[3]; a[2] = f0; a[3] = f1;
+    }
 }
 
 // x . (sum_t w_t * row_t) over the 16 columns of the slab in buffer `cur`: x is the wave's parked vector of the
 // sample's query row (q or dout), read from LDS in the same rotated pieces as the taps.
+// d: x . row_t of the four taps (the lane's order), for the caller that needs them one by one.
 __device__ __forceinline__ float slab_dot(const float4 *slab4, const float4 *xrow, const unsigned (&off)[4], unsigned cur,
-                                          const unsigned (&chv)[4], const float (&w)[4])
+                                          const unsigned (&chv)[4], const float (&w)[4], float (&d)[4])
 {
     unsigned ob[4] = { off[0] + cur, off[1] + cur, off[2] + cur, off[3] + cur };
     keep_here(ob);
-    float d[4] = { 0.f, 0.f, 0.f, 0.f };
+    d[0] = d[1] = d[2] = d[3] = 0.f;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         const float4 x = xrow[chv[c]];
@@ -297,7 +311,8 @@ __global__ __launch_bounds__(NW *kWave) void fwd_slab_kernel(
             const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                part[it] += slab_dot(slab4, qlds + ((it / KB) * 4 + rg) * 4, off[it], cur, chv, w[it]);
+                float d[4];
+                part[it] += slab_dot(slab4, qlds + ((it / KB) * 4 + rg) * 4, off[it], cur, chv, w[it], d);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (s + 1 < NSLAB && lane < 4 * RW) qlds[lane] = qnext;      // (this wave has read the present piece)
@@ -365,12 +380,15 @@ __global__ __launch_bounds__(NW *kWave) void fwd_slab_kernel(
 // parked the same way), then p = 2^(s - lse), ds = p (dp - delta), and the K slabs again for dq += ds * k~, the
 // 16 samples of a row combined as in the forward's V walk. Covers the query rows of the (batch, head) pairs
 // [bh0, bh0 + gridDim.x / nblk).
-template <int D, int IT, int NW, int KB>
+// CG: also the gradient of the coordinates (see bwd_dq_gather_kernel): the per-tap products q . K_t and dout . V_t
+// are kept tap by tap over the slabs, and g_t = sm_scale * ds * (q . K_t) + p * (dout . V_t) meets the tap
+// derivatives once per sample and view; two float atomics per sample (the heads share the coordinates).
+template <int D, int IT, int NW, int KB, bool CG>
 __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
     const float *__restrict__ q_, const float *__restrict__ k_, const float *__restrict__ v_,
     const float *__restrict__ coords_, const float *__restrict__ out_, const float *__restrict__ lse_,
     const float *__restrict__ dout_, float *__restrict__ dq_, float2 *__restrict__ stats_,
-    float2 *__restrict__ handed_, Dims dm, int bh0, int nblk, int pitch, unsigned buf_bytes)
+    float2 *__restrict__ handed_, float *__restrict__ dcoords_, Dims dm, int bh0, int nblk, int pitch, unsigned buf_bytes)
 {
     constexpr int NSLAB = D / kSlabCols;
     constexpr int NR = IT / KB, RW = 4 * NR, RB = NW * RW;       // query rows per lane, wave, workgroup (see the forward)
@@ -463,12 +481,22 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
     for (int s2 = 0; s2 < dm.V; ++s2) {
         unsigned off[IT][4];
         float w[IT][4], ps[IT], pd[IT];
+        constexpr int ITG = CG ? IT : 1;
+        float dkt[ITG][4], dvt[ITG][4];          // CG: q . K_t and dout . V_t, tap by tap (the lane's order)
+        float2 xy[ITG];
+        int rot[ITG];
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
-            slab_sample(cb[coff[it / KB] + (unsigned)s2 * (unsigned)dm.P + (unsigned)(it % KB) * kSlabSamples], dm, pitch, g4,
-                        off[it], w[it]);
+            const float2 c = cb[coff[it / KB] + (unsigned)s2 * (unsigned)dm.P + (unsigned)(it % KB) * kSlabSamples];
+            const int r = slab_sample(c, dm, pitch, g4, off[it], w[it]);
             ps[it] = 0.f;
             pd[it] = 0.f;
+            if constexpr (CG) {
+                xy[it] = c;
+                rot[it] = r;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) dkt[it][k] = dvt[it][k] = 0.f;
+            }
         }
         // ---- logits: K slabs, q parked
 #pragma unroll 1
@@ -479,7 +507,12 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
             const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                ps[it] += slab_dot(slab4, xlds + ((it / KB) * 4 + rg) * 4, off[it], cur, chv, w[it]);
+                float d[4];
+                ps[it] += slab_dot(slab4, xlds + ((it / KB) * 4 + rg) * 4, off[it], cur, chv, w[it], d);
+                if constexpr (CG) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) dkt[it][k] += d[k];
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (lane < 4 * RW) xlds[lane] = xnext;
@@ -494,7 +527,12 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
             const unsigned cur = (unsigned)(ph & 1) * (buf_bytes / 16);
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
-                pd[it] += slab_dot(slab4, xlds + ((it / KB) * 4 + rg) * 4, off[it], cur, chv, w[it]);
+                float d[4];
+                pd[it] += slab_dot(slab4, xlds + ((it / KB) * 4 + rg) * 4, off[it], cur, chv, w[it], d);
+                if constexpr (CG) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) dvt[it][k] += d[k];
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (s + 1 < NSLAB && lane < 4 * RW) xlds[lane] = xnext;
@@ -510,6 +548,25 @@ __global__ __launch_bounds__(NW *kWave) void bwd_dq_slab_kernel(
             if (handed_ && live[r])
                 handed_[(size_t)bhl * VL * dm.N + coff[r] + (unsigned)s2 * (unsigned)dm.P + (unsigned)(it % KB) * kSlabSamples] =
                     make_float2(p, ds * dm.sm_scale);
+            if constexpr (CG) {
+                // the tap derivatives (zero for a tap outside the image) in the lane's tap order, times g_t
+                TapGrads tg = make_tap_grads(xy[it].x, xy[it].y, dm.Wimg, dm.Himg);
+                slab_rotate(tg.gx, rot[it]);
+                slab_rotate(tg.gy, rot[it]);
+                const float a = ds * dm.sm_scale;
+                float gx = 0.f, gy = 0.f;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float gk = fmaf(a, dkt[it][k], p * dvt[it][k]);
+                    gx = fmaf(tg.gx[k], gk, gx);
+                    gy = fmaf(tg.gy[k], gk, gy);
+                }
+                if (live[r]) {
+                    float *dst = dcoords_ + 2 * ((size_t)b * VL * dm.N + coff[r] + (unsigned)s2 * (unsigned)dm.P + (unsigned)(it % KB) * kSlabSamples);
+                    atomicAdd(dst, gx);
+                    atomicAdd(dst + 1, gy);
+                }
+            }
 #pragma unroll
             for (int t = 0; t < 4; ++t) w[it][t] *= ds;
         }

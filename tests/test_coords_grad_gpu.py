@@ -42,6 +42,8 @@ CASES = [
     (36, 1, 2, 1, 3, 3, 256, 9, -0.1, 1.1),
     (37, 1, 3, 2, 1, 11, 32, 5, -0.2, 1.2),      # single-row image: no y gradient
     (38, 1, 2, 1, 21, 22, 32, 4, -0.1, 1.1),     # fp32: the planes fit in LDS only without the gradient's block
+    (39, 1, 2, 2, 20, 22, 64, 16, -0.15, 1.15),  # fp32: dq by the slab kernel, two samples per lane and view
+    (40, 1, 2, 1, 19, 19, 64, 32, -0.1, 1.1),    # ... 32 samples per view: the two blocks of a row in one lane
 ]
 
 
