@@ -167,6 +167,9 @@ int launch_fwd_gather(const void *q, const void *k, const void *v, const float *
 // Waves per workgroup and samples per lane and view of the slab kernels: 12 x 4 (168 registers a lane, no spills at
 // D = 64) measured 3-4 % ahead of 16 x 3 (128 registers) at 32x32, D = 64; both cover 192 query rows.
 constexpr int kSlabWaves = 12, kSlabItems = 4;
+// (D = 128 with 32 samples per view: two samples per lane and view -- one query row -- measured 15 % ahead of four,
+//  which spill there; with 16 samples per view four stay ahead on the larger images)
+template <int D, int KB> struct SlabItems { static constexpr int value = (D >= 128 && KB == 2) ? kSlabItems / 2 : kSlabItems; };
 // The slab forward (fp32 storage, 16 samples per view): a workgroup per block of 192 query rows of a
 // (batch, head); the whole image of a view in LDS, 16 columns at a time, in two buffers.
 template <typename S, int D>
@@ -176,13 +179,14 @@ int launch_fwd_slab(const void *q, const void *k, const void *v, const float *co
     if constexpr (S::kBytes != 4 || (D != 32 && D != 64 && D != 128)) {
         return DSDPA_ERR_UNSUPPORTED;
     } else {
-        constexpr int IT = kSlabItems, NW = kSlabWaves;
+        constexpr int IT1 = SlabItems<D, 1>::value, IT2 = SlabItems<D, 2>::value, NW = kSlabWaves;
         const int kb = dm.P / kSlabSamples;                  // 1 or 2 (slab_path_fits)
+        const int IT = kb == 1 ? IT1 : IT2;
         const int RB = NW * 4 * IT / kb;
         const int nblk = (dm.V * dm.L + RB - 1) / RB;
         const long long blocks = (long long)dm.B * dm.H * nblk;
         if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
-        auto kern = kb == 1 ? fwd_slab_kernel<D, IT, NW, 1> : fwd_slab_kernel<D, IT, NW, 2>;
+        auto kern = kb == 1 ? fwd_slab_kernel<D, IT1, NW, 1> : fwd_slab_kernel<D, IT2, NW, 2>;
         static std::atomic<unsigned long long> lds_set[2];
         if (int rc = allow_full_lds(kern, lds_set[kb >> 1])) return rc;
         ScopedKernelTimer timer(0, st);
@@ -204,13 +208,15 @@ int launch_bwd_dq_slab_cg(const void *q, const void *k, const void *v, const flo
     if constexpr (S::kBytes != 4 || (D != 32 && D != 64 && D != 128)) {
         return DSDPA_ERR_UNSUPPORTED;
     } else {
-        constexpr int IT = CG ? kSlabItems / 2 : kSlabItems, NW = kSlabWaves;
+        constexpr int IT1 = CG ? kSlabItems / 2 : SlabItems<D, 1>::value, IT2 = CG ? kSlabItems / 2 : SlabItems<D, 2>::value;
+        constexpr int NW = kSlabWaves;
         const int kb = dm.P / kSlabSamples;
+        const int IT = kb == 1 ? IT1 : IT2;
         const int RB = NW * 4 * IT / kb;
         const int nblk = (dm.V * dm.L + RB - 1) / RB;
         const long long blocks = (long long)nbh * nblk;
         if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
-        auto kern = kb == 1 ? bwd_dq_slab_kernel<D, IT, NW, 1, CG> : bwd_dq_slab_kernel<D, IT, NW, 2, CG>;
+        auto kern = kb == 1 ? bwd_dq_slab_kernel<D, IT1, NW, 1, CG> : bwd_dq_slab_kernel<D, IT2, NW, 2, CG>;
         static std::atomic<unsigned long long> lds_set[2];
         if (int rc = allow_full_lds(kern, lds_set[kb >> 1])) return rc;
         ScopedKernelTimer timer(2, st);
