@@ -209,7 +209,9 @@ int dsdpa_version(void);
  * or more views, where staging costs more than it saves), GATHER always reads the
  * taps from global memory, one query at a time. AUTO alone lets the forward work on
  * tiles of 16 queries with the matrix instructions where the shape allows it
- * (16-bit storage, D = 64 or 128, P >= 64, planes too large for LDS).
+ * (16-bit storage, D = 64 or 128, P >= 64, planes too large for LDS), and lets the
+ * forward and dq walk the planes through LDS 16 columns at a time (fp32 storage,
+ * P = 16 or 32, images of up to 1024 pixels whose planes do not fit in LDS whole).
  * Backward dk/dv: AUTO = cell-binned register accumulation, LDS = tiles of the
  * plane accumulated in LDS with fp64 atomics, GATHER = global float atomics per
  * tap as in the reference (ops/triton.py:345-360). */
