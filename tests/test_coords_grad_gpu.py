@@ -44,6 +44,7 @@ CASES = [
     (38, 1, 2, 1, 21, 22, 32, 4, -0.1, 1.1),     # fp32: the planes fit in LDS only without the gradient's block
     (39, 1, 2, 2, 20, 22, 64, 16, -0.15, 1.15),  # fp32: dq by the slab kernel, two samples per lane and view
     (40, 1, 2, 1, 19, 19, 64, 32, -0.1, 1.1),    # ... 32 samples per view: the two blocks of a row in one lane
+    (41, 1, 2, 1, 24, 24, 64, 16, -0.1, 1.1),    # large enough for the slab kernels at 16-bit storage too
 ]
 
 

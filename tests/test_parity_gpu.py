@@ -129,6 +129,7 @@ SLABS = [
     (89, 1, 2, 2, 20, 20, 64, 32, -0.1, 1.1),   # 32 samples per view: two blocks of 16 per query row in one lane
     (90, 2, 1, 1, 25, 30, 32, 32, -0.2, 1.2),
     (91, 1, 3, 1, 18, 18, 128, 32, 0.0, 1.0),
+    (92, 1, 2, 1, 30, 31, 64, 32, -0.1, 1.1),
 ]
 
 
