@@ -459,6 +459,32 @@ def test_named_workloads_full_size(name):
         assert rel(slice_bh(dv, bb_, hh), rdv) < TOL_BWD[dt], (bb_, hh)
 
 
+def test_backward_recomputes_where_one_pair_exceeds_the_hand_over_buffer():
+    """6 views of 90x90 with 64 samples: the (p, ds) pairs of ONE (batch, head) are 149 MB, more than the buffer
+    the dq kernel may fill, so nothing is handed over and the cell kernel recomputes p and ds on a shape that
+    otherwise takes the gather kernels (window mode in the forward and dq)."""
+    B, V, H, Himg, Wimg, D, P = 1, 6, 1, 90, 90, 16, 64
+    dtype = torch.float32
+    lib = _native.load()
+    # (the workspace holds no pair buffer: lists, counters and per-row pairs only)
+    ws = lib.dsdpa_bwd_workspace_bytes(_native.DSDPA_F32, B, V, H, Himg, Wimg, D, P, 0)
+    assert ws < 12 * B * V * Himg * Wimg * V * P + (64 << 20)
+    say(f"[case] no hand-over B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} {dtype}")
+    g = torch.Generator().manual_seed(97)
+    L = Himg * Wimg
+    q, k, v = (torch.randn(B, V, H, L, D, generator=g).to(dtype) for _ in range(3))
+    mu = torch.rand(B, V, L, V, 1, 2, generator=g) * 0.8 + 0.1
+    c = mu + 0.03 * torch.randn(B, V, L, V, P, 2, generator=g)
+    do = torch.randn(B, V, H, L, D, generator=g).to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    out, dq, dk, dv = run_op(q, k, v, c, do, Wimg, Himg, scale)
+    ro, _, rdq, rdk, rdv = oracle_all(q, k, v, c, do, Wimg, Himg, scale)
+    assert rel(out, ro) < TOL_FWD[dtype]
+    assert rel(dq, rdq) < TOL_BWD[dtype]
+    assert rel(dk, rdk) < TOL_BWD[dtype]
+    assert rel(dv, rdv) < TOL_BWD[dtype]
+
+
 @pytest.mark.parametrize("name", ["C2", "C4", "C5"])
 def test_peak_memory_is_linear_in_tensor_size(name):
     """No sampled-tensor materialisation, no softmax matrix either: the fwd+bwd peak beyond the inputs and dout is
