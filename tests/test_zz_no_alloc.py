@@ -68,6 +68,23 @@ def test_noalloc_forward_matches_workspace_forward_twice(dtype):
         assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
 
 
+def test_noalloc_forward_tile_flags_and_slabs():
+    lib = _native.load()
+    # 16-bit storage, 64 samples per view, planes too large for LDS: the kernel on tiles of 16 queries keeps its
+    # tile flags in the built-in buffer (uniform coordinates: most tiles are left to the per-query kernel behind it)
+    for seed, shape in ((55, (1, 2, 2, 40, 36, 64, 64)), (56, (1, 2, 1, 33, 30, 128, 64))):
+        print(f"[case] no-alloc forward, tile flags {shape}", flush=True)
+        need, (out_a, lse_a), (out_b, lse_b) = _both(lib, shape, torch.bfloat16, seed)
+        assert 0 < need <= _native.NOALLOC_SCRATCH_BYTES
+        assert torch.isfinite(out_b.float()).all()
+        assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
+    # fp32, 16 samples per view: the slab kernel (no workspace, 150 KB of LDS)
+    print("[case] no-alloc forward, slab kernel", flush=True)
+    need, (out_a, lse_a), (out_b, lse_b) = _both(lib, (1, 2, 2, 28, 30, 64, 16), torch.float32, 57)
+    assert need == 0
+    assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
+
+
 def test_noalloc_forward_without_workspace_and_refusal():
     lib = _native.load()
     # planes too large for LDS: the gather kernels, no workspace at all
