@@ -106,7 +106,11 @@ def test_caller_stream_is_ordered_before_and_after():
         assert abs(s_.item() - r_.double().sum().item()) <= 1e-4 * r_.double().abs().sum().item()
 
 
-@pytest.mark.parametrize("dims", [(2, 3, 4, 10, 9, 32, 13), (2, 4, 16, 12, 12, 32, 32)], ids=["small", "forking"])
+# "slabs": fp32 takes the slab kernels (planes loaded straight into LDS), 16-bit the gather kernels; "windows": planes too
+# large for LDS with 64 samples per view: fp32 the window mode of the gather kernels, 16-bit the forward on tiles of 16
+# queries with the per-query kernel behind it
+@pytest.mark.parametrize("dims", [(2, 3, 4, 10, 9, 32, 13), (2, 4, 16, 12, 12, 32, 32), (1, 2, 2, 22, 24, 64, 16),
+                                  (1, 2, 2, 24, 40, 64, 64)], ids=["small", "forking", "slabs", "windows"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_captured_graph_replays_to_the_eager_result(dtype, dims):
     """Forward + backward captured once in a HIP graph (torch.cuda.graph), replayed with new inputs copied into
