@@ -308,8 +308,9 @@ void bwd_dkdv_cell_kernel(
     __shared__ float2 s_f[S::kBytes == 2 ? kCellWaves : 1][kWave];          // 16-bit storage: (fx, fy) of the entry
     __shared__ __attribute__((aligned(16))) float s_flush[kCellWaves][4 * D];                 // the flush: four rows of dk, then of dv
     constexpr bool kQuad = HANDED && S::kBytes == 2 && DC >= 8;            // four-entry trips (below)
-    __shared__ float4 s_wq[kQuad ? kCellWaves : 1][2 * kWave];               // kQuad: two sets of entry tables, used in turn
-    __shared__ unsigned s_rowq[kQuad ? kCellWaves : 1][2 * kWave], s_qrowq[kQuad ? kCellWaves : 1][2 * kWave];
+    // kQuad: a ring of merged entries; the coefficients as [tap][place]
+    __shared__ __attribute__((aligned(16))) float s_ckq[kQuad ? kCellWaves : 1][2 * 4 * kWave], s_cvq[kQuad ? kCellWaves : 1][2 * 4 * kWave];
+    __shared__ __attribute__((aligned(16))) unsigned s_rowq[kQuad ? kCellWaves : 1][2 * kWave], s_qrowq[kQuad ? kCellWaves : 1][2 * kWave];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave index is uniform: keep it in an SGPR
     const unsigned work = (unsigned)xcd_logical_block(blockIdx.x, gridDim.x) * kCellWaves + wave;
@@ -442,83 +443,138 @@ void bwd_dkdv_cell_kernel(
         // lanes with their elements of the four query rows -- as stored, regrouped by two byte permutes per pair
         // of rows. 4 * DC instructions do what 4 * 2 * DC rank-1 updates and as many bf16 -> fp32 conversions did.
         //
-        // Everything is requested ahead, across the 64-entry blocks too: the q rows of the next trip when this
-        // trip's are used up, the dout rows likewise (one set of registers each); the entry tables of the next
-        // block are made while this block is worked on (two sets in LDS, used in turn), from ids fetched three
-        // blocks ahead and pairs and positions fetched two blocks ahead, so that the last trip of a block can
-        // request the rows of the first trip of the next.
-        constexpr int QT = 4 * NS;
-        static_assert(kWave % QT == 0, "a block of 64 entries is a whole number of four-entry trips");
-        // (one array per table, the set chosen by an index: pointers picked at run time would be generic ones,
-        // whose loads count as memory loads and make every wait a wait for the rows in flight)
-        auto prepare = [&](unsigned cstart, int buf, unsigned sid, float2 ff, float2 pdv) {
+        // Entries of ONE query in one cell are merged before their rows are requested: a query's samples cluster,
+        // the fill pass of the binning leaves the samples that one wave places in one list next to each other (the
+        // ranks that one returning LDS atomic hands out), and the sums are linear in the coefficients -- so a run
+        // of up to four neighbouring entries with the same query row becomes one entry with the summed tap
+        // coefficients: one gather of q and dout and one set of matrix instructions instead of up to four.
+        //
+        // The merged entries of the list's 64-entry blocks are appended to a ring of kRing places in LDS (tables
+        // [tap][place] of coefficients and [place] of row offsets); trips of QT merged entries are taken off its
+        // head. Everything is requested ahead: the q and dout rows of the next trip while this trip is worked on
+        // (one set of registers each), which needs the next trip's places filled -- so blocks are merged two ahead
+        // of the trips, and trips run while two whole trips are in the ring (all of them once the last block is in;
+        // the places after the last entry then hold zero coefficients and the row of a live entry).
+        constexpr int QT = 4 * NS, kRing = 2 * kWave;
+        static_assert(QT % 4 == 0 && kRing % QT == 0 && kRing >= 2 * kWave && kRing >= kWave + 3 * QT,
+                      "two blocks fit before the first trip; places written by one block never reach the trips in flight");
+        // (requests past the end of the list repeat its last entry: no request sits under a branch, and the number
+        // of requests in flight at any point is the same on every path -- the compiler's waits are exact then)
+        auto load_id_q = [&](unsigned cstart) -> unsigned { return list[min(cstart + (unsigned)lane, hi - 1u)]; };
+        auto load_frac_q = [&](unsigned cstart) -> float2 { return fracl[min(cstart + (unsigned)lane, hi - 1u)]; };
+        auto prepare = [&](unsigned cstart, int tail, unsigned sid, float2 ff, float2 pdv) -> int {
             const unsigned ql = dm.divP.div(sid);                                  // ql = s1*L + l
             const unsigned s1 = dm.divL.div(ql), l = ql - s1 * (unsigned)dm.L;
             const bool live = cstart + (unsigned)lane < hi;                        // a dead entry adds nothing
-            s_wq[wave][buf * kWave + lane] = make_float4(ff.x, ff.y, live ? pdv.x : 0.f, live ? pdv.y : 0.f);
-            s_rowq[wave][buf * kWave + lane] = (s1 * view_rows + l) * kRowBytes;
-            s_qrowq[wave][buf * kWave + lane] = (s1 * (unsigned)dm.q_sv + l * (unsigned)dm.q_sl) * S::kBytes;
+            const unsigned before = (unsigned)__shfl_up((int)ql, 1, kWave);
+            const unsigned long long below = (1ull << lane) - 1ull;                // the lanes under this one
+            const unsigned long long first = __ballot(lane == 0 || ql != before);  // first entries of the runs of one row
+            const int run0 = 63 - __builtin_clzll(first & (below | (1ull << lane)));
+            const bool lead = live && ((lane - run0) & 3) == 0;                    // runs are cut into merged entries of up to four
+            const unsigned long long leads = __ballot(lead);
+            const int idx = __builtin_popcountll(leads & below);                   // a leader's place after the tail
+            const int n = __builtin_popcountll(leads);
+            // the entries after this one that belong to the same merged entry: the lanes up to the next leader
+            const bool f1 = lane < 63 && !((leads >> (lane + 1)) & 1ull);
+            const bool f2 = f1 && lane < 62 && !((leads >> (lane + 2)) & 1ull);
+            const float m1 = f1 ? 1.0f : 0.0f, m2 = f2 ? 1.0f : 0.0f;
+            const float pn = live ? pdv.x : 0.f, dsn = live ? pdv.y : 0.f;
+            const float gx = 1.0f - ff.x, gy = 1.0f - ff.y;
+            const float wt[4] = { gx * gy, ff.x * gy, gx * ff.y, ff.x * ff.y };
+            float c[8];
+#pragma unroll
+            for (int tpi = 0; tpi < 4; ++tpi) { c[tpi] = wt[tpi] * dsn; c[4 + tpi] = wt[tpi] * pn; }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float pairsum = fmaf(m1, __shfl_down(c[i], 1, kWave), c[i]);
+                c[i] = fmaf(m2, __shfl_down(pairsum, 2, kWave), pairsum);
+            }
+            const unsigned row = (s1 * view_rows + l) * kRowBytes;
+            const unsigned qrow = (s1 * (unsigned)dm.q_sv + l * (unsigned)dm.q_sl) * S::kBytes;
+            float *ck = s_ckq[wave], *cv = s_cvq[wave];
+            if (lead) {
+                const int at = (tail + idx) & (kRing - 1);
+#pragma unroll
+                for (int tpi = 0; tpi < 4; ++tpi) { ck[tpi * kRing + at] = c[tpi]; cv[tpi * kRing + at] = c[4 + tpi]; }
+                s_rowq[wave][at] = row;
+                s_qrowq[wave][at] = qrow;
+            }
+            // the places up to the end of a last, partial trip: no coefficients, and a row that is in this list
+            // (no further: the two blocks merged before the first trip may fill the ring to its last place)
+            if (tail + n + lane < ((tail + n + QT - 1) & ~(QT - 1))) {
+                const int at = (tail + n + lane) & (kRing - 1);
+#pragma unroll
+                for (int tpi = 0; tpi < 4; ++tpi) { ck[tpi * kRing + at] = 0.f; cv[tpi * kRing + at] = 0.f; }
+                s_rowq[wave][at] = (unsigned)__builtin_amdgcn_readfirstlane((int)row);
+                s_qrowq[wave][at] = (unsigned)__builtin_amdgcn_readfirstlane((int)qrow);
+            }
+            return n;
         };
         uint32_t rq[4][kRowWords], rd[4][kRowWords];
-        auto issue_q = [&](int buf, int j0) {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) load_words<kRowWords>(q_bh + (s_qrowq[wave][buf * kWave + j0 + 4 * slot + k] + lane_byte), rq[k]);
+        auto issue_q = [&](int at0) {
+            const uint4 r = reinterpret_cast<const uint4 *>(s_qrowq[wave])[((at0 >> 2) + slot) & (kRing / 4 - 1)];
+            load_words<kRowWords>(q_bh + (r.x + lane_byte), rq[0]);
+            load_words<kRowWords>(q_bh + (r.y + lane_byte), rq[1]);
+            load_words<kRowWords>(q_bh + (r.z + lane_byte), rq[2]);
+            load_words<kRowWords>(q_bh + (r.w + lane_byte), rq[3]);
         };
-        auto issue_d = [&](int buf, int j0) {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) load_words<kRowWords>(do_bh + (s_rowq[wave][buf * kWave + j0 + 4 * slot + k] + lane_byte), rd[k]);
+        auto issue_d = [&](int at0) {
+            const uint4 r = reinterpret_cast<const uint4 *>(s_rowq[wave])[((at0 >> 2) + slot) & (kRing / 4 - 1)];
+            load_words<kRowWords>(do_bh + (r.x + lane_byte), rd[0]);
+            load_words<kRowWords>(do_bh + (r.y + lane_byte), rd[1]);
+            load_words<kRowWords>(do_bh + (r.z + lane_byte), rd[2]);
+            load_words<kRowWords>(do_bh + (r.w + lane_byte), rd[3]);
         };
+        // (places that were never written are read for requests that nothing uses: any row of the pair will do)
+        s_rowq[wave][lane] = 0u;
+        s_rowq[wave][kWave + lane] = 0u;
+        s_qrowq[wave][lane] = 0u;
+        s_qrowq[wave][kWave + lane] = 0u;
+        int head = 0, tail;
+        unsigned id_a;
         {
-            const unsigned id0 = load_id(lo);
-            prepare(lo, 0, id0, load_frac(lo), load_pair(id0));
+            const unsigned id0 = load_id_q(lo), id1 = load_id_q(lo + kWave);
+            id_a = load_id_q(lo + 2 * kWave);
+            const float2 ff0 = load_frac_q(lo), ff1 = load_frac_q(lo + kWave);
+            const float2 pd0 = load_pair(id0), pd1 = load_pair(id1);
+            tail = prepare(lo, 0, id0, ff0, pd0);
+            tail += prepare(lo + kWave, tail, id1, ff1, pd1);
         }
-        unsigned id_a = load_id(lo + kWave);                                        // of the next block
-        float2 ff_a = load_frac(lo + kWave), pd_a = load_pair(id_a);
-        unsigned id_b = load_id(lo + 2 * kWave);                                    // of the block after it
         wave_lds_sync();
-        issue_q(0, 0);
-        issue_d(0, 0);
-        int cur = 0;
-        for (unsigned c0 = lo; c0 < hi; c0 += kWave) {
-            const bool has_next = c0 + kWave < hi;
-            const float2 pd_b = load_pair(id_b), ff_b = load_frac(c0 + 2 * kWave);
-            const unsigned id_c = load_id(c0 + 3 * kWave);
+        issue_q(0);
+        issue_d(0);
+        const int tap_lane = (lane & 3) * (kRing / 4) + slot;                       // this lane's tap, its slot's four entries (in float4 units)
+        for (unsigned cnext = lo + 2 * kWave;; cnext += kWave) {
+            const bool more = cnext < hi;                      // a block is left to merge
+            const float2 pd_a = load_pair(id_a), ff_a = load_frac_q(cnext);
+            const unsigned id_n = load_id_q(cnext + kWave);
             __builtin_amdgcn_sched_barrier(0);                 // (requested here, not where they are used)
-            wave_lds_sync();
-            prepare(c0 + kWave, cur ^ 1, id_a, ff_a, pd_a);
-            wave_lds_sync();
-            const int cnt = (int)min((unsigned)kWave, hi - c0);
-            for (int j0 = 0; j0 < cnt; j0 += QT) {
-                float ck[4], cv[4];
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const float4 e = s_wq[wave][cur * kWave + j0 + 4 * slot + k];        // (fx, fy, p, sm_scale * ds)
-                    const float cl = fmaf(e.x, row_sx, row_ox) * fmaf(e.y, row_sy, row_oy);
-                    ck[k] = cl * e.w;
-                    cv[k] = cl * e.z;
-                }
-                const uint4 sk = split_coefficients<S>(ck[0], ck[1], ck[2], ck[3]);
-                const uint4 sv = split_coefficients<S>(cv[0], cv[1], cv[2], cv[3]);
-                // the next trip: of this block, or the first of the next block (none: this block's first, unused)
-                const bool over = j0 + QT >= kWave && has_next;
-                const int nbuf = over ? cur ^ 1 : cur, nj = (j0 + QT) & (kWave - 1);
+            // (at least one trip: a whole block adds QT merged entries or more to the QT or more that the trips before left)
+            const int stop = more ? tail - 2 * QT : tail - 1;
+            do {
+                const int at = (head & (kRing - 1)) >> 2;
+                const float4 ck4 = reinterpret_cast<const float4 *>(s_ckq[wave])[tap_lane + at];
+                const float4 cv4 = reinterpret_cast<const float4 *>(s_cvq[wave])[tap_lane + at];
+                const uint4 sk = split_coefficients<S>(ck4.x, ck4.y, ck4.z, ck4.w);
+                const uint4 sv = split_coefficients<S>(cv4.x, cv4.y, cv4.z, cv4.w);
                 __builtin_amdgcn_sched_barrier(0);
                 block_blend4_pair<S, DC>(rq, __builtin_bit_cast(shortx4, make_uint2(sk.x, sk.y)),
                                          __builtin_bit_cast(shortx4, make_uint2(sk.z, sk.w)), mK);
                 __builtin_amdgcn_sched_barrier(0);
-                issue_q(nbuf, nj);
+                issue_q(head + QT);
                 __builtin_amdgcn_sched_barrier(0);
                 block_blend4_pair<S, DC>(rd, __builtin_bit_cast(shortx4, make_uint2(sv.x, sv.y)),
                                          __builtin_bit_cast(shortx4, make_uint2(sv.z, sv.w)), mV);
                 __builtin_amdgcn_sched_barrier(0);
-                issue_d(nbuf, nj);
+                issue_d(head + QT);
                 __builtin_amdgcn_sched_barrier(0);
-            }
-            id_a = id_b;
-            ff_a = ff_b;
-            pd_a = pd_b;
-            id_b = id_c;
-            cur ^= 1;
+                head += QT;
+            } while (head <= stop);
+            if (!more) break;
+            wave_lds_sync();
+            tail += prepare(cnext, tail, id_a, ff_a, pd_a);
+            wave_lds_sync();
+            id_a = id_n;
         }
     }
     unsigned id_nxt = kQuad ? 0u : load_id(lo);

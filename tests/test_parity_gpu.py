@@ -485,6 +485,35 @@ def test_backward_recomputes_where_one_pair_exceeds_the_hand_over_buffer():
     assert rel(dv, rdv) < TOL_BWD[dtype]
 
 
+@pytest.mark.parametrize("spread, seed", [("uniform", 101), ("clustered", 102), ("tight", 103)])
+def test_backward_merges_entries_of_one_query_in_long_lists(spread, seed):
+    """D = 128 in bf16 with the pairs handed over: the dk/dv kernel merges neighbouring list entries of one query
+    and keeps the merged ones in a ring. 20x20 images (too large for the staged kernels) with 64 samples from 4 views
+    give lists of some 230 entries
+    per cell -- several 64-entry blocks, so the ring wraps. `uniform`: hardly any entry merges (the two blocks
+    merged before the first trip fill the ring to its last place); `clustered`: sigma of one pixel, about half of
+    them merge; `tight`: sigma of a tenth of a pixel, runs longer than the four entries that merge into one."""
+    B, V, H, Himg, Wimg, D, P = 1, 4, 2, 20, 20, 128, 64
+    dtype = torch.bfloat16
+    say(f"[case] merged entries {spread} B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} {dtype}")
+    g = torch.Generator().manual_seed(seed)
+    L = Himg * Wimg
+    q, k, v = (torch.randn(B, V, H, L, D, generator=g).to(dtype) for _ in range(3))
+    if spread == "uniform":
+        c = torch.rand(B, V, L, V, P, 2, generator=g)
+    else:
+        mu = torch.rand(B, V, L, V, 1, 2, generator=g) * 0.8 + 0.1
+        c = mu + (1.0 / 20 if spread == "clustered" else 0.1 / 20) * torch.randn(B, V, L, V, P, 2, generator=g)
+    do = torch.randn(B, V, H, L, D, generator=g).to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    out, dq, dk, dv = run_op(q, k, v, c, do, Wimg, Himg, scale)
+    ro, _, rdq, rdk, rdv = oracle_all(q, k, v, c, do, Wimg, Himg, scale)
+    assert rel(out, ro) < TOL_FWD[dtype]
+    assert rel(dq, rdq) < TOL_BWD[dtype]
+    assert rel(dk, rdk) < TOL_BWD[dtype]
+    assert rel(dv, rdv) < TOL_BWD[dtype]
+
+
 @pytest.mark.parametrize("name", ["C2", "C4", "C5"])
 def test_peak_memory_is_linear_in_tensor_size(name):
     """No sampled-tensor materialisation, no softmax matrix either: the fwd+bwd peak beyond the inputs and dout is
