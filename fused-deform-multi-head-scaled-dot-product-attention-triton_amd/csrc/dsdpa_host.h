@@ -226,15 +226,17 @@ struct WorkspaceLayout {
 };
 
 // Work list of the dk/dv kernel: a cell list is cut into items of at most `piece` entries, four times the
-// average list length over the whole cell grid (at least 512, a multiple of 64): lists near the average
-// stay whole, the heavy ones of clustered coordinates are shared by several waves (64x64, 64 samples per
-// view, clustered: 1024 entries a piece, 4.13 ms for the kernel; 2048: 4.35 ms, the last pieces running alone). NC + M/piece bounds the
-// number of items per (batch, key view), M = V*L*P being all its entries.
+// average list length over the whole cell grid (at least 768, a multiple of 64): lists near the average
+// stay whole, the heavy ones of clustered coordinates are shared by several waves. Every item ends with a flush
+// of 8*D float atomics, a quarter of the kernel's time where the lists are long (64x64, 64 samples per view,
+// clustered, two groups of query views: pieces of 512 entries 1.63 ms, 768 1.58, 1024 1.60, 2048 1.68 -- the last
+// pieces then run alone). NC + M/piece bounds the number of items per (batch, key view), M = V*L*P being all its
+// entries.
 inline void work_list_geometry(size_t V, size_t L, size_t P, size_t NC, unsigned *piece, unsigned *wmax)
 {
     const size_t M = V * L * P;
     size_t pc = 4 * M / NC;
-    if (pc < 512) pc = 512;
+    if (pc < 768) pc = 768;
     pc = (pc + 63) / 64 * 64;
     if (pc > 0x40000000u) pc = 0x40000000u;
     *piece = (unsigned)pc;

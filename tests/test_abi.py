@@ -78,7 +78,7 @@ def test_workspace_bytes():
         total += r256(B * V * V * Himg * Wimg * P * 8)          # positions beside the ids
         # work list of the dk/dv kernel: items of at most `piece` list entries, (cell, first entry, end) in 16 bytes each
         M = V * Himg * Wimg * P
-        piece = (max(512, 4 * M // NC) + 63) // 64 * 64
+        piece = (max(768, 4 * M // NC) + 63) // 64 * 64
         total += r256(B * V * (NC + M // piece + 1) * 16)
         # (p, ds) per query*sample of one group of (batch, head) pairs, dq kernel -> dk/dv kernel
         total += r256(handed_group(B, V, H, Himg, Wimg, D, P, storage16) * V * Himg * Wimg * V * P * 8)
