@@ -217,8 +217,45 @@ __device__ __forceinline__ void window_dots(const char *__restrict__ base, const
             d[k] = acc;
         }
     }
+    if constexpr (G > 0) {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) d[k] = group_sum<G>(d[k]);
+        for (int k = 0; k < 4; ++k) d[k] = group_sum<G>(d[k]);
+    }
+}
+
+// Sums over the 16 lanes of a slot of EIGHT values per lane, a[0..3] and b[0..3], by reduce-scatter: a step adds two
+// halves of the slot and leaves each half with half of the values, so that the steps cost 8 + 4 + 2 + 2 instructions
+// where butterflies over all eight values cost 32. The first two steps are vector adds whose first operand comes
+// from the partner lane (row rotation by 8, then by 4 up or down) and whose bank mask -- a bank is four lanes -- makes
+// them write one half of the lanes only: lanes 0-7 of the slot take a, lanes 8-15 take b; then banks 0 and 2 take
+// values 0 and 1, banks 1 and 3 values 2 and 3. The last two steps are butterflies inside the banks. Afterwards
+// lane 4j + i holds in (r0, r1): j = 0: (a0, a1), j = 1: (a2, a3), j = 2: (b0, b1), j = 3: (b2, b3), summed.
+// (A rotation by N hands lane i the value of lane (i - N) mod 16. The s_nop covers the two wait states between a
+// vector instruction's write and a cross-lane read of the same register.)
+__device__ __forceinline__ void slot16_sums(const float (&a)[4], const float (&b)[4], float &r0, float &r1)
+{
+    float h0, h1, h2, h3;
+    asm volatile("s_nop 1\n\t"
+                 "v_add_f32_dpp %0, %4, %4 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                 "v_add_f32_dpp %1, %5, %5 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                 "v_add_f32_dpp %2, %6, %6 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                 "v_add_f32_dpp %3, %7, %7 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                 "v_add_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %1, %9, %9 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %2, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %3, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc"
+                 : "=&v"(h0), "=&v"(h1), "=&v"(h2), "=&v"(h3)
+                 : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]));
+    float q0, q1;
+    asm volatile("s_nop 1\n\t"
+                 "v_add_f32_dpp %0, %2, %2 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+                 "v_add_f32_dpp %1, %3, %3 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+                 "v_add_f32_dpp %0, %4, %4 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+                 "v_add_f32_dpp %1, %5, %5 row_ror:4 row_mask:0xf bank_mask:0xa"
+                 : "=&v"(q0), "=&v"(q1)
+                 : "v"(h0), "v"(h1), "v"(h2), "v"(h3));
+    r0 = group_sum<4>(q0);
+    r1 = group_sum<4>(q1);
 }
 
 // The same with EIGHT lanes per pixel (16-bit storage, rows of 16 lanes): lane g2 of a slot takes DC elements of
@@ -822,11 +859,23 @@ __global__ __launch_bounds__(kGatherWaves *kWave, (WIN && !CG && DC <= 8) ? 4 : 
                     const uint4 ent = *reinterpret_cast<const uint4 *>(q_ent + 4 * qd);
                     const unsigned o[4] = { off.x + lane_byte, off.y + lane_byte, off.z + lane_byte, off.w + lane_byte };
                     float dk4[4], dv4[4];
-                    window_dots<S, DC, G>(kb, o, qf, qp, dk4);
-                    window_dots<S, DC, G>(vb, o, dof, dop, dv4);
-                    if (g == 0) {
-                        tS[ent.x] = dk4[0]; tS[ent.y] = dk4[1]; tS[ent.z] = dk4[2]; tS[ent.w] = dk4[3];
-                        tT[ent.x] = dv4[0]; tT[ent.y] = dv4[1]; tT[ent.z] = dv4[2]; tT[ent.w] = dv4[3];
+                    if constexpr (G == 16) {
+                        // the eight sums over the slot by reduce-scatter: every bank of four lanes ends up with two of
+                        // them, which its first lane stores
+                        window_dots<S, DC, 0>(kb, o, qf, qp, dk4);
+                        window_dots<S, DC, 0>(vb, o, dof, dop, dv4);
+                        float r0, r1;
+                        slot16_sums(dk4, dv4, r0, r1);
+                        float *tab = (g & 8) ? tT : tS;
+                        const unsigned e0 = (g & 4) ? ent.z : ent.x, e1 = (g & 4) ? ent.w : ent.y;
+                        if ((g & 3) == 0) { tab[e0] = r0; tab[e1] = r1; }
+                    } else {
+                        window_dots<S, DC, G>(kb, o, qf, qp, dk4);
+                        window_dots<S, DC, G>(vb, o, dof, dop, dv4);
+                        if (g == 0) {
+                            tS[ent.x] = dk4[0]; tS[ent.y] = dk4[1]; tS[ent.z] = dk4[2]; tS[ent.w] = dk4[3];
+                            tT[ent.x] = dv4[0]; tT[ent.y] = dv4[1]; tT[ent.z] = dv4[2]; tT[ent.w] = dv4[3];
+                        }
                     }
                 }
                 if (lane == 0) tA[kWinDummy] = 0.0;
