@@ -53,19 +53,35 @@ constexpr int kPlaneGradBytes = kPlaneWaves * kPlaneDescPlaces * 8;         // f
 template <typename S, int D>
 __host__ __device__ constexpr int plane_lds_bytes(int L) { return (L + 2) * 2 * D * S::kBytes; }
 
-// global plane of L rows of D elements, `px_bytes` apart -> LDS rows 1..L of the interleaved image
-// (which = 0: K half, 1: V half)
+// The K and V planes of one view (L rows of D elements, `px_bytes` apart in memory) -> LDS rows 1..L of the
+// interleaved image: row q = pixel q - 1 holds the pixel's K row and V row side by side, K in the half q & 1.
+// The rows go from memory to LDS without passing through registers (global_load_lds_dwordx4: lane i of a wave
+// writes 16 bytes at the wave's LDS base + 16 i): a wave fills 1 KB of the image per instruction, every lane
+// fetching the 16 bytes of K or of V that belong at its place, and all of a wave's instructions are in flight
+// together -- a loop of load, wait, LDS write pays one round trip to memory per 16 bytes of a thread, six per
+// view at 18x18, D = 32. Ends with this wave's wait; the caller's barrier follows.
 template <typename S, int D>
-__device__ __forceinline__ void stage_plane(unsigned char *lds, const char *src, int L, unsigned px_bytes, int which)
+__device__ __forceinline__ void stage_plane_pair(unsigned char *lds, const char *ksrc, const char *vsrc, int L,
+                                                 unsigned px_bytes)
 {
-    constexpr int kRow = D * S::kBytes;
-    constexpr int kChunksPerRow = kRow / 16;
-    const int n16 = L * kChunksPerRow;
-    for (int i = threadIdx.x; i < n16; i += (int)blockDim.x) {
-        const int p = i / kChunksPerRow, q = p + 1, c = i % kChunksPerRow;
-        const uint4 t = *reinterpret_cast<const uint4 *>(src + (size_t)p * px_bytes + c * 16);
-        *reinterpret_cast<uint4 *>(lds + (size_t)q * 2 * kRow + ((q & 1) ^ which) * kRow + c * 16) = t;
+    constexpr unsigned kRow = D * S::kBytes;
+    static_assert((kRow & (kRow - 1)) == 0 && kRow >= 16, "row bytes: a power of two");
+    const unsigned total = (unsigned)L * 2u * kRow;                    // bytes of rows 1..L
+    const unsigned wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63u;
+    const unsigned step = (unsigned)__builtin_amdgcn_readfirstlane((int)(blockDim.x >> 6)) * 1024u;
+    const unsigned lds1 = lds_offset(lds) + 2u * kRow;                 // row 1
+    for (unsigned o0 = wave * 1024u; o0 < total; o0 += step) {
+        const unsigned o = o0 + 16u * lane;
+        if (o < total) {                                               // (the last instruction of an image may be part full)
+            const unsigned p = o / (2u * kRow), within = o % (2u * kRow);
+            const unsigned half = within / kRow, col = within % kRow;
+            const bool from_v = ((half ^ (p + 1u)) & 1u) != 0u;
+            const char *src = (from_v ? vsrc : ksrc) + (size_t)p * px_bytes + col;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                             (__attribute__((address_space(3))) void *)(uintptr_t)(lds1 + o0), 16, 0, 0);
+        }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 template <typename S, int D>
@@ -306,8 +322,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void fwd_slot_kernel(
         const size_t plane = dm.kv_plane(pb.b, s2, pb.h) * S::kBytes;
         const unsigned px_bytes = (unsigned)dm.kv_sl * S::kBytes;
         __syncthreads();                                       // the previous view's readers are done
-        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, px_bytes, 0);
-        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, px_bytes, 1);
+        stage_plane_pair<S, D>(smem, (const char *)k_ + plane, (const char *)v_ + plane, dm.L, px_bytes);
         __syncthreads();
 #pragma unroll
         for (int rb = 0; rb < ROWS; ++rb) {
@@ -469,8 +484,7 @@ __global__ __launch_bounds__(kPlaneWaves *kWave) void bwd_dq_slot_kernel(
         const size_t plane = dm.kv_plane(pb.b, s2, pb.h) * S::kBytes;
         const unsigned px_bytes = (unsigned)dm.kv_sl * S::kBytes;
         __syncthreads();
-        stage_plane<S, D>(smem, (const char *)k_ + plane, dm.L, px_bytes, 0);
-        stage_plane<S, D>(smem, (const char *)v_ + plane, dm.L, px_bytes, 1);
+        stage_plane_pair<S, D>(smem, (const char *)k_ + plane, (const char *)v_ + plane, dm.L, px_bytes);
         __syncthreads();
 #pragma unroll
         for (int rb = 0; rb < ROWS; ++rb) {
