@@ -54,13 +54,29 @@ __device__ __forceinline__ bool taps_any(const Taps &tp)
 //
 // One thread per coordinate pair, in memory order (b, s1, l, s2, p).
 // mode 0: count[(b*V+s2)*NK + key] += 1
-// mode 1: sorted[(b*V+s2)*M + cursor[(b*V+s2)*NK + key]++] = (s1*L + l)*P + p, and frac[same] = its (fx, fy)
+// mode 1: the sample's list entry at place (b*V+s2)*M + cursor[(b*V+s2)*NK + key]++: with `records` a 12-byte
+//         record (id = (s1*L + l)*P + p, then its position (fx, fy) inside the cell as two floats) in `sorted` taken
+//         as an array of records -- one scattered store per sample, and the dk/dv kernel reads id and position in
+//         list order instead of gathering the coordinate pair again; without, the id alone as sorted[place] (the
+//         deterministic backward sorts the ids of every list before use).
+struct CellEntry { unsigned id; float fx, fy; };
+__device__ __forceinline__ void store_cell_entry(unsigned *sorted, size_t place, unsigned id, const float2 &ff, int records)
+{
+    if (records) {
+        unsigned *r = sorted + 3 * place;
+        r[0] = id;
+        r[1] = __float_as_uint(ff.x);
+        r[2] = __float_as_uint(ff.y);
+    } else {
+        sorted[place] = id;
+    }
+}
+
 template <int MODE>
 __global__ __launch_bounds__(kBinThreads) void bin_samples_kernel(const float *__restrict__ coords_, Dims dm,
                                                                   int NC, int NK, int vpg,
                                                                   unsigned *__restrict__ counters,
-                                                                  unsigned *__restrict__ sorted,
-                                                                  float2 *__restrict__ frac)
+                                                                  unsigned *__restrict__ sorted, int records)
 {
     const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
     const long long i = (long long)blockIdx.x * kBinThreads + threadIdx.x;
@@ -81,8 +97,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_samples_kernel(const float *_
     } else {
         const unsigned pos = atomicAdd(ctr, 1u);
         const size_t M = (size_t)dm.V * dm.L * dm.P;
-        sorted[grp * M + pos] = (unsigned)ql * (unsigned)dm.P + (unsigned)p;
-        frac[grp * M + pos] = cell_fraction(xy, dm);
+        store_cell_entry(sorted, grp * M + pos, (unsigned)ql * (unsigned)dm.P + (unsigned)p, cell_fraction(xy, dm), records);
     }
 }
 
@@ -99,7 +114,7 @@ constexpr int kBinLdsThreads = 1024;
 template <int MODE>
 __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
     const float *__restrict__ coords_, Dims dm, int NC, int NK, int vpg, int lchunk, int nlc,
-    unsigned *__restrict__ counters, unsigned *__restrict__ sorted, float2 *__restrict__ frac)
+    unsigned *__restrict__ counters, unsigned *__restrict__ sorted, int records)
 {
     extern __shared__ unsigned s_hist[];                 // [V][NC]; mode 1 adds [V][NC] bases
     unsigned *s_base = s_hist + (size_t)dm.V * NC;
@@ -140,8 +155,8 @@ __global__ __launch_bounds__(kBinLdsThreads) void bin_samples_lds_kernel(
             const int p = i % dm.P, s2 = (i / dm.P) % dm.V, l = l0 + i / dm.N;
             const int hidx = s2 * NC + cell_of(tp, dm.Wimg);
             const unsigned pos = s_base[hidx] + atomicAdd(&s_hist[hidx], 1u);
-            sorted[((size_t)b * dm.V + s2) * M + pos] = ((unsigned)s1 * dm.L + l) * (unsigned)dm.P + (unsigned)p;
-            frac[((size_t)b * dm.V + s2) * M + pos] = cell_fraction(xy, dm);
+            store_cell_entry(sorted, ((size_t)b * dm.V + s2) * M + pos, ((unsigned)s1 * dm.L + l) * (unsigned)dm.P + (unsigned)p,
+                             cell_fraction(xy, dm), records);
         }
     }
 }
@@ -287,8 +302,8 @@ struct CellGrid {
 
 // HANDED: the dq kernel has left (p, sm_scale * ds) of every sample in `handed_` (per query row of this head,
 // in the order of the row's coordinates): an entry then costs a gather of that pair and the two rank-1 updates --
-// no taps in registers, no dot products, no exponential. Only with the work list (colour < 0) and with the
-// positions beside the ids (frac).
+// no taps in registers, no dot products, no exponential. Only with the work list (colour < 0) and with
+// records (the positions beside the ids).
 template <typename S, int D, int DC, bool HANDED>
 __global__ __launch_bounds__(kCellWaves *kWave, HANDED ? (DC <= 4 ? 5 : (S::kBytes == 2 ? 3 : 4))
                                                        : DC <= 4 ? (S::kBytes == 2 && D >= 64 ? 5 : 4) : (S::kBytes == 2 ? 3 : 2))
@@ -296,7 +311,7 @@ void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float2 *__restrict__ stats_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
-    const float2 *__restrict__ frac, const uint4 *__restrict__ items, const float2 *__restrict__ handed_,
+    int records, const uint4 *__restrict__ items, const float2 *__restrict__ handed_,
     float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC, CellGrid cg)
 {
     constexpr int G = D / DC;
@@ -402,7 +417,7 @@ void bwd_dkdv_cell_kernel(
     }
     const float qscale = dm.sm_scale * kLog2e;
     const size_t M = (size_t)dm.V * dm.L * dm.P;
-    const unsigned *list = sorted + grp * M;
+    const unsigned *list = sorted + grp * M * (records ? 3u : 1u);      // ids, or 12-byte records (id, fx, fy)
     // Query rows of this wave's (b, h) are addressed as a uniform base plus a 32-bit byte offset
     // (s1*H*L + l) * ROW < V*H*L*D*e <= 2^32 (the shape limits keep one batch item of a tensor below 2^30
     // elements): one add per gather instead of 64-bit address arithmetic per lane.
@@ -417,14 +432,22 @@ void bwd_dkdv_cell_kernel(
     const unsigned view_rows = (unsigned)dm.H * (unsigned)dm.L;
     const float2 *coords = reinterpret_cast<const float2 *>(coords_);
 
-    // Walk the list 64 entries at a time. Sample ids, and the samples' positions in the cell when the binning
-    // pass left them beside the ids (frac; null after the lists were reordered), are fetched one chunk ahead.
-    const float2 *fracl = frac ? frac + grp * M : nullptr;
-    auto load_id = [&](unsigned cstart) -> unsigned {
-        return cstart < hi ? list[min(cstart + (unsigned)lane, hi - 1u)] : 0u;
-    };
-    auto load_frac = [&](unsigned cstart) -> float2 {
-        return (fracl && cstart < hi) ? fracl[min(cstart + (unsigned)lane, hi - 1u)] : make_float2(0.f, 0.f);
+    // Walk the list 64 entries at a time. The entries -- sample id and, when the binning pass left records, the
+    // sample's position in the cell beside it (ids alone after the lists were reordered) -- are fetched one chunk ahead.
+    auto load_entry = [&](unsigned cstart) -> CellEntry {
+        CellEntry e{0u, 0.f, 0.f};
+        if (cstart < hi) {
+            const unsigned at = min(cstart + (unsigned)lane, hi - 1u);
+            if (records) {
+                const unsigned *r = list + 3u * at;
+                e.id = r[0];
+                e.fx = __uint_as_float(r[1]);
+                e.fy = __uint_as_float(r[2]);
+            } else {
+                e.id = list[at];
+            }
+        }
+        return e;
     };
     // HANDED: the entry's pair, gathered one chunk ahead (so the ids are fetched two chunks ahead). The pairs of
     // this launch's (batch, head) pairs lie as [pair][s1][l][sample]; those of this wave's pair are a uniform base
@@ -460,8 +483,10 @@ void bwd_dkdv_cell_kernel(
                       "two blocks fit before the first trip; places written by one block never reach the trips in flight");
         // (requests past the end of the list repeat its last entry: no request sits under a branch, and the number
         // of requests in flight at any point is the same on every path -- the compiler's waits are exact then)
-        auto load_id_q = [&](unsigned cstart) -> unsigned { return list[min(cstart + (unsigned)lane, hi - 1u)]; };
-        auto load_frac_q = [&](unsigned cstart) -> float2 { return fracl[min(cstart + (unsigned)lane, hi - 1u)]; };
+        auto load_entry_q = [&](unsigned cstart) -> CellEntry {
+            const unsigned *r = list + 3u * min(cstart + (unsigned)lane, hi - 1u);
+            return CellEntry{r[0], __uint_as_float(r[1]), __uint_as_float(r[2])};
+        };
         auto prepare = [&](unsigned cstart, int tail, unsigned sid, float2 ff, float2 pdv) -> int {
             const unsigned ql = dm.divP.div(sid);                                  // ql = s1*L + l
             const unsigned s1 = dm.divL.div(ql), l = ql - s1 * (unsigned)dm.L;
@@ -531,14 +556,13 @@ void bwd_dkdv_cell_kernel(
         s_qrowq[wave][lane] = 0u;
         s_qrowq[wave][kWave + lane] = 0u;
         int head = 0, tail;
-        unsigned id_a;
+        CellEntry e_a;
         {
-            const unsigned id0 = load_id_q(lo), id1 = load_id_q(lo + kWave);
-            id_a = load_id_q(lo + 2 * kWave);
-            const float2 ff0 = load_frac_q(lo), ff1 = load_frac_q(lo + kWave);
-            const float2 pd0 = load_pair(id0), pd1 = load_pair(id1);
-            tail = prepare(lo, 0, id0, ff0, pd0);
-            tail += prepare(lo + kWave, tail, id1, ff1, pd1);
+            const CellEntry e0 = load_entry_q(lo), e1 = load_entry_q(lo + kWave);
+            e_a = load_entry_q(lo + 2 * kWave);
+            const float2 pd0 = load_pair(e0.id), pd1 = load_pair(e1.id);
+            tail = prepare(lo, 0, e0.id, make_float2(e0.fx, e0.fy), pd0);
+            tail += prepare(lo + kWave, tail, e1.id, make_float2(e1.fx, e1.fy), pd1);
         }
         wave_lds_sync();
         issue_q(0);
@@ -546,8 +570,8 @@ void bwd_dkdv_cell_kernel(
         const int tap_lane = (lane & 3) * (kRing / 4) + slot;                       // this lane's tap, its slot's four entries (in float4 units)
         for (unsigned cnext = lo + 2 * kWave;; cnext += kWave) {
             const bool more = cnext < hi;                      // a block is left to merge
-            const float2 pd_a = load_pair(id_a), ff_a = load_frac_q(cnext);
-            const unsigned id_n = load_id_q(cnext + kWave);
+            const float2 pd_a = load_pair(e_a.id);
+            const CellEntry e_n = load_entry_q(cnext + kWave);
             __builtin_amdgcn_sched_barrier(0);                 // (requested here, not where they are used)
             // (at least one trip: a whole block adds QT merged entries or more to the QT or more that the trips before left)
             const int stop = more ? tail - 2 * QT : tail - 1;
@@ -572,35 +596,32 @@ void bwd_dkdv_cell_kernel(
             } while (head <= stop);
             if (!more) break;
             wave_lds_sync();
-            tail += prepare(cnext, tail, id_a, ff_a, pd_a);
+            tail += prepare(cnext, tail, e_a.id, make_float2(e_a.fx, e_a.fy), pd_a);
             wave_lds_sync();
-            id_a = id_n;
+            e_a = e_n;
         }
     }
-    unsigned id_nxt = kQuad ? 0u : load_id(lo);
-    float2 ff_nxt = kQuad ? make_float2(0.f, 0.f) : load_frac(lo);
-    unsigned id_nxt2 = 0u;
+    CellEntry e_nxt = kQuad ? CellEntry{0u, 0.f, 0.f} : load_entry(lo), e_nxt2{0u, 0.f, 0.f};
     float2 pd_nxt = make_float2(0.f, 0.f);
     if constexpr (HANDED && !kQuad) {
-        id_nxt2 = load_id(lo + kWave);
-        pd_nxt = load_pair(id_nxt);
+        e_nxt2 = load_entry(lo + kWave);
+        pd_nxt = load_pair(e_nxt.id);
     }
     for (unsigned c0 = lo; c0 < (kQuad ? lo : hi); c0 += kWave) {
-        const unsigned id = id_nxt;
-        float2 ff = ff_nxt;
+        const unsigned id = e_nxt.id;
+        float2 ff = make_float2(e_nxt.fx, e_nxt.fy);
         const float2 pdv = pd_nxt;
         if constexpr (HANDED) {
-            id_nxt = id_nxt2;
-            id_nxt2 = load_id(c0 + 2 * kWave);
-            pd_nxt = load_pair(id_nxt);
+            e_nxt = e_nxt2;
+            e_nxt2 = load_entry(c0 + 2 * kWave);
+            pd_nxt = load_pair(e_nxt.id);
         } else {
-            id_nxt = load_id(c0 + kWave);
+            e_nxt = load_entry(c0 + kWave);
         }
-        ff_nxt = load_frac(c0 + kWave);
         // one list entry per lane: weights and query row
         const unsigned ql = dm.divP.div(id), p = id - ql * (unsigned)dm.P;     // ql = s1*L + l
         const unsigned s1 = dm.divL.div(ql), l = ql - s1 * (unsigned)dm.L;
-        if (!fracl) {
+        if (!records) {
             const size_t ci = (((size_t)b * dm.V * dm.L + ql) * dm.V + s2) * (size_t)dm.P + p;
             ff = cell_fraction(coords[ci], dm);
         }

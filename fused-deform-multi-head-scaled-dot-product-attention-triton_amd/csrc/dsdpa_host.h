@@ -196,8 +196,9 @@ inline bool slab_path_fits(size_t V, size_t Himg, size_t Wimg, size_t D, size_t 
 //   delta    rows floats                     dout.out per query row
 //   counters B*V*NC u32                      per (batch, key view) cell counts, then fill cursors
 //   start    B*V*(NC+1) u32                  exclusive scan of the counts
-//   sorted   B*V*(V*L*P) u32                 sample ids ordered by cell
-//   frac     B*V*(V*L*P) x 8 bytes           (fx, fy) of the same samples, same order
+//   sorted   B*V*(V*L*P) u32                 the cell lists: 12-byte records (sample id, its position (fx, fy) in the
+//   frac     B*V*(V*L*P) x 8 bytes           cell) that run from `sorted` on through `frac`, which follows it; the
+//                                            deterministic backward keeps plain ids in `sorted` (and sorts them)
 //   items    B*V*wmax x 16 bytes             work list of the dk/dv kernel: (cell, first entry, end) per item
 //   handed   bhg*V*L*(V*P) x 8 bytes         (p, sm_scale*ds) per query*sample of one GROUP of bhg (batch, head) pairs,
 //                                            dq kernel -> dk/dv kernel (shapes on the gather kernels only); at most

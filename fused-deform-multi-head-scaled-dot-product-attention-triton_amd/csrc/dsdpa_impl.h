@@ -505,13 +505,14 @@ template <typename S, int D> struct CellChunk {
     static constexpr int value = S::kBytes == 2 ? (D <= 64 ? 4 : 8) : (D <= 128 ? 4 : 8);
 };
 
+// records: the lists as 12-byte records (id and position in the cell) from wl.sorted on, through the room of
+// wl.frac behind it; else plain ids in wl.sorted (the deterministic backward, which sorts them).
 static inline int launch_binning(const float *coords, const Dims &dm, const WorkspaceLayout &wl, char *ws,
-                                 hipStream_t st)
+                                 int records, hipStream_t st)
 {
     unsigned *counters = (unsigned *)(ws + wl.counters);
     unsigned *start = (unsigned *)(ws + wl.start);
     unsigned *sorted = (unsigned *)(ws + wl.sorted);
-    float2 *frac = (float2 *)(ws + wl.frac);
     const size_t hist_bytes = (size_t)dm.V * wl.NC * sizeof(unsigned);
     // each of the three launches carries its own pair of events: the timer's slot 3 adds up their busy time
     ScopedKernelTimer t_count(3, st), t_scan(3, st), t_fill(3, st);
@@ -532,13 +533,13 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
         if (int rc = allow_full_lds(k1, lds_set[1])) return rc;
         DSDPA_LAUNCH(k0, dim3((unsigned)blocks), dim3(kBinLdsThreads), hist_bytes, st,
                               t_count.start(), t_count.stop(),
-                           coords, dm, wl.NC, wl.NK, wl.vpg, lchunk, nlc, counters, sorted, frac);
+                           coords, dm, wl.NC, wl.NK, wl.vpg, lchunk, nlc, counters, sorted, records);
         DSDPA_LAUNCH(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st,
                               t_scan.start(), t_scan.stop(), counters, start, wl.NK, wl.NC, wl.piece, wl.wmax,
                               (uint4 *)(ws + wl.items));
         DSDPA_LAUNCH(k1, dim3((unsigned)blocks), dim3(kBinLdsThreads), 2 * hist_bytes, st,
                               t_fill.start(), t_fill.stop(),
-                           coords, dm, wl.NC, wl.NK, wl.vpg, lchunk, nlc, counters, sorted, frac);
+                           coords, dm, wl.NC, wl.NK, wl.vpg, lchunk, nlc, counters, sorted, records);
         return check_launch();
     }
     const long long total = (long long)dm.B * dm.V * dm.L * dm.N;
@@ -546,13 +547,13 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
     if (blocks > 0x7fffffffll) return DSDPA_ERR_TOO_LARGE;
     DSDPA_LAUNCH(bin_samples_kernel<0>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
                           t_count.start(), t_count.stop(),
-                       coords, dm, wl.NC, wl.NK, wl.vpg, counters, sorted, frac);
+                       coords, dm, wl.NC, wl.NK, wl.vpg, counters, sorted, records);
     DSDPA_LAUNCH(bin_scan_kernel, dim3((unsigned)(dm.B * dm.V)), dim3(1024), 0, st,
                           t_scan.start(), t_scan.stop(), counters, start, wl.NK, wl.NC, wl.piece, wl.wmax,
                               (uint4 *)(ws + wl.items));
     DSDPA_LAUNCH(bin_samples_kernel<1>, dim3((unsigned)blocks), dim3(kBinThreads), 0, st,
                           t_fill.start(), t_fill.stop(),
-                       coords, dm, wl.NC, wl.NK, wl.vpg, counters, sorted, frac);
+                       coords, dm, wl.NC, wl.NK, wl.vpg, counters, sorted, records);
     return check_launch();
 }
 
@@ -560,7 +561,7 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
 template <typename S, int D>
 int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const float *coords,
                          const float2 *stats, const void *dout, const unsigned *start, const unsigned *sorted,
-                         const float2 *frac, const uint4 *items, unsigned wmax, const float2 *handed,
+                         int records, const uint4 *items, unsigned wmax, const float2 *handed,
                          float *dk_acc, float *dv_acc, const Dims &dm, int NC, bool deterministic, int bh0, int nbh,
                          hipStream_t st)
 {
@@ -586,14 +587,14 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
         cg.div_h = FastDiv::make((unsigned)dm.H);
         const unsigned blocks = (unsigned)((nwork + kCellWaves - 1) / kCellWaves);
         const bool first = colour <= 0, last = colour < 0 || colour == 3;
-        if (handed && colour < 0 && frac)
+        if (handed && colour < 0 && records)
             DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC, true>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
                                   first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
-                                  stats, dout, start, sorted, frac, items, handed, dk_acc, dv_acc, dm, NC, cg);
+                                  stats, dout, start, sorted, records, items, handed, dk_acc, dv_acc, dm, NC, cg);
         else
             DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC, false>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
                                   first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
-                                  stats, dout, start, sorted, frac, items, handed, dk_acc, dv_acc, dm, NC, cg);
+                                  stats, dout, start, sorted, records, items, handed, dk_acc, dv_acc, dm, NC, cg);
     }
     return check_launch();
 }
@@ -674,8 +675,8 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
     const float4 *desc_g = (const float4 *)(ws + wl.desc + wl.dl.g);
     const unsigned *start = (const unsigned *)(ws + wl.start);
     const unsigned *sorted = (const unsigned *)(ws + (deterministic ? wl.sorted2 : wl.sorted));
-    // (the reordered lists of the deterministic backward have no positions beside them: coordinates are read again)
-    const float2 *frac = deterministic ? nullptr : (const float2 *)(ws + wl.frac);
+    // (the reordered lists of the deterministic backward are ids without positions beside them: coordinates are read again)
+    const int records = deterministic ? 0 : 1;
     // (p, sm_scale * ds) per query*sample from the dq kernel to the dk/dv kernel, where the layout has room for it
     // (shapes on the gather dq kernel, which then runs before dk/dv on the same stream)
     float2 *handed = (wl.handed_bytes && cell_binned && !staged) ? (float2 *)(ws + wl.handed) : nullptr;
@@ -723,7 +724,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
                            stats, (size_t)dm.rows, D);
         if ((rc = check_launch()) != DSDPA_OK) return rc;
     }
-    if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, bst)) != DSDPA_OK) return rc;
+    if (cell_binned && (rc = launch_binning(coords, dm, wl, ws, deterministic ? 0 : 1, bst)) != DSDPA_OK) return rc;
     if (deterministic && (rc = launch_list_ordering(dm, wl, ws, bst)) != DSDPA_OK) return rc;
     float2 *dq_stats = side_on ? nullptr : stats;       // the dq kernel writes them only when dk/dv runs behind it
     // With the pairs handed over the two kernels go group by group of (batch, head) pairs: the buffer holds one
@@ -746,7 +747,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const float *coords, c
                         : launch_bwd_dq_gather<S, DD>(q, k, v, coords, out, lse, dout, dq, dq_stats, dcoords,   \
                                                       handed, dm, bh0, nbh, st);                                \
             if (rc == DSDPA_OK && cell_binned)                                                                  \
-                rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, stats, dout, start, sorted, frac,             \
+                rc = launch_bwd_dkdv_cell<S, DD>(q, k, v, coords, stats, dout, start, sorted, records,          \
                                                  (const uint4 *)(ws + wl.items), wl.wmax, handed, dk_acc,       \
                                                  dv_acc, dm, wl.NK, deterministic, bh0, nbh, bst);              \
             else if (rc == DSDPA_OK)                                                                            \
