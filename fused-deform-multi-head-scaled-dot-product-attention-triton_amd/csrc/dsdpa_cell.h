@@ -304,23 +304,23 @@ struct CellGrid {
 // in the order of the row's coordinates): an entry then costs a gather of that pair and the two rank-1 updates --
 // no taps in registers, no dot products, no exponential. Only with the work list (colour < 0) and with
 // records (the positions beside the ids).
-template <typename S, int D, int DC, bool HANDED>
+template <typename S, int D, int DC, bool HANDED, bool RECORDS>
 __global__ __launch_bounds__(kCellWaves *kWave, HANDED ? (DC <= 4 ? 5 : (S::kBytes == 2 ? 3 : 4))
                                                        : DC <= 4 ? (S::kBytes == 2 && D >= 64 ? 5 : 4) : (S::kBytes == 2 ? 3 : 2))
 void bwd_dkdv_cell_kernel(
     const void *__restrict__ q_, const void *__restrict__ k_, const void *__restrict__ v_,
     const float *__restrict__ coords_, const float2 *__restrict__ stats_,
     const void *__restrict__ dout_, const unsigned *__restrict__ start, const unsigned *__restrict__ sorted,
-    int records, const uint4 *__restrict__ items, const float2 *__restrict__ handed_,
+    const uint4 *__restrict__ items, const float2 *__restrict__ handed_,
     float *__restrict__ dk_acc, float *__restrict__ dv_acc, Dims dm, int NC, CellGrid cg)
 {
     constexpr int G = D / DC;
     constexpr int NS = kWave / G;
     static_assert(G >= 4 && G <= 64 && G * DC == D, "lane split (a block of four lanes must not straddle two samples)");
-    __shared__ float4 s_w[kCellWaves][kWave];
-    __shared__ unsigned s_row[kCellWaves][kWave];           // byte offset of the entry's query row in dout (and its (lse, delta))
-    __shared__ unsigned s_qrow[kCellWaves][kWave];          // ... in q (which may be strided)
-    __shared__ float2 s_f[S::kBytes == 2 ? kCellWaves : 1][kWave];          // 16-bit storage: (fx, fy) of the entry
+    __shared__ float4 s_w[kCellWaves][2 * kWave];           // two sets of entry tables, used in turn
+    __shared__ unsigned s_row[kCellWaves][2 * kWave];       // byte offset of the entry's query row in dout (and its (lse, delta))
+    __shared__ unsigned s_qrow[kCellWaves][2 * kWave];      // ... in q (which may be strided)
+    __shared__ float2 s_f[S::kBytes == 2 ? kCellWaves : 1][2 * kWave];      // 16-bit storage: (fx, fy) of the entry
     __shared__ __attribute__((aligned(16))) float s_flush[kCellWaves][4 * D];                 // the flush: four rows of dk, then of dv
     constexpr bool kQuad = HANDED && S::kBytes == 2 && DC >= 8;            // four-entry trips (below)
     // kQuad: a ring of merged entries; the coefficients as [tap][place]
@@ -417,7 +417,8 @@ void bwd_dkdv_cell_kernel(
     }
     const float qscale = dm.sm_scale * kLog2e;
     const size_t M = (size_t)dm.V * dm.L * dm.P;
-    const unsigned *list = sorted + grp * M * (records ? 3u : 1u);      // ids, or 12-byte records (id, fx, fy)
+    static_assert(RECORDS || !HANDED, "the pairs are handed over to lists of records only");
+    const unsigned *list = sorted + grp * M * (RECORDS ? 3u : 1u);      // ids, or 12-byte records (id, fx, fy)
     // Query rows of this wave's (b, h) are addressed as a uniform base plus a 32-bit byte offset
     // (s1*H*L + l) * ROW < V*H*L*D*e <= 2^32 (the shape limits keep one batch item of a tensor below 2^30
     // elements): one add per gather instead of 64-bit address arithmetic per lane.
@@ -432,23 +433,6 @@ void bwd_dkdv_cell_kernel(
     const unsigned view_rows = (unsigned)dm.H * (unsigned)dm.L;
     const float2 *coords = reinterpret_cast<const float2 *>(coords_);
 
-    // Walk the list 64 entries at a time. The entries -- sample id and, when the binning pass left records, the
-    // sample's position in the cell beside it (ids alone after the lists were reordered) -- are fetched one chunk ahead.
-    auto load_entry = [&](unsigned cstart) -> CellEntry {
-        CellEntry e{0u, 0.f, 0.f};
-        if (cstart < hi) {
-            const unsigned at = min(cstart + (unsigned)lane, hi - 1u);
-            if (records) {
-                const unsigned *r = list + 3u * at;
-                e.id = r[0];
-                e.fx = __uint_as_float(r[1]);
-                e.fy = __uint_as_float(r[2]);
-            } else {
-                e.id = list[at];
-            }
-        }
-        return e;
-    };
     // HANDED: the entry's pair, gathered one chunk ahead (so the ids are fetched two chunks ahead). The pairs of
     // this launch's (batch, head) pairs lie as [pair][s1][l][sample]; those of this wave's pair are a uniform base
     // plus a 32-bit byte offset (the host checks V*L*N*8 < 2^32).
@@ -601,67 +585,65 @@ void bwd_dkdv_cell_kernel(
             e_a = e_n;
         }
     }
-    CellEntry e_nxt = kQuad ? CellEntry{0u, 0.f, 0.f} : load_entry(lo), e_nxt2{0u, 0.f, 0.f};
-    float2 pd_nxt = make_float2(0.f, 0.f);
-    if constexpr (HANDED && !kQuad) {
-        e_nxt2 = load_entry(lo + kWave);
-        pd_nxt = load_pair(e_nxt.id);
-    }
-    for (unsigned c0 = lo; c0 < (kQuad ? lo : hi); c0 += kWave) {
-        const unsigned id = e_nxt.id;
-        float2 ff = make_float2(e_nxt.fx, e_nxt.fy);
-        const float2 pdv = pd_nxt;
-        if constexpr (HANDED) {
-            e_nxt = e_nxt2;
-            e_nxt2 = load_entry(c0 + 2 * kWave);
-            pd_nxt = load_pair(e_nxt.id);
-        } else {
-            e_nxt = load_entry(c0 + kWave);
-        }
-        // one list entry per lane: weights and query row
-        const unsigned ql = dm.divP.div(id), p = id - ql * (unsigned)dm.P;     // ql = s1*L + l
-        const unsigned s1 = dm.divL.div(ql), l = ql - s1 * (unsigned)dm.L;
-        if (!records) {
-            const size_t ci = (((size_t)b * dm.V * dm.L + ql) * dm.V + s2) * (size_t)dm.P + p;
-            ff = cell_fraction(coords[ci], dm);
-        }
-        // Plain bilinear weights, not masked: every sample of this list lies in this cell, whose taps
-        // outside the image were loaded as zeros above and are skipped by the flush below.
-        const float fx = ff.x, fy = ff.y;
-        const float gx = 1.0f - fx, gy = 1.0f - fy;
-        // entries past the end of the list repeat its last sample with zero weights: they add nothing
-        const bool live = c0 + (unsigned)lane < hi;
-        wave_lds_sync();
-        if constexpr (HANDED) {
-            // (fx, fy, p, sm_scale * ds); a dead entry adds nothing
-            s_w[wave][lane] = make_float4(fx, fy, live ? pdv.x : 0.f, live ? pdv.y : 0.f);
-        } else if constexpr (kPacked) {
-            s_w[wave][lane] = live ? make_float4(gx * gy, fx * gy, gx * fy, fx * fy) : make_float4(0.f, 0.f, 0.f, 0.f);
-            s_f[wave][lane] = make_float2(fx, live ? fy : __int_as_float(0x7fc00000));     // NaN marks a dead entry
-        } else {
-            s_w[wave][lane] = make_float4(fx, fy, fx * fy, live ? 1.0f : 0.0f);
-        }
-        s_row[wave][lane] = (s1 * view_rows + l) * kRowBytes;
-        s_qrow[wave][lane] = (s1 * (unsigned)dm.q_sv + l * (unsigned)dm.q_sl) * S::kBytes;
-        wave_lds_sync();
-        const int cnt = (int)min((unsigned)kWave, hi - c0);
-        // The NS samples of a trip need their query rows (q, dout, lse, delta) from memory, a round trip of
-        // several hundred nanoseconds that the two or three other waves of the SIMD do not cover. So the rows
-        // of trip t+1 are requested before trip t is worked on: two sets of row registers, used in turn (the
-        // loop is unrolled by two so that no set is ever copied).
-        auto issue = [&](int j0, RowFetch<kRowWords> &f) {
-            const unsigned r = s_row[wave][j0 + slot];
+    if constexpr (!kQuad) {
+        // One list entry per lane and 64-entry block: weights and query row go into tables in LDS, which the slots
+        // walk NS entries a trip. Two sets of tables, used in turn: the next block's are made while this block is
+        // worked on, so that the last trip of a block can request the rows of the next block's first. The NS
+        // samples of a trip need their query rows (q, dout, lse, delta) from memory, a round trip of several
+        // hundred nanoseconds that the other waves of the SIMD do not cover: the rows of trip t+1 are requested
+        // before trip t is worked on (two sets of row registers, the loop unrolled by two so that no set is ever
+        // copied). Every request is unconditional -- entries past the end of the list repeat its last one, with
+        // zero weights, and the last request of a list is never used -- and the trip loop runs at least once: the
+        // number of requests in flight is the same on every path, so the compiler's waits name exactly the
+        // younger requests instead of "everything" (a request under a branch, or a loop that may run zero times,
+        // makes the wait at the join a wait for all outstanding loads, which undoes the overlap).
+        auto load_entry_c = [&](unsigned cstart) -> CellEntry {
+            const unsigned at = min(cstart + (unsigned)lane, hi - 1u);
+            if constexpr (RECORDS) {
+                const unsigned *r = list + 3u * at;
+                return CellEntry{r[0], __uint_as_float(r[1]), __uint_as_float(r[2])};
+            } else {
+                return CellEntry{list[at], 0.f, 0.f};
+            }
+        };
+        auto tables = [&](unsigned cstart, int buf, const CellEntry &e, const float2 &pdv) {
+            const unsigned ql = dm.divP.div(e.id), p = e.id - ql * (unsigned)dm.P;     // ql = s1*L + l
+            const unsigned s1 = dm.divL.div(ql), l = ql - s1 * (unsigned)dm.L;
+            float2 ff = make_float2(e.fx, e.fy);
+            if constexpr (!RECORDS) {
+                const size_t ci = (((size_t)b * dm.V * dm.L + ql) * dm.V + s2) * (size_t)dm.P + p;
+                ff = cell_fraction(coords[ci], dm);
+            }
+            // Plain bilinear weights, not masked: every sample of this list lies in this cell, whose taps
+            // outside the image were loaded as zeros above and are skipped by the flush below.
+            const float fx = ff.x, fy = ff.y;
+            const float gx = 1.0f - fx, gy = 1.0f - fy;
+            const bool live = cstart + (unsigned)lane < hi;           // a dead entry adds nothing
+            const int at = buf * kWave + lane;
+            if constexpr (HANDED) {
+                s_w[wave][at] = make_float4(fx, fy, live ? pdv.x : 0.f, live ? pdv.y : 0.f);     // (fx, fy, p, sm_scale * ds)
+            } else if constexpr (kPacked) {
+                s_w[wave][at] = live ? make_float4(gx * gy, fx * gy, gx * fy, fx * fy) : make_float4(0.f, 0.f, 0.f, 0.f);
+                s_f[wave][at] = make_float2(fx, live ? fy : __int_as_float(0x7fc00000));          // NaN marks a dead entry
+            } else {
+                s_w[wave][at] = make_float4(fx, fy, fx * fy, live ? 1.0f : 0.0f);
+            }
+            s_row[wave][at] = (s1 * view_rows + l) * kRowBytes;
+            s_qrow[wave][at] = (s1 * (unsigned)dm.q_sv + l * (unsigned)dm.q_sl) * S::kBytes;
+        };
+        auto issue = [&](int buf, int j0, RowFetch<kRowWords> &f) {
+            const unsigned r = s_row[wave][buf * kWave + j0 + slot];
             const unsigned roff = r + lane_byte, soff = r >> kRowToPairShift;
-            load_words<kRowWords>(q_bh + (s_qrow[wave][j0 + slot] + lane_byte), f.qw);
+            load_words<kRowWords>(q_bh + (s_qrow[wave][buf * kWave + j0 + slot] + lane_byte), f.qw);
             load_words<kRowWords>(do_bh + roff, f.dw);
             if constexpr (!HANDED) f.ld = *(const float2 *)(stats_bh + soff);
         };
-        auto consume = [&](int j0, const RowFetch<kRowWords> &f) {
+        auto consume = [&](int buf, int j0, const RowFetch<kRowWords> &f) {
             float qf[DC], dof[DC];
             widen_words<S, DC>(f.qw, qf);
             widen_words<S, DC>(f.dw, dof);
             if constexpr (HANDED) {
-                const float4 w4 = s_w[wave][j0 + slot];                 // (fx, fy, p, sm_scale * ds)
+                const float4 w4 = s_w[wave][buf * kWave + j0 + slot];                 // (fx, fy, p, sm_scale * ds)
                 const float cl = fmaf(w4.x, row_sx, row_ox) * fmaf(w4.y, row_sy, row_oy);
                 const float ck = cl * w4.w, cv = cl * w4.z;
 #pragma unroll
@@ -670,7 +652,7 @@ void bwd_dkdv_cell_kernel(
                     mV[d] = block_outer_fma(cv, dof[d], mV[d]);
                 }
             } else {
-            const float4 w = s_w[wave][j0 + slot];
+            const float4 w = s_w[wave][buf * kWave + j0 + slot];
             const float lse = f.ld.x, delta = f.ld.y;
             float dot = 0.f, dp = 0.f;
             if constexpr (kPacked) {
@@ -701,7 +683,7 @@ void bwd_dkdv_cell_kernel(
             // so they share the sample and supply its four coefficients between them.
             float fxs, fys;
             if constexpr (kPacked) {
-                const float2 ff = s_f[wave][j0 + slot];
+                const float2 ff = s_f[wave][buf * kWave + j0 + slot];
                 fxs = ff.x;
                 fys = ff.y;
             } else {
@@ -718,22 +700,64 @@ void bwd_dkdv_cell_kernel(
             }
             }
         };
-        // Trips go in pairs, and every request is unconditional: entries past the end of the list (up to the
-        // end of the 64-entry block) are dead ones with valid row offsets and zero weights, and the last
-        // request of a block wraps to entry 0 and is never used. (A request under a branch makes the compiler
-        // wait for all outstanding loads at the join, which undoes the overlap.)
         static_assert(kWave % (2 * NS) == 0, "a block of 64 entries is a whole number of trip pairs");
+        // entries are fetched one block ahead of their tables; with the pairs handed over two, and the pairs -- whose
+        // addresses come from the ids -- one
+        CellEntry e_a, e_b{0u, 0.f, 0.f};
+        float2 pd_a = make_float2(0.f, 0.f);
+        {
+            const CellEntry e0 = load_entry_c(lo);
+            e_a = load_entry_c(lo + kWave);
+            float2 pd0 = make_float2(0.f, 0.f);
+            if constexpr (HANDED) {
+                e_b = load_entry_c(lo + 2 * kWave);
+                pd0 = load_pair(e0.id);
+                pd_a = load_pair(e_a.id);
+            }
+            tables(lo, 0, e0, pd0);
+        }
+        wave_lds_sync();
         RowFetch<kRowWords> fa, fb;
-        issue(0, fa);
-        for (int j0 = 0; j0 < cnt; j0 += 2 * NS) {
-            issue(j0 + NS, fb);
-            __builtin_amdgcn_sched_barrier(0);         // (keeps the requests where they are written)
-            consume(j0, fa);
-            __builtin_amdgcn_sched_barrier(0);
-            issue((j0 + 2 * NS) & (kWave - 1), fa);
-            __builtin_amdgcn_sched_barrier(0);
-            consume(j0 + NS, fb);
-            __builtin_amdgcn_sched_barrier(0);
+        issue(0, 0, fa);
+        int cur = 0;
+        for (unsigned c0 = lo;; c0 += kWave) {
+            const bool has_next = c0 + kWave < hi;
+            CellEntry e_c;
+            float2 pd_b = make_float2(0.f, 0.f);
+            if constexpr (HANDED) {
+                pd_b = load_pair(e_b.id);
+                e_c = load_entry_c(c0 + 3 * kWave);
+            } else {
+                e_c = load_entry_c(c0 + 2 * kWave);
+            }
+            __builtin_amdgcn_sched_barrier(0);         // (requested here, not where they are used)
+            wave_lds_sync();
+            tables(c0 + kWave, cur ^ 1, e_a, pd_a);
+            wave_lds_sync();
+            const int cnt = (int)min((unsigned)kWave, hi - c0);
+            int j0 = 0;
+            do {
+                issue(cur, j0 + NS, fb);
+                __builtin_amdgcn_sched_barrier(0);     // (keeps the requests where they are written)
+                consume(cur, j0, fa);
+                __builtin_amdgcn_sched_barrier(0);
+                // the next pair of trips: of this block, or the first of the next block
+                const bool over = j0 + 2 * NS >= kWave && has_next;
+                issue(over ? cur ^ 1 : cur, (j0 + 2 * NS) & (kWave - 1), fa);
+                __builtin_amdgcn_sched_barrier(0);
+                consume(cur, j0 + NS, fb);
+                __builtin_amdgcn_sched_barrier(0);
+                j0 += 2 * NS;
+            } while (j0 < cnt);
+            if (!has_next) break;
+            if constexpr (HANDED) {
+                e_a = e_b;
+                pd_a = pd_b;
+                e_b = e_c;
+            } else {
+                e_a = e_c;
+            }
+            cur ^= 1;
         }
     }
 #pragma unroll

@@ -588,13 +588,17 @@ int launch_bwd_dkdv_cell(const void *q, const void *k, const void *v, const floa
         const unsigned blocks = (unsigned)((nwork + kCellWaves - 1) / kCellWaves);
         const bool first = colour <= 0, last = colour < 0 || colour == 3;
         if (handed && colour < 0 && records)
-            DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC, true>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
+            DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC, true, true>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
                                   first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
-                                  stats, dout, start, sorted, records, items, handed, dk_acc, dv_acc, dm, NC, cg);
+                                  stats, dout, start, sorted, items, handed, dk_acc, dv_acc, dm, NC, cg);
+        else if (records)
+            DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC, false, true>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
+                                  first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
+                                  stats, dout, start, sorted, items, handed, dk_acc, dv_acc, dm, NC, cg);
         else
-            DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC, false>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
+            DSDPA_LAUNCH((bwd_dkdv_cell_kernel<S, D, DC, false, false>), dim3(blocks), dim3(kCellWaves * kWave), 0, st,
                                   first ? timer.start() : nullptr, last ? timer.stop() : nullptr, q, k, v, coords,
-                                  stats, dout, start, sorted, records, items, handed, dk_acc, dv_acc, dm, NC, cg);
+                                  stats, dout, start, sorted, items, handed, dk_acc, dv_acc, dm, NC, cg);
     }
     return check_launch();
 }
