@@ -485,16 +485,19 @@ def test_backward_recomputes_where_one_pair_exceeds_the_hand_over_buffer():
     assert rel(dv, rdv) < TOL_BWD[dtype]
 
 
-@pytest.mark.parametrize("spread, seed", [("uniform", 101), ("clustered", 102), ("tight", 103)])
-def test_backward_merges_entries_of_one_query_in_long_lists(spread, seed):
+@pytest.mark.parametrize("spread, seed, D, dtype", [
+    ("uniform", 101, 128, torch.bfloat16), ("clustered", 102, 128, torch.bfloat16), ("tight", 103, 128, torch.bfloat16),
+    ("clustered", 104, 128, torch.float16), ("clustered", 105, 256, torch.float16), ("uniform", 106, 256, torch.bfloat16)],
+    ids=["uniform", "clustered", "tight", "clustered-fp16", "clustered-d256-fp16", "uniform-d256"])
+def test_backward_merges_entries_of_one_query_in_long_lists(spread, seed, D, dtype):
     """D = 128 in bf16 with the pairs handed over: the dk/dv kernel merges neighbouring list entries of one query
     and keeps the merged ones in a ring. 20x20 images (too large for the staged kernels) with 64 samples from 4 views
     give lists of some 230 entries
     per cell -- several 64-entry blocks, so the ring wraps. `uniform`: hardly any entry merges (the two blocks
     merged before the first trip fill the ring to its last place); `clustered`: sigma of one pixel, about half of
-    them merge; `tight`: sigma of a tenth of a pixel, runs longer than the four entries that merge into one."""
-    B, V, H, Himg, Wimg, D, P = 1, 4, 2, 20, 20, 128, 64
-    dtype = torch.bfloat16
+    them merge; `tight`: sigma of a tenth of a pixel, runs longer than the four entries that merge into one.
+    D = 256: trips of eight merged entries instead of sixteen."""
+    B, V, H, Himg, Wimg, P = 1, 4, 2 if D == 128 else 1, 20, 20, 64
     say(f"[case] merged entries {spread} B{B} V{V} H{H} {Himg}x{Wimg} D{D} P{P} {dtype}")
     g = torch.Generator().manual_seed(seed)
     L = Himg * Wimg
