@@ -517,9 +517,19 @@ static inline int launch_binning(const float *coords, const Dims &dm, const Work
     // each of the three launches carries its own pair of events: the timer's slot 3 adds up their busy time
     ScopedKernelTimer t_count(3, st), t_scan(3, st), t_fill(3, st);
     if (2 * hist_bytes <= (size_t)kLdsBytes - 1024) {
-        // LDS-aggregated passes: a workgroup per run of about 4k samples of one (b, s1); 8k when the
-        // histogram is large, since every workgroup walks all of it twice (measured on 18x18 and 48x48)
-        int lchunk = (dm.V * wl.NC < 4096 ? 4096 : 8192) / dm.N;
+        // LDS-aggregated passes: a workgroup per run of about 4k samples of one (b, s1); more when the histogram
+        // is large, since every workgroup walks all of it twice: twice its counters, between 8k and 32k samples, as
+        // long as that leaves 128 workgroups (64x64, 4 views, 8.4 M samples: 0.203 ms for the three launches with
+        // runs of 8k, 0.179 with 16k or 32k, 0.229 with 64k; 48x48, 6 views, 5.3 M: 0.177 / 0.174 / 0.157 / 0.221;
+        // 32x32, 6 views, 0.6 M: 0.037 / 0.050 / 0.072)
+        const long long hist_entries = (long long)dm.V * wl.NC, total_samples = (long long)dm.B * dm.V * dm.L * dm.N;
+        long long run = 4096;
+        if (hist_entries >= 4096) {
+            run = 2 * hist_entries < 8192 ? 8192 : (2 * hist_entries > 32768 ? 32768 : 2 * hist_entries);
+            while (run > 8192 && total_samples / run < 128) run /= 2;
+            if (run < 8192) run = 8192;
+        }
+        int lchunk = (int)(run / dm.N);
         if (lchunk < 1) lchunk = 1;
         if (lchunk > dm.L) lchunk = dm.L;
         const int nlc = (dm.L + lchunk - 1) / lchunk;
