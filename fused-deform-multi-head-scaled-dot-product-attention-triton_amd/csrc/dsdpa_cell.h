@@ -304,6 +304,8 @@ struct CellGrid {
 // in the order of the row's coordinates): an entry then costs a gather of that pair and the two rank-1 updates --
 // no taps in registers, no dot products, no exponential. Only with the work list (colour < 0) and with
 // records (the positions beside the ids).
+// RECORDS: the lists hold 12-byte records (sample id and position in the cell); without, ids alone, and every
+// entry's coordinate pair is read again (the deterministic backward, whose lists are sorted id arrays).
 template <typename S, int D, int DC, bool HANDED, bool RECORDS>
 __global__ __launch_bounds__(kCellWaves *kWave, HANDED ? (DC <= 4 ? 5 : (S::kBytes == 2 ? 3 : 4))
                                                        : DC <= 4 ? (S::kBytes == 2 && D >= 64 ? 5 : 4) : (S::kBytes == 2 ? 3 : 2))
